@@ -1,0 +1,138 @@
+/*
+ * mi8 - float8 linear path for gfx950 (MI355X): C ABI of libmi8.so.
+ *
+ * Every entry point is a plain C function over raw device pointers, sizes and a HIP stream handle.
+ * Unless a function says otherwise it
+ *   - returns MI8_OK (0) or a negative mi8_status; mi8_last_error() gives the text for the calling
+ *     thread's most recent failure;
+ *   - only enqueues work on `stream` (a hipStream_t passed as void*; NULL = the default stream): it never
+ *     synchronises, never allocates or frees device memory, and keeps no state between calls;
+ *   - requires every pointer to be 16-byte aligned device memory of at least the stated size.
+ * All matrices are dense row-major with the row pitch given (or implied) in elements.
+ *
+ * The arithmetic these functions implement is the dynamic-scaling float8 training path the reference
+ * reaches through torchao (reference: src/olmo_core/float8/__init__.py:133-150 converts every eligible
+ * nn.Linear; src/olmo_core/float8/ao.py:152-186 carries the options).  The per-function comments cite
+ * the reference interface each one stands in for.
+ */
+#ifndef MI8_H
+#define MI8_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define MI8_VERSION 100 /* major*10000 + minor*100 + patch */
+
+typedef enum mi8_status {
+    MI8_OK = 0,
+    MI8_ERR_ARG = -1,         /* NULL pointer, negative size, unknown enum value */
+    MI8_ERR_UNSUPPORTED = -2, /* shape or alignment outside what the kernels handle */
+    MI8_ERR_LAUNCH = -3       /* HIP reported an error at launch */
+} mi8_status;
+
+/* float8 encodings (OCP): reference dtype names src/olmo_core/config.py:373-374 */
+typedef enum mi8_fp8 { MI8_E4M3 = 0 /* float8_e4m3fn, max 448 */, MI8_E5M2 = 1 /* float8_e5m2, max 57344 */ } mi8_fp8;
+
+/* high-precision element types accepted by the casts (src/olmo_core/config.py:370-372) */
+typedef enum mi8_hp { MI8_BF16 = 0, MI8_F32 = 1 } mi8_hp;
+
+/* flags shared by the cast entry points */
+#define MI8_FLAG_POW2_SCALE 1u /* round every scale down to a power of two (ao.py:167 round_scales_to_power_of_2) */
+#define MI8_FLAG_SW_CVT 2u     /* convert with integer arithmetic instead of v_cvt_pk_{fp8,bf8}_f32 (same bytes) */
+
+/* Number of uint32 slots a tensorwise amax workspace must have. */
+#define MI8_AMAX_SLOTS 2048
+
+int mi8_version(void);
+const char* mi8_last_error(void);
+
+/* ---------------------------------------------------------------------------------------------
+ * Tensorwise dynamic cast.   Stands in for torchao tensor_to_amax / amax_to_scale /
+ * hp_tensor_and_scale_to_float8 as invoked by Float8Linear for TENSORWISE cast configs
+ * (reference: the default AOCastConfig, src/olmo_core/float8/ao.py:76-86).
+ * ------------------------------------------------------------------------------------------- */
+
+/* Partial maxima of |x| over n contiguous elements.  Writes *n_slots_used (host int, may be NULL) and
+ * fills slots[0 .. used) with the bit patterns of per-workgroup maxima (float32 bit pattern of |x|; a NaN
+ * input yields a NaN pattern, which compares greatest).  slots must hold MI8_AMAX_SLOTS uint32.
+ * The number of slots used depends only on n. */
+int mi8_amax_partials(const void* x, int hp_dtype, int64_t n, uint32_t* slots, int32_t* n_slots_used, void* stream);
+
+/* Number of slots mi8_amax_partials uses for n elements (host-side, no GPU work). */
+int32_t mi8_amax_slots_for(int64_t n);
+
+/* amax = max(slots[0..n_slots)), scale = float32(FP8_MAX * (1 / max(float64(amax), 1e-12))), optionally rounded
+ * down to a power of two.  out[0] = scale, out[1] = amax (both float32, device). */
+int mi8_scale_from_partials(const uint32_t* slots, int32_t n_slots, int fp8_dtype, uint32_t flags, float* out,
+                            void* stream);
+
+/* Saturating cast of x[rows, cols] with one scale for the whole tensor.
+ *   scale source: if slots != NULL the scale is reduced from slots[0..n_slots) exactly as
+ *   mi8_scale_from_partials does (and written to scale_out[0] if scale_out != NULL);
+ *   otherwise it is read from scale_in[0] (device float32).
+ *   out   (may be NULL): fp8 [rows, cols], row-major.
+ *   out_t (may be NULL): fp8 [cols, ld_t], the transposed copy; ld_t >= rows, ld_t % 16 == 0; columns
+ *                        rows..ld_t-1 of out_t are written as zero.
+ * cols % 16 == 0 is required. */
+int mi8_cast_tensorwise(const void* x, int hp_dtype, int64_t rows, int64_t cols, const uint32_t* slots,
+                        int32_t n_slots, const float* scale_in, int fp8_dtype, uint32_t flags, void* out,
+                        void* out_t, int64_t ld_t, float* scale_out, void* stream);
+
+/* ---------------------------------------------------------------------------------------------
+ * Axiswise ("rowwise" recipe) dynamic casts: AXISWISE cast configs of the rowwise recipes
+ * (reference: AOFloat8LinearRecipe.rowwise / rowwise_with_gw_hp, src/olmo_core/float8/ao.py:100-109).
+ * ------------------------------------------------------------------------------------------- */
+
+/* One scale per row (amax over the last axis): out fp8 [rows, cols], scale_out float32 [rows].
+ * cols % 16 == 0, cols <= 65536. Single pass over x. */
+int mi8_cast_rowwise(const void* x, int hp_dtype, int64_t rows, int64_t cols, int fp8_dtype, uint32_t flags,
+                     void* out, float* scale_out, void* stream);
+
+/* Number of uint32 a column-amax workspace needs for a [rows, cols] input. */
+int64_t mi8_colamax_workspace_slots(int64_t rows, int64_t cols);
+
+/* One scale per column (amax over axis 0), output written TRANSPOSED: out_t fp8 [cols, ld_t] (pad columns
+ * rows..ld_t-1 zero), scale_out float32 [cols].  This is the operand layout the grad_weight GEMM and the
+ * axiswise grad_input GEMM consume.  workspace: mi8_colamax_workspace_slots(rows, cols) uint32.
+ * Two kernels: column amax, then cast + transpose. */
+int mi8_cast_colwise_t(const void* x, int hp_dtype, int64_t rows, int64_t cols, int fp8_dtype, uint32_t flags,
+                       uint32_t* workspace, void* out_t, int64_t ld_t, float* scale_out, void* stream);
+
+/* ---------------------------------------------------------------------------------------------
+ * Scaled float8 GEMM.  Stands in for torch._scaled_mm as driven by torchao's float8 mm dispatch
+ * (the three GEMMs of one linear: output, grad_input, grad_weight).
+ *   out[M, N] = bf16( (sum_k A[m,k] * B[n,k]) * (1/sa) * (1/sb) ), fp32 accumulation on fp8 MFMA.
+ *   A: fp8 [M, lda] row-major, B: fp8 [N, ldb] row-major - both operands K-contiguous; K % 16 == 0,
+ *   lda, ldb % 16 == 0.  a_dtype / b_dtype may differ (e5m2 x e4m3 for the gradient GEMMs).
+ *   sa: quantisation scale(s) of A - one float32 if sa_rows == 0, else float32 [M]; sb likewise ([N]).
+ *   out: [M, ldc] of out_dtype (MI8_BF16 or MI8_F32), ldc >= N.
+ *   variant: -1 picks a tile configuration from the shape; 0..mi8_gemm_num_variants()-1 forces one.
+ * ------------------------------------------------------------------------------------------- */
+int mi8_gemm_fp8(const void* a, int a_dtype, int64_t lda, const void* b, int b_dtype, int64_t ldb, int64_t M,
+                 int64_t N, int64_t K, const float* sa, int sa_is_vector, const float* sb, int sb_is_vector,
+                 void* out, int out_dtype, int64_t ldc, int variant, void* stream);
+
+/* Number of GEMM kernel variants compiled in (variant ids 0..n-1; 0 is the default). */
+int mi8_gemm_num_variants(void);
+const char* mi8_gemm_variant_name(int variant);
+
+/* ---------------------------------------------------------------------------------------------
+ * SwiGLU pointwise kernels between the projections of the feed-forward block
+ * (reference: src/olmo_core/nn/feed_forward.py:171  w2(silu(w1 x) * w3 x)).
+ *   forward : h = bf16(bf16(silu(x1)) * x3), optionally also the amax partials of h.
+ *   backward: given gh, g1 = gh * x3 * silu'(x1), g3 = gh * silu(x1), evaluated with bf16 roundings of
+ *             torch's elementwise autograd formulas; optionally amax partials of g1 and g3.
+ * All tensors bf16, n elements, n % 8 == 0.
+ * ------------------------------------------------------------------------------------------- */
+int mi8_swiglu_fwd(const void* x1, const void* x3, void* h, int64_t n, uint32_t* slots_h, void* stream);
+int mi8_swiglu_bwd(const void* x1, const void* x3, const void* gh, void* g1, void* g3, int64_t n,
+                   uint32_t* slots_g1, uint32_t* slots_g3, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MI8_H */

@@ -1,0 +1,95 @@
+"""
+Build recipe for libmi8.so: plain ``hipcc`` for gfx950, no torch headers (the library has a C ABI).
+
+    python -m olmo_core_amd.build            # compile if sources are newer than the library
+    python -m olmo_core_amd.build --force    # always compile
+"""
+
+from __future__ import annotations
+
+import argparse
+import os
+import shutil
+import subprocess
+import sys
+from concurrent.futures import ThreadPoolExecutor
+from pathlib import Path
+
+PKG_DIR = Path(__file__).resolve().parent
+CSRC = PKG_DIR / "csrc"
+LIB_PATH = PKG_DIR / "lib" / "libmi8.so"
+OBJ_DIR = PKG_DIR / "lib" / "obj"
+
+SOURCES = ["mi8_api.hip", "mi8_cast.hip", "mi8_gemm.hip", "mi8_pointwise.hip", "mi8_grouped.hip"]
+
+HIPCC_FLAGS = [
+    "--offload-arch=gfx950",
+    "-O3",
+    "-std=c++17",
+    "-fPIC",
+    "-ffp-contract=off",
+    "-fno-fast-math",
+    # hipcc must not form packed-fp32 instructions on its own
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-Wall",
+    "-Wno-unused-function",
+]
+
+
+def hipcc() -> str:
+    exe = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
+    if not Path(exe).exists():
+        raise RuntimeError("hipcc not found; libmi8.so cannot be built on this machine")
+    return exe
+
+
+def sources() -> list[Path]:
+    return [CSRC / s for s in SOURCES if (CSRC / s).exists()]
+
+
+def is_stale() -> bool:
+    if not LIB_PATH.exists():
+        return True
+    built = LIB_PATH.stat().st_mtime
+    deps = list(CSRC.glob("*.hip")) + list(CSRC.glob("*.h")) + [PKG_DIR.parent / "include" / "mi8.h"]
+    return any(d.stat().st_mtime > built for d in deps)
+
+
+def build(force: bool = True, verbose: bool = False) -> Path:
+    if not force and not is_stale():
+        return LIB_PATH
+    OBJ_DIR.mkdir(parents=True, exist_ok=True)
+    cc = hipcc()
+
+    def compile_one(src: Path) -> Path:
+        obj = OBJ_DIR / (src.stem + ".o")
+        cmd = [cc, *HIPCC_FLAGS, "-c", str(src), "-o", str(obj)]
+        if verbose:
+            print(" ".join(cmd), flush=True)
+        res = subprocess.run(cmd, capture_output=True, text=True)
+        if res.returncode != 0:
+            raise RuntimeError(f"hipcc failed on {src.name}:\n{res.stdout}\n{res.stderr}")
+        noise = "unknown target feature"  # host pass does not know the device-only feature flag
+        warn = "\n".join(line for line in res.stderr.splitlines() if line.strip() and noise not in line and "-packed-fp32-ops" not in line)
+        if warn and verbose:
+            print(warn, file=sys.stderr)
+        return obj
+
+    jobs = min(len(sources()), int(os.environ.get("MAX_JOBS", "8")))
+    with ThreadPoolExecutor(max_workers=max(jobs, 1)) as pool:
+        objs = list(pool.map(compile_one, sources()))
+    tmp = LIB_PATH.with_suffix(".so.tmp")
+    cmd = [cc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", str(tmp), *map(str, objs)]
+    res = subprocess.run(cmd, capture_output=True, text=True)
+    if res.returncode != 0:
+        raise RuntimeError(f"link failed:\n{res.stdout}\n{res.stderr}")
+    os.replace(tmp, LIB_PATH)
+    return LIB_PATH
+
+
+if __name__ == "__main__":
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--force", action="store_true")
+    ap.add_argument("-v", "--verbose", action="store_true")
+    ns = ap.parse_args()
+    print(build(force=ns.force or is_stale(), verbose=ns.verbose))

@@ -1,0 +1,565 @@
+// amax reductions and saturating float8 casts (tensorwise, per-row, per-column with transposed output).
+// All kernels are HBM-bound streaming kernels: 16-byte loads per lane, wave-shuffle reductions, an
+// LDS-staged byte transpose for the transposed copy.
+#include "mi8_common.h"
+
+namespace mi8 {
+namespace {
+
+constexpr int kThreads = 256;
+
+// ------------------------------------------------------------------------------------------------
+// tensorwise amax -> per-workgroup partial maxima
+// ------------------------------------------------------------------------------------------------
+
+typedef unsigned short us2 __attribute__((ext_vector_type(2)));
+
+__device__ __forceinline__ uint32_t pk_absmax_u16(uint32_t acc, uint32_t v)
+{
+    // two bf16 per dword: clear both sign bits, packed unsigned 16-bit max (v_pk_max_u16)
+    us2 a = __builtin_bit_cast(us2, acc);
+    us2 b = __builtin_bit_cast(us2, v & 0x7FFF7FFFu);
+    return __builtin_bit_cast(uint32_t, __builtin_elementwise_max(a, b));
+}
+
+template <int HP>
+__device__ __forceinline__ void absmax_accumulate(uint4 v, uint32_t (&acc)[4])
+{
+    if constexpr (HP == MI8_BF16) {
+        acc[0] = pk_absmax_u16(acc[0], v.x);
+        acc[1] = pk_absmax_u16(acc[1], v.y);
+        acc[2] = pk_absmax_u16(acc[2], v.z);
+        acc[3] = pk_absmax_u16(acc[3], v.w);
+    } else {
+        acc[0] = umax32(acc[0], v.x & 0x7FFFFFFFu);
+        acc[1] = umax32(acc[1], v.y & 0x7FFFFFFFu);
+        acc[2] = umax32(acc[2], v.z & 0x7FFFFFFFu);
+        acc[3] = umax32(acc[3], v.w & 0x7FFFFFFFu);
+    }
+}
+
+// fold the four accumulators into one float32 |x| bit pattern
+template <int HP>
+__device__ __forceinline__ uint32_t absmax_fold(const uint32_t (&acc)[4])
+{
+    if constexpr (HP == MI8_BF16) {
+        uint32_t m = pk_absmax_u16(pk_absmax_u16(acc[0], acc[1]), pk_absmax_u16(acc[2], acc[3]));
+        uint32_t hi = m >> 16, lo = m & 0xFFFFu;
+        return umax32(hi, lo) << 16;
+    } else {
+        return umax32(umax32(acc[0], acc[1]), umax32(acc[2], acc[3]));
+    }
+}
+
+__device__ __forceinline__ uint32_t block_umax(uint32_t v, uint32_t* smem /* >= 4 words */)
+{
+    v = wave_umax(v);
+    const int wave = threadIdx.x >> 6;
+    if ((threadIdx.x & 63) == 0) smem[wave] = v;
+    __syncthreads();
+    v = umax32(umax32(smem[0], smem[1]), umax32(smem[2], smem[3]));
+    __syncthreads();
+    return v;
+}
+
+template <int HP>
+__global__ __launch_bounds__(kThreads) void amax_partials_kernel(const uint4* __restrict__ x, int64_t nvec,
+                                                                 const void* __restrict__ tail, int ntail,
+                                                                 uint32_t* __restrict__ slots)
+{
+    __shared__ uint32_t smem[4];
+    uint32_t acc[4] = {0, 0, 0, 0};
+    const int64_t stride = (int64_t)gridDim.x * kThreads;
+    int64_t i = (int64_t)blockIdx.x * kThreads + threadIdx.x;
+    // four independent 16-byte loads in flight per lane
+    for (; i + 3 * stride < nvec; i += 4 * stride) {
+        uint4 v0 = x[i], v1 = x[i + stride], v2 = x[i + 2 * stride], v3 = x[i + 3 * stride];
+        absmax_accumulate<HP>(v0, acc);
+        absmax_accumulate<HP>(v1, acc);
+        absmax_accumulate<HP>(v2, acc);
+        absmax_accumulate<HP>(v3, acc);
+    }
+    for (; i < nvec; i += stride) absmax_accumulate<HP>(x[i], acc);
+    uint32_t m = absmax_fold<HP>(acc);
+    if (blockIdx.x == 0 && (int)threadIdx.x < ntail) {
+        if constexpr (HP == MI8_BF16)
+            m = umax32(m, ((uint32_t) reinterpret_cast<const uint16_t*>(tail)[threadIdx.x] & 0x7FFFu) << 16);
+        else
+            m = umax32(m, reinterpret_cast<const uint32_t*>(tail)[threadIdx.x] & 0x7FFFFFFFu);
+    }
+    m = block_umax(m, smem);
+    if (threadIdx.x == 0) slots[blockIdx.x] = m;
+}
+
+template <int FP8>
+__global__ __launch_bounds__(kThreads) void scale_from_partials_kernel(const uint32_t* __restrict__ slots,
+                                                                       int n_slots, bool pow2,
+                                                                       float* __restrict__ out)
+{
+    __shared__ uint32_t smem[4];
+    uint32_t m = 0;
+    for (int i = threadIdx.x; i < n_slots; i += kThreads) m = umax32(m, slots[i]);
+    m = block_umax(m, smem);
+    if (threadIdx.x == 0) {
+        out[0] = scale_from_amax_bits<FP8>(m, pow2);
+        out[1] = bits_to_f32(m);
+    }
+}
+
+// ------------------------------------------------------------------------------------------------
+// tile cast: 128 x 128 elements per workgroup, optional row-major output, optional transposed output
+// ------------------------------------------------------------------------------------------------
+
+constexpr int kTile = 128;
+
+enum ScaleMode { kScalarFromSlots = 0, kScalarFromPtr = 1, kPerColumnFromWorkspace = 2 };
+
+struct TileCastArgs {
+    const void* x;
+    int64_t rows, cols;
+    const uint32_t* slots;  // kScalarFromSlots: partial maxima; kPerColumnFromWorkspace: [n_slots][cols]
+    int n_slots;
+    const float* scale_in;
+    bool pow2;
+    uint8_t* out;    // [rows, cols] or null
+    uint8_t* out_t;  // [cols, ld_t] or null
+    int64_t ld_t;
+    float* scale_out;  // scalar modes: [1]; per-column mode: [cols]; may be null
+};
+
+// LDS holds the transposed tile as 128 columns x 128 row-bytes.  Two columns share a 256-byte line; the
+// 16-byte chunk index inside the line is XORed with a function of the column's group of eight so that
+// both the dword writes (lanes spread over 16 column groups x 4 row groups) and the 16-byte reads
+// (lanes spread over 8 columns x 8 chunks) touch every bank once.
+__device__ __forceinline__ int tile_lds_chunk(int col, int part /* 0..7: which 16 row-bytes */)
+{
+    const int grp = col >> 3;
+    const int key = (((grp >> 3) & 1) << 3) | (grp & 7);
+    return (col >> 1) * 16 + ((((col & 1) << 3) | part) ^ key);
+}
+
+template <int HP, int FP8, bool SW, int MODE>
+__global__ __launch_bounds__(kThreads) void tile_cast_kernel(TileCastArgs a)
+{
+    __shared__ __attribute__((aligned(16))) uint32_t lds_t[kTile * kTile / 4];
+    __shared__ float s_scale[kTile];
+    __shared__ uint32_t smem[4];
+
+    const int tid = threadIdx.x;
+    const int wave = tid >> 6, lane = tid & 63;
+    const int cl = lane & 15, g = lane >> 4;
+    const int64_t row0 = (int64_t)blockIdx.y * kTile;
+    const int64_t col0 = (int64_t)blockIdx.x * kTile;
+
+    // ---- scale(s) -------------------------------------------------------------------------
+    float sc[8];
+    if constexpr (MODE == kPerColumnFromWorkspace) {
+        if (tid < kTile) {
+            const int64_t c = col0 + tid;
+            float s = 0.0f;
+            if (c < a.cols) {
+                uint32_t m = 0;
+                for (int k = 0; k < a.n_slots; ++k) m = umax32(m, a.slots[(int64_t)k * a.cols + c]);
+                s = scale_from_amax_bits<FP8>(m, a.pow2);
+                if (blockIdx.y == 0 && a.scale_out) a.scale_out[c] = s;
+            }
+            s_scale[tid] = s;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int i = 0; i < 8; ++i) sc[i] = s_scale[8 * cl + i];
+    } else {
+        float s;
+        if constexpr (MODE == kScalarFromSlots) {
+            uint32_t m = 0;
+            for (int i = tid; i < a.n_slots; i += kThreads) m = umax32(m, a.slots[i]);
+            m = block_umax(m, smem);
+            s = scale_from_amax_bits<FP8>(m, a.pow2);  // every lane: same bits in, same bits out
+            if (a.scale_out && tid == 0 && blockIdx.x == 0 && blockIdx.y == 0) a.scale_out[0] = s;
+        } else {
+            s = a.scale_in[0];
+            if (a.scale_out && tid == 0 && blockIdx.x == 0 && blockIdx.y == 0) a.scale_out[0] = s;
+        }
+#pragma unroll
+        for (int i = 0; i < 8; ++i) sc[i] = s;
+    }
+
+    // ---- load, quantise, write row-major, stage transposed ----------------------------------
+    const int64_t c8 = col0 + 8 * cl;
+    const bool col_ok = c8 < a.cols;
+    const char* xb = reinterpret_cast<const char*>(a.x);
+
+    float f[2][4][8];
+#pragma unroll
+    for (int it = 0; it < 2; ++it)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int64_t r = row0 + 32 * wave + 16 * it + 4 * g + j;
+            const bool ok = col_ok && r < a.rows;
+            HpVec<HP>::load8(xb + (r * a.cols + c8) * HpVec<HP>::kBytes, ok, f[it][j]);
+        }
+
+#pragma unroll
+    for (int it = 0; it < 2; ++it) {
+        uint32_t lo[4], hi[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int64_t r = row0 + 32 * wave + 16 * it + 4 * g + j;
+            const bool ok = col_ok && r < a.rows;
+            const float* v = f[it][j];
+            lo[j] = quant4<FP8, SW>(v[0], v[1], v[2], v[3], sc[0], sc[1], sc[2], sc[3]);
+            hi[j] = quant4<FP8, SW>(v[4], v[5], v[6], v[7], sc[4], sc[5], sc[6], sc[7]);
+            if (!ok) lo[j] = hi[j] = 0;  // padding is zero bytes whatever the scale is (0 * NaN is NaN)
+            if (a.out && ok) *reinterpret_cast<uint2*>(a.out + r * a.cols + c8) = make_uint2(lo[j], hi[j]);
+        }
+        if (a.out_t) {
+            uint32_t t[8];
+            transpose4x4_bytes(lo[0], lo[1], lo[2], lo[3], t[0], t[1], t[2], t[3]);
+            transpose4x4_bytes(hi[0], hi[1], hi[2], hi[3], t[4], t[5], t[6], t[7]);
+            const int rd = 8 * wave + 4 * it + g;  // which dword of the column's 32 row-dwords
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const int col = 8 * cl + i;
+                lds_t[tile_lds_chunk(col, rd >> 2) * 4 + (rd & 3)] = t[i];
+            }
+        }
+    }
+
+    if (a.out_t) {
+        __syncthreads();
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int q = tid + kThreads * i;
+            const int col = q >> 3, part = q & 7;
+            const uint4 v = reinterpret_cast<const uint4*>(lds_t)[tile_lds_chunk(col, part)];
+            const int64_t c = col0 + col;
+            const int64_t r = row0 + 16 * part;
+            if (c < a.cols && r < a.ld_t) *reinterpret_cast<uint4*>(a.out_t + c * a.ld_t + r) = v;
+        }
+    }
+}
+
+// ------------------------------------------------------------------------------------------------
+// per-column amax partials: workspace[chunk][col] = max |x[r, col]| over the chunk's rows
+// ------------------------------------------------------------------------------------------------
+
+template <int HP>
+__global__ __launch_bounds__(kThreads) void colamax_kernel(const void* __restrict__ x, int64_t rows,
+                                                           int64_t cols, int64_t rows_per_chunk,
+                                                           uint32_t* __restrict__ ws)
+{
+    __shared__ uint32_t red[16][kTile + 1];
+    const int tid = threadIdx.x;
+    const int cl = tid & 15, rg = tid >> 4;
+    const int64_t col0 = (int64_t)blockIdx.x * kTile;
+    const int64_t c8 = col0 + 8 * cl;
+    const bool col_ok = c8 < cols;
+    const int64_t r_begin = (int64_t)blockIdx.y * rows_per_chunk;
+    const int64_t r_end = (r_begin + rows_per_chunk < rows) ? r_begin + rows_per_chunk : rows;
+    const char* xb = reinterpret_cast<const char*>(x);
+    constexpr int NV = HpVec<HP>::kBytes == 2 ? 1 : 2;  // 16-byte vectors per 8 elements
+
+    uint32_t acc[NV][4];
+#pragma unroll
+    for (int v = 0; v < NV; ++v)
+#pragma unroll
+        for (int k = 0; k < 4; ++k) acc[v][k] = 0;
+
+    if (col_ok) {
+        int64_t r = r_begin + rg;
+        for (; r + 48 < r_end; r += 64) {
+            uint4 v[4][NV];
+#pragma unroll
+            for (int u = 0; u < 4; ++u)
+#pragma unroll
+                for (int k = 0; k < NV; ++k)
+                    v[u][k] = reinterpret_cast<const uint4*>(xb + ((r + 16 * u) * cols + c8) * HpVec<HP>::kBytes)[k];
+#pragma unroll
+            for (int u = 0; u < 4; ++u)
+#pragma unroll
+                for (int k = 0; k < NV; ++k) absmax_accumulate<HP>(v[u][k], acc[k]);
+        }
+        for (; r < r_end; r += 16) {
+#pragma unroll
+            for (int k = 0; k < NV; ++k)
+                absmax_accumulate<HP>(reinterpret_cast<const uint4*>(xb + (r * cols + c8) * HpVec<HP>::kBytes)[k],
+                                      acc[k]);
+        }
+    }
+    // spread this lane's 8 columns into the reduction buffer as float32 |x| bit patterns
+    if constexpr (HP == MI8_BF16) {
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            red[rg][8 * cl + 2 * k] = (acc[0][k] & 0xFFFFu) << 16;
+            red[rg][8 * cl + 2 * k + 1] = acc[0][k] & 0xFFFF0000u;
+        }
+    } else {
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            red[rg][8 * cl + k] = acc[0][k];
+            red[rg][8 * cl + 4 + k] = acc[NV - 1][k];
+        }
+    }
+    __syncthreads();
+    if (tid < kTile && col0 + tid < cols) {
+        uint32_t m = 0;
+#pragma unroll
+        for (int k = 0; k < 16; ++k) m = umax32(m, red[k][tid]);
+        ws[(int64_t)blockIdx.y * cols + col0 + tid] = m;
+    }
+}
+
+// ------------------------------------------------------------------------------------------------
+// per-row cast: TPR lanes cooperate on one row, the whole row stays in registers between the amax and
+// the conversion (single pass over HBM)
+// ------------------------------------------------------------------------------------------------
+
+template <int HP, int FP8, bool SW, int TPR /* 64 or 256 */, int NV /* 8-element vectors per lane */>
+__global__ __launch_bounds__(kThreads) void rowwise_cast_kernel(const void* __restrict__ x, int64_t rows,
+                                                                int64_t cols, bool pow2,
+                                                                uint8_t* __restrict__ out,
+                                                                float* __restrict__ scale_out)
+{
+    __shared__ uint32_t smem[4];
+    constexpr int ROWS_PER_BLOCK = kThreads / TPR;
+    const int tid = threadIdx.x;
+    const int sub = tid / TPR, lane = tid % TPR;
+    const int64_t row = (int64_t)blockIdx.x * ROWS_PER_BLOCK + sub;
+    const bool row_ok = row < rows;
+    const int nvec = (int)(cols >> 3);
+    const char* xr = reinterpret_cast<const char*>(x) + row * cols * HpVec<HP>::kBytes;
+
+    float f[NV][8];
+    uint32_t m = 0;
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+        const int v = lane + TPR * i;
+        HpVec<HP>::load8(xr + (int64_t)v * 8 * HpVec<HP>::kBytes, row_ok && v < nvec, f[i]);
+        m = umax32(m, absmax8_bits(f[i]));
+    }
+    if constexpr (TPR == 64)
+        m = wave_umax(m);
+    else
+        m = block_umax(m, smem);
+    const float s = scale_from_amax_bits<FP8>(m, pow2);
+    if (row_ok && lane == 0) scale_out[row] = s;
+    uint8_t* orow = out + row * cols;
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+        const int v = lane + TPR * i;
+        if (row_ok && v < nvec) {
+            const uint32_t lo = quant4<FP8, SW>(f[i][0], f[i][1], f[i][2], f[i][3], s, s, s, s);
+            const uint32_t hi = quant4<FP8, SW>(f[i][4], f[i][5], f[i][6], f[i][7], s, s, s, s);
+            *reinterpret_cast<uint2*>(orow + (int64_t)v * 8) = make_uint2(lo, hi);
+        }
+    }
+}
+
+// ---- dispatch helpers ------------------------------------------------------------------------------
+
+template <int HP, int FP8, bool SW>
+void launch_tile_cast(int mode, const TileCastArgs& a, dim3 grid, hipStream_t st)
+{
+    switch (mode) {
+        case kScalarFromSlots:
+            hipLaunchKernelGGL((tile_cast_kernel<HP, FP8, SW, kScalarFromSlots>), grid, dim3(kThreads), 0, st, a);
+            break;
+        case kScalarFromPtr:
+            hipLaunchKernelGGL((tile_cast_kernel<HP, FP8, SW, kScalarFromPtr>), grid, dim3(kThreads), 0, st, a);
+            break;
+        default:
+            hipLaunchKernelGGL((tile_cast_kernel<HP, FP8, SW, kPerColumnFromWorkspace>), grid, dim3(kThreads), 0,
+                               st, a);
+            break;
+    }
+}
+
+void dispatch_tile_cast(int hp, int fp8, bool sw, int mode, const TileCastArgs& a, hipStream_t st)
+{
+    dim3 grid((unsigned)ceil_div(a.cols, kTile), (unsigned)ceil_div(a.rows, kTile));
+#define MI8_TC(HP_, FP8_)                                       \
+    if (sw)                                                     \
+        launch_tile_cast<HP_, FP8_, true>(mode, a, grid, st);   \
+    else                                                        \
+        launch_tile_cast<HP_, FP8_, false>(mode, a, grid, st)
+    if (hp == MI8_BF16) {
+        if (fp8 == MI8_E4M3) { MI8_TC(MI8_BF16, MI8_E4M3); } else { MI8_TC(MI8_BF16, MI8_E5M2); }
+    } else {
+        if (fp8 == MI8_E4M3) { MI8_TC(MI8_F32, MI8_E4M3); } else { MI8_TC(MI8_F32, MI8_E5M2); }
+    }
+#undef MI8_TC
+}
+
+template <int HP, int FP8, bool SW>
+int launch_rowwise(const void* x, int64_t rows, int64_t cols, bool pow2, uint8_t* out, float* scale_out,
+                   hipStream_t st)
+{
+    const int64_t nvec = cols / 8;
+#define MI8_RW(TPR_, NV_)                                                                                    \
+    hipLaunchKernelGGL((rowwise_cast_kernel<HP, FP8, SW, TPR_, NV_>), dim3((unsigned)ceil_div(rows, kThreads / TPR_)), \
+                       dim3(kThreads), 0, st, x, rows, cols, pow2, out, scale_out)
+    if (nvec <= 64 * 2) { MI8_RW(64, 2); }
+    else if (nvec <= 64 * 4) { MI8_RW(64, 4); }
+    else if (nvec <= 64 * 8) { MI8_RW(64, 8); }
+    else if (nvec <= 256 * 4) { MI8_RW(256, 4); }
+    else if (nvec <= 256 * 8) { MI8_RW(256, 8); }
+    else if (nvec <= 256 * 16) { MI8_RW(256, 16); }
+    else if (nvec <= 256 * 32) { MI8_RW(256, 32); }
+    else return MI8_ERR_UNSUPPORTED;
+#undef MI8_RW
+    return MI8_OK;
+}
+
+bool valid_hp(int v) { return v == MI8_BF16 || v == MI8_F32; }
+bool valid_fp8(int v) { return v == MI8_E4M3 || v == MI8_E5M2; }
+
+int64_t colamax_rows_per_chunk(int64_t rows)
+{
+    int64_t rpc = round_up(ceil_div(rows, 32), 16);
+    return rpc < 256 ? 256 : rpc;
+}
+
+}  // namespace
+}  // namespace mi8
+
+using namespace mi8;
+
+extern "C" int32_t mi8_amax_slots_for(int64_t n)
+{
+    if (n <= 0) return 1;
+    // one workgroup per 256 lanes x 4 vectors x 8 (bf16) elements at least, capped by the workspace size
+    int64_t blocks = ceil_div(n, (int64_t)kThreads * 4 * 8);
+    if (blocks < 1) blocks = 1;
+    if (blocks > MI8_AMAX_SLOTS) blocks = MI8_AMAX_SLOTS;
+    return (int32_t)blocks;
+}
+
+extern "C" int mi8_amax_partials(const void* x, int hp_dtype, int64_t n, uint32_t* slots, int32_t* n_slots_used,
+                                 void* stream)
+{
+    MI8_REQUIRE(x && slots, MI8_ERR_ARG, "mi8_amax_partials: null pointer");
+    MI8_REQUIRE(valid_hp(hp_dtype), MI8_ERR_ARG, "mi8_amax_partials: unknown hp dtype %d", hp_dtype);
+    MI8_REQUIRE(n > 0, MI8_ERR_ARG, "mi8_amax_partials: n must be positive (got %lld)", (long long)n);
+    MI8_REQUIRE(aligned16(x), MI8_ERR_UNSUPPORTED, "mi8_amax_partials: x must be 16-byte aligned");
+    const int per_vec = hp_dtype == MI8_BF16 ? 8 : 4;
+    const int64_t nvec = n / per_vec;
+    const int ntail = (int)(n % per_vec);
+    const int esz = hp_dtype == MI8_BF16 ? 2 : 4;
+    const void* tail = reinterpret_cast<const char*>(x) + nvec * per_vec * esz;
+    const int32_t blocks = mi8_amax_slots_for(n);
+    if (n_slots_used) *n_slots_used = blocks;
+    hipStream_t st = (hipStream_t)stream;
+    if (hp_dtype == MI8_BF16)
+        hipLaunchKernelGGL((amax_partials_kernel<MI8_BF16>), dim3(blocks), dim3(kThreads), 0, st,
+                           (const uint4*)x, nvec, tail, ntail, slots);
+    else
+        hipLaunchKernelGGL((amax_partials_kernel<MI8_F32>), dim3(blocks), dim3(kThreads), 0, st, (const uint4*)x,
+                           nvec, tail, ntail, slots);
+    return launch_status("mi8_amax_partials");
+}
+
+extern "C" int mi8_scale_from_partials(const uint32_t* slots, int32_t n_slots, int fp8_dtype, uint32_t flags,
+                                       float* out, void* stream)
+{
+    MI8_REQUIRE(slots && out, MI8_ERR_ARG, "mi8_scale_from_partials: null pointer");
+    MI8_REQUIRE(valid_fp8(fp8_dtype), MI8_ERR_ARG, "mi8_scale_from_partials: unknown fp8 dtype %d", fp8_dtype);
+    MI8_REQUIRE(n_slots > 0 && n_slots <= MI8_AMAX_SLOTS, MI8_ERR_ARG, "mi8_scale_from_partials: n_slots %d out of range",
+                n_slots);
+    const bool pow2 = flags & MI8_FLAG_POW2_SCALE;
+    hipStream_t st = (hipStream_t)stream;
+    if (fp8_dtype == MI8_E4M3)
+        hipLaunchKernelGGL((scale_from_partials_kernel<MI8_E4M3>), dim3(1), dim3(kThreads), 0, st, slots, n_slots,
+                           pow2, out);
+    else
+        hipLaunchKernelGGL((scale_from_partials_kernel<MI8_E5M2>), dim3(1), dim3(kThreads), 0, st, slots, n_slots,
+                           pow2, out);
+    return launch_status("mi8_scale_from_partials");
+}
+
+extern "C" int mi8_cast_tensorwise(const void* x, int hp_dtype, int64_t rows, int64_t cols, const uint32_t* slots,
+                                   int32_t n_slots, const float* scale_in, int fp8_dtype, uint32_t flags, void* out,
+                                   void* out_t, int64_t ld_t, float* scale_out, void* stream)
+{
+    MI8_REQUIRE(x, MI8_ERR_ARG, "mi8_cast_tensorwise: x is null");
+    MI8_REQUIRE(out || out_t, MI8_ERR_ARG, "mi8_cast_tensorwise: no output requested");
+    MI8_REQUIRE(valid_hp(hp_dtype) && valid_fp8(fp8_dtype), MI8_ERR_ARG, "mi8_cast_tensorwise: unknown dtype");
+    MI8_REQUIRE(rows > 0 && cols > 0, MI8_ERR_ARG, "mi8_cast_tensorwise: empty input (%lld x %lld)", (long long)rows,
+                (long long)cols);
+    MI8_REQUIRE((slots != nullptr) != (scale_in != nullptr), MI8_ERR_ARG,
+                "mi8_cast_tensorwise: give exactly one of slots / scale_in");
+    MI8_REQUIRE(!slots || (n_slots > 0 && n_slots <= MI8_AMAX_SLOTS), MI8_ERR_ARG,
+                "mi8_cast_tensorwise: n_slots %d out of range", n_slots);
+    MI8_REQUIRE(cols % 16 == 0, MI8_ERR_UNSUPPORTED, "mi8_cast_tensorwise: cols (%lld) must be a multiple of 16",
+                (long long)cols);
+    MI8_REQUIRE(aligned16(x) && aligned16(out) && aligned16(out_t), MI8_ERR_UNSUPPORTED,
+                "mi8_cast_tensorwise: pointers must be 16-byte aligned");
+    if (out_t)
+        MI8_REQUIRE(ld_t >= rows && ld_t % 16 == 0 && ld_t <= round_up(rows, kTile), MI8_ERR_UNSUPPORTED,
+                    "mi8_cast_tensorwise: ld_t (%lld) must be a multiple of 16 in [rows, round_up(rows,128)]",
+                    (long long)ld_t);
+    TileCastArgs a{x, rows, cols, slots, n_slots, scale_in, (flags & MI8_FLAG_POW2_SCALE) != 0,
+                   (uint8_t*)out, (uint8_t*)out_t, ld_t, scale_out};
+    dispatch_tile_cast(hp_dtype, fp8_dtype, (flags & MI8_FLAG_SW_CVT) != 0, slots ? kScalarFromSlots : kScalarFromPtr,
+                       a, (hipStream_t)stream);
+    return launch_status("mi8_cast_tensorwise");
+}
+
+extern "C" int mi8_cast_rowwise(const void* x, int hp_dtype, int64_t rows, int64_t cols, int fp8_dtype,
+                                uint32_t flags, void* out, float* scale_out, void* stream)
+{
+    MI8_REQUIRE(x && out && scale_out, MI8_ERR_ARG, "mi8_cast_rowwise: null pointer");
+    MI8_REQUIRE(valid_hp(hp_dtype) && valid_fp8(fp8_dtype), MI8_ERR_ARG, "mi8_cast_rowwise: unknown dtype");
+    MI8_REQUIRE(rows > 0 && cols > 0, MI8_ERR_ARG, "mi8_cast_rowwise: empty input");
+    MI8_REQUIRE(cols % 16 == 0 && cols <= 65536, MI8_ERR_UNSUPPORTED,
+                "mi8_cast_rowwise: cols (%lld) must be a multiple of 16 and at most 65536", (long long)cols);
+    MI8_REQUIRE(aligned16(x) && aligned16(out), MI8_ERR_UNSUPPORTED, "mi8_cast_rowwise: pointers must be 16-byte aligned");
+    const bool pow2 = flags & MI8_FLAG_POW2_SCALE, sw = flags & MI8_FLAG_SW_CVT;
+    hipStream_t st = (hipStream_t)stream;
+    int rc;
+#define MI8_ROW(HP_, FP8_) \
+    rc = sw ? launch_rowwise<HP_, FP8_, true>(x, rows, cols, pow2, (uint8_t*)out, scale_out, st) \
+            : launch_rowwise<HP_, FP8_, false>(x, rows, cols, pow2, (uint8_t*)out, scale_out, st)
+    if (hp_dtype == MI8_BF16) {
+        if (fp8_dtype == MI8_E4M3) { MI8_ROW(MI8_BF16, MI8_E4M3); } else { MI8_ROW(MI8_BF16, MI8_E5M2); }
+    } else {
+        if (fp8_dtype == MI8_E4M3) { MI8_ROW(MI8_F32, MI8_E4M3); } else { MI8_ROW(MI8_F32, MI8_E5M2); }
+    }
+#undef MI8_ROW
+    MI8_REQUIRE(rc == MI8_OK, rc, "mi8_cast_rowwise: unsupported row length %lld", (long long)cols);
+    return launch_status("mi8_cast_rowwise");
+}
+
+extern "C" int64_t mi8_colamax_workspace_slots(int64_t rows, int64_t cols)
+{
+    if (rows <= 0 || cols <= 0) return 0;
+    return ceil_div(rows, colamax_rows_per_chunk(rows)) * cols;
+}
+
+extern "C" int mi8_cast_colwise_t(const void* x, int hp_dtype, int64_t rows, int64_t cols, int fp8_dtype,
+                                  uint32_t flags, uint32_t* workspace, void* out_t, int64_t ld_t, float* scale_out,
+                                  void* stream)
+{
+    MI8_REQUIRE(x && workspace && out_t && scale_out, MI8_ERR_ARG, "mi8_cast_colwise_t: null pointer");
+    MI8_REQUIRE(valid_hp(hp_dtype) && valid_fp8(fp8_dtype), MI8_ERR_ARG, "mi8_cast_colwise_t: unknown dtype");
+    MI8_REQUIRE(rows > 0 && cols > 0, MI8_ERR_ARG, "mi8_cast_colwise_t: empty input");
+    MI8_REQUIRE(cols % 16 == 0, MI8_ERR_UNSUPPORTED, "mi8_cast_colwise_t: cols (%lld) must be a multiple of 16",
+                (long long)cols);
+    MI8_REQUIRE(ld_t >= rows && ld_t % 16 == 0 && ld_t <= round_up(rows, kTile), MI8_ERR_UNSUPPORTED,
+                "mi8_cast_colwise_t: ld_t (%lld) must be a multiple of 16 in [rows, round_up(rows,128)]", (long long)ld_t);
+    MI8_REQUIRE(aligned16(x) && aligned16(out_t), MI8_ERR_UNSUPPORTED,
+                "mi8_cast_colwise_t: pointers must be 16-byte aligned");
+    hipStream_t st = (hipStream_t)stream;
+    const int64_t rpc = colamax_rows_per_chunk(rows);
+    const int n_chunks = (int)ceil_div(rows, rpc);
+    dim3 grid((unsigned)ceil_div(cols, kTile), (unsigned)n_chunks);
+    if (hp_dtype == MI8_BF16)
+        hipLaunchKernelGGL((colamax_kernel<MI8_BF16>), grid, dim3(kThreads), 0, st, x, rows, cols, rpc, workspace);
+    else
+        hipLaunchKernelGGL((colamax_kernel<MI8_F32>), grid, dim3(kThreads), 0, st, x, rows, cols, rpc, workspace);
+    int rc = launch_status("mi8_cast_colwise_t(amax)");
+    if (rc != MI8_OK) return rc;
+    TileCastArgs a{x, rows, cols, workspace, n_chunks, nullptr, (flags & MI8_FLAG_POW2_SCALE) != 0,
+                   nullptr, (uint8_t*)out_t, ld_t, scale_out};
+    dispatch_tile_cast(hp_dtype, fp8_dtype, (flags & MI8_FLAG_SW_CVT) != 0, kPerColumnFromWorkspace, a, st);
+    return launch_status("mi8_cast_colwise_t(cast)");
+}

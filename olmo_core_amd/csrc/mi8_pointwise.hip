@@ -1,0 +1,152 @@
+// SwiGLU pointwise kernels of the feed-forward block, with the amax reduction of their outputs fused in so
+// that the tensorwise cast that follows needs no separate pass over the (largest) activation tensor.
+// Rounding points follow torch's eager bf16 evaluation: every elementwise op computes in fp32 and rounds
+// its result to bf16 before the next op reads it.
+#include "mi8_common.h"
+
+namespace mi8 {
+namespace {
+
+constexpr int kThreads = 256;
+
+__device__ __forceinline__ float bf16_round(float f)
+{
+    __bf16 h = (__bf16)f;
+    return (float)h;
+}
+
+__device__ __forceinline__ uint32_t pack_bf16(float lo, float hi)
+{
+    __bf16 a = (__bf16)lo, b = (__bf16)hi;
+    return (uint32_t)__builtin_bit_cast(uint16_t, a) | ((uint32_t)__builtin_bit_cast(uint16_t, b) << 16);
+}
+
+__device__ __forceinline__ float sigmoid_f32(float x) { return 1.0f / (1.0f + expf(-x)); }
+
+__device__ __forceinline__ void unpack8(uint4 v, float (&f)[8])
+{
+    f[0] = bits_to_f32(v.x << 16);
+    f[1] = bits_to_f32(v.x & 0xFFFF0000u);
+    f[2] = bits_to_f32(v.y << 16);
+    f[3] = bits_to_f32(v.y & 0xFFFF0000u);
+    f[4] = bits_to_f32(v.z << 16);
+    f[5] = bits_to_f32(v.z & 0xFFFF0000u);
+    f[6] = bits_to_f32(v.w << 16);
+    f[7] = bits_to_f32(v.w & 0xFFFF0000u);
+}
+
+__device__ __forceinline__ uint4 pack8(const float (&f)[8])
+{
+    return make_uint4(pack_bf16(f[0], f[1]), pack_bf16(f[2], f[3]), pack_bf16(f[4], f[5]), pack_bf16(f[6], f[7]));
+}
+
+// max over |bf16| of the 8 packed values, as a float32 bit pattern
+__device__ __forceinline__ uint32_t absmax_packed(uint4 v)
+{
+    uint32_t m = 0;
+    const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        m = umax32(m, (w[i] & 0x7FFFu) << 16);
+        m = umax32(m, w[i] & 0x7FFF0000u);
+    }
+    return m;
+}
+
+__device__ __forceinline__ void publish_block_max(uint32_t m, uint32_t* slots)
+{
+    __shared__ uint32_t smem[4];
+    m = wave_umax(m);
+    if ((threadIdx.x & 63) == 0) smem[threadIdx.x >> 6] = m;
+    __syncthreads();
+    if (threadIdx.x == 0) slots[blockIdx.x] = umax32(umax32(smem[0], smem[1]), umax32(smem[2], smem[3]));
+}
+
+__global__ __launch_bounds__(kThreads) void swiglu_fwd_kernel(const uint4* __restrict__ x1,
+                                                              const uint4* __restrict__ x3, uint4* __restrict__ h,
+                                                              int64_t nvec, uint32_t* __restrict__ slots)
+{
+    uint32_t m = 0;
+    const int64_t stride = (int64_t)gridDim.x * kThreads;
+    for (int64_t i = (int64_t)blockIdx.x * kThreads + threadIdx.x; i < nvec; i += stride) {
+        float a[8], b[8], o[8];
+        unpack8(x1[i], a);
+        unpack8(x3[i], b);
+#pragma unroll
+        for (int k = 0; k < 8; ++k) {
+            const float s = bf16_round(a[k] * sigmoid_f32(a[k]));  // silu output as a bf16 tensor
+            o[k] = s * b[k];
+        }
+        const uint4 out = pack8(o);
+        h[i] = out;
+        m = umax32(m, absmax_packed(out));
+    }
+    if (slots) publish_block_max(m, slots);
+}
+
+__global__ __launch_bounds__(kThreads) void swiglu_bwd_kernel(const uint4* __restrict__ x1,
+                                                              const uint4* __restrict__ x3,
+                                                              const uint4* __restrict__ gh, uint4* __restrict__ g1,
+                                                              uint4* __restrict__ g3, int64_t nvec,
+                                                              uint32_t* __restrict__ slots1,
+                                                              uint32_t* __restrict__ slots3)
+{
+    uint32_t m1 = 0, m3 = 0;
+    const int64_t stride = (int64_t)gridDim.x * kThreads;
+    for (int64_t i = (int64_t)blockIdx.x * kThreads + threadIdx.x; i < nvec; i += stride) {
+        float a[8], b[8], g[8], o1[8], o3[8];
+        unpack8(x1[i], a);
+        unpack8(x3[i], b);
+        unpack8(gh[i], g);
+#pragma unroll
+        for (int k = 0; k < 8; ++k) {
+            const float sig = sigmoid_f32(a[k]);
+            const float s = bf16_round(a[k] * sig);   // saved silu output
+            o3[k] = g[k] * s;                         // d/dx3
+            const float gs = bf16_round(g[k] * b[k]); // gradient reaching silu's output
+            o1[k] = gs * (sig * (1.0f + a[k] * (1.0f - sig)));
+        }
+        const uint4 p1 = pack8(o1), p3 = pack8(o3);
+        g1[i] = p1;
+        g3[i] = p3;
+        m1 = umax32(m1, absmax_packed(p1));
+        m3 = umax32(m3, absmax_packed(p3));
+    }
+    if (slots1) publish_block_max(m1, slots1);
+    if (slots3) {
+        __syncthreads();
+        publish_block_max(m3, slots3);
+    }
+}
+
+}  // namespace
+}  // namespace mi8
+
+using namespace mi8;
+
+extern "C" int mi8_swiglu_fwd(const void* x1, const void* x3, void* h, int64_t n, uint32_t* slots_h, void* stream)
+{
+    MI8_REQUIRE(x1 && x3 && h, MI8_ERR_ARG, "mi8_swiglu_fwd: null pointer");
+    MI8_REQUIRE(n > 0 && n % 8 == 0, MI8_ERR_UNSUPPORTED, "mi8_swiglu_fwd: n (%lld) must be a positive multiple of 8",
+                (long long)n);
+    MI8_REQUIRE(aligned16(x1) && aligned16(x3) && aligned16(h), MI8_ERR_UNSUPPORTED,
+                "mi8_swiglu_fwd: pointers must be 16-byte aligned");
+    const int blocks = mi8_amax_slots_for(n);
+    hipLaunchKernelGGL(swiglu_fwd_kernel, dim3(blocks), dim3(kThreads), 0, (hipStream_t)stream, (const uint4*)x1,
+                       (const uint4*)x3, (uint4*)h, n / 8, slots_h);
+    return launch_status("mi8_swiglu_fwd");
+}
+
+extern "C" int mi8_swiglu_bwd(const void* x1, const void* x3, const void* gh, void* g1, void* g3, int64_t n,
+                              uint32_t* slots_g1, uint32_t* slots_g3, void* stream)
+{
+    MI8_REQUIRE(x1 && x3 && gh && g1 && g3, MI8_ERR_ARG, "mi8_swiglu_bwd: null pointer");
+    MI8_REQUIRE(n > 0 && n % 8 == 0, MI8_ERR_UNSUPPORTED, "mi8_swiglu_bwd: n (%lld) must be a positive multiple of 8",
+                (long long)n);
+    MI8_REQUIRE(aligned16(x1) && aligned16(x3) && aligned16(gh) && aligned16(g1) && aligned16(g3),
+                MI8_ERR_UNSUPPORTED, "mi8_swiglu_bwd: pointers must be 16-byte aligned");
+    const int blocks = mi8_amax_slots_for(n);
+    hipLaunchKernelGGL(swiglu_bwd_kernel, dim3(blocks), dim3(kThreads), 0, (hipStream_t)stream, (const uint4*)x1,
+                       (const uint4*)x3, (const uint4*)gh, (uint4*)g1, (uint4*)g3, n / 8, slots_g1, slots_g3);
+    return launch_status("mi8_swiglu_bwd");
+}

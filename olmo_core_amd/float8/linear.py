@@ -1,0 +1,270 @@
+"""
+``Float8Linear`` and the model swap.
+
+The module keeps the ``nn.Linear`` surface (same ``weight`` / ``bias`` Parameters, same state-dict keys) and
+routes its matmuls through one ``torch.autograd.Function`` that quantises the operands with the HIP cast
+kernels and multiplies them on the fp8 matrix cores.  This is the native counterpart of what the reference
+obtains from ``torchao.float8.convert_to_float8_training`` (reference call site:
+src/olmo_core/float8/__init__.py:133-150).
+
+Per linear and training step (M tokens, weight [N, K]):
+
+    output      y  [M, N] = q(x)  [M, K] . q(W)  [N, K]^T
+    grad_input  gx [M, K] = q(go) [M, N] . q(W)^T [K, N]^T
+    grad_weight gW [N, K] = q(go)^T [N, M] . q(x)^T [K, M]^T
+
+Every GEMM reads both operands K-contiguous, so the casts emit row-major and/or transposed fp8 copies:
+tensorwise casts emit both orientations from one pass with one scale; axiswise ("rowwise" recipes) casts
+emit a per-row-scaled row-major copy for operands reduced along their rows and a per-column-scaled
+transposed copy for operands reduced along their columns.
+"""
+
+from __future__ import annotations
+
+from typing import Callable, Optional, Tuple
+
+import torch
+import torch.nn as nn
+
+from . import ops
+from .native_config import CastConfig, Float8LinearConfig, ScalingGranularity, ScalingType
+
+__all__ = ["Float8Linear", "convert_to_float8_training", "float8_linear_function"]
+
+
+def _is_tensorwise(c: CastConfig) -> bool:
+    return c.scaling_type is ScalingType.DYNAMIC and c.scaling_granularity is ScalingGranularity.TENSORWISE
+
+
+def _is_axiswise(c: CastConfig) -> bool:
+    return c.scaling_type is ScalingType.DYNAMIC and c.scaling_granularity is ScalingGranularity.AXISWISE
+
+
+def _is_disabled(c: CastConfig) -> bool:
+    return c.scaling_type is ScalingType.DISABLED
+
+
+def _shared_tensorwise(a: CastConfig, b: CastConfig) -> bool:
+    """Two uses of one tensor that quantise identically (one scale, one dtype): cast once, emit both layouts."""
+    return _is_tensorwise(a) and _is_tensorwise(b) and a.target_dtype == b.target_dtype
+
+
+def _rows_operand(x: torch.Tensor, c: CastConfig, pow2: bool) -> Tuple[torch.Tensor, torch.Tensor]:
+    """Operand reduced along its rows' elements (K = last dim of x): row-major fp8 + scale [1] or [rows]."""
+    if _is_tensorwise(c):
+        q, _, s = ops.cast_tensorwise(x, c.target_dtype, pow2=pow2, want_rowmajor=True, want_transposed=False)
+        return q, s
+    return ops.cast_rowwise(x, c.target_dtype, pow2=pow2)
+
+
+def _cols_operand(x: torch.Tensor, c: CastConfig, pow2: bool) -> Tuple[torch.Tensor, torch.Tensor]:
+    """Operand whose K is x's first dim: transposed fp8 [cols, pad16(rows)] + scale [1] or [cols]."""
+    if _is_tensorwise(c):
+        _, q_t, s = ops.cast_tensorwise(x, c.target_dtype, pow2=pow2, want_rowmajor=False, want_transposed=True)
+        return q_t, s
+    return ops.cast_colwise_t(x, c.target_dtype, pow2=pow2)
+
+
+class _Float8Matmul(torch.autograd.Function):
+    """y = x @ W^T with float8 operands; x [M, K] and W [N, K] in high precision."""
+
+    @staticmethod
+    def forward(ctx, x2: torch.Tensor, weight: torch.Tensor, config: Float8LinearConfig):
+        c = config
+        pow2 = c.round_scales_to_power_of_2
+        need_gx = ctx.needs_input_grad[0]
+        need_gw = ctx.needs_input_grad[1]
+        ctx.config = c
+        ctx.x_dtype = x2.dtype
+        ctx.w_dtype = weight.dtype
+        ctx.shapes = (x2.shape[0], x2.shape[1], weight.shape[0])
+        out_dtype = x2.dtype
+
+        x_saved = w_saved = None
+        x_is_q = w_is_q = False
+        if _is_disabled(c.cast_config_input):
+            y = torch.mm(x2, weight.t().to(x2.dtype))
+        else:
+            share_x = need_gw and _shared_tensorwise(c.cast_config_input, c.cast_config_input_for_grad_weight)
+            share_w = need_gx and _shared_tensorwise(c.cast_config_weight, c.cast_config_weight_for_grad_input)
+            if _is_tensorwise(c.cast_config_input):
+                xq, xq_t, sx = ops.cast_tensorwise(
+                    x2, c.cast_config_input.target_dtype, pow2=pow2, want_rowmajor=True, want_transposed=share_x
+                )
+                if share_x:
+                    x_saved, x_is_q = (xq_t, sx), True
+            else:
+                xq, sx = ops.cast_rowwise(x2, c.cast_config_input.target_dtype, pow2=pow2)
+            if _is_tensorwise(c.cast_config_weight):
+                wq, wq_t, sw = ops.cast_tensorwise(
+                    weight, c.cast_config_weight.target_dtype, pow2=pow2, want_rowmajor=True, want_transposed=share_w
+                )
+                if share_w:
+                    w_saved, w_is_q = (wq_t, sw), True
+            else:
+                wq, sw = ops.cast_rowwise(weight, c.cast_config_weight.target_dtype, pow2=pow2)
+            y = ops.gemm_fp8(xq, sx, wq, sw, out_dtype=out_dtype)
+
+        ctx.x_is_q, ctx.w_is_q = x_is_q, w_is_q
+        to_save = []
+        if need_gw:
+            to_save += list(x_saved) if x_is_q else [x2]
+        if need_gx:
+            to_save += list(w_saved) if w_is_q else [weight]
+        ctx.n_x = (2 if x_is_q else 1) if need_gw else 0
+        ctx.save_for_backward(*to_save)
+        return y
+
+    @staticmethod
+    def backward(ctx, go: torch.Tensor):
+        c: Float8LinearConfig = ctx.config
+        pow2 = c.round_scales_to_power_of_2
+        M, K, N = ctx.shapes
+        need_gx, need_gw = ctx.needs_input_grad[0], ctx.needs_input_grad[1]
+        saved = ctx.saved_tensors
+        x_part, w_part = saved[: ctx.n_x], saved[ctx.n_x :]
+        go2 = go.reshape(M, N)
+        if go2.dtype != ctx.x_dtype:
+            go2 = go2.to(ctx.x_dtype)
+
+        # quantise grad_output once if both backward GEMMs want the same tensorwise cast
+        go_rows = go_cols = None
+        cg, cgw = c.cast_config_grad_output, c.cast_config_grad_output_for_grad_weight
+        if need_gx and need_gw and _shared_tensorwise(cg, cgw):
+            q, q_t, s = ops.cast_tensorwise(go2, cg.target_dtype, pow2=pow2, want_rowmajor=True, want_transposed=True)
+            go_rows, go_cols = (q, s), (q_t, s)
+
+        gx = gw = None
+        if need_gx:
+            if _is_disabled(cg):
+                w = w_part[0]
+                gx = torch.mm(go2, w.to(go2.dtype))
+            else:
+                if go_rows is None:
+                    go_rows = _rows_operand(go2, cg, pow2)
+                if ctx.w_is_q:
+                    w_op = (w_part[0], w_part[1])
+                else:
+                    w_op = _cols_operand(w_part[0], c.cast_config_weight_for_grad_input, pow2)
+                gx = ops.gemm_fp8(go_rows[0], go_rows[1], w_op[0], w_op[1], k=N, out_dtype=ctx.x_dtype)
+        if need_gw:
+            if _is_disabled(cgw):
+                x2 = x_part[0]
+                gw = torch.mm(go2.t(), x2.to(go2.dtype))
+            else:
+                if go_cols is None:
+                    go_cols = _cols_operand(go2, cgw, pow2)
+                if ctx.x_is_q:
+                    x_op = (x_part[0], x_part[1])
+                else:
+                    x_op = _cols_operand(x_part[0], c.cast_config_input_for_grad_weight, pow2)
+                gw = ops.gemm_fp8(go_cols[0], go_cols[1], x_op[0], x_op[1], out_dtype=ctx.x_dtype)
+            if gw.dtype != ctx.w_dtype:
+                gw = gw.to(ctx.w_dtype)
+        return gx, gw, None
+
+
+def float8_linear_function(x: torch.Tensor, weight: torch.Tensor, config: Float8LinearConfig) -> torch.Tensor:
+    """``x [*, K] @ weight[N, K].T`` through the float8 path, differentiable in x and weight."""
+    K = x.shape[-1]
+    if weight.dim() != 2 or weight.shape[1] != K:
+        raise ValueError(f"float8 linear: input features {K} do not match weight {tuple(weight.shape)}")
+    x2 = x.reshape(-1, K)
+    y = _Float8Matmul.apply(x2, weight, config)
+    return y.reshape(*x.shape[:-1], weight.shape[0])
+
+
+class Float8Linear(nn.Linear):
+    """
+    Drop-in ``nn.Linear`` whose forward / backward matmuls run in float8 with dynamic scaling.
+    Use :meth:`from_float` (or :func:`convert_to_float8_training`) to create it from an existing module.
+    """
+
+    def __init__(self, *args, config: Optional[Float8LinearConfig] = None, **kwargs):
+        super().__init__(*args, **kwargs)
+        self.config = config if config is not None else Float8LinearConfig()
+        self._bind_config()
+
+    def _bind_config(self) -> None:
+        c = self.config
+        self.scaling_type_input = c.cast_config_input.scaling_type
+        self.scaling_type_weight = c.cast_config_weight.scaling_type
+        self.scaling_type_grad_output = c.cast_config_grad_output.scaling_type
+
+    def forward(self, input: torch.Tensor) -> torch.Tensor:
+        if torch.is_autocast_enabled():
+            input = input.to(torch.get_autocast_dtype(input.device.type))
+        out = float8_linear_function(input, self.weight, self.config)
+        if self.bias is not None:
+            out = out + self.bias.to(out.dtype)
+        return out
+
+    def extra_repr(self) -> str:
+        c = self.config
+        parts = [
+            f"i:{c.cast_config_input.short_str()}",
+            f"w:{c.cast_config_weight.short_str()}",
+            f"go:{c.cast_config_grad_output.short_str()}",
+        ]
+        if c.cast_config_input_for_grad_weight != c.cast_config_input:
+            parts.append(f"i_gw:{c.cast_config_input_for_grad_weight.short_str()}")
+        if c.cast_config_weight_for_grad_input != c.cast_config_weight:
+            parts.append(f"w_gi:{c.cast_config_weight_for_grad_input.short_str()}")
+        if c.cast_config_grad_output_for_grad_weight != c.cast_config_grad_output:
+            parts.append(f"go_gw:{c.cast_config_grad_output_for_grad_weight.short_str()}")
+        return f'{super().extra_repr()}, cast_configs={",".join(parts)}'
+
+    @classmethod
+    def from_float(cls, mod: nn.Linear, config: Optional[Float8LinearConfig] = None) -> "Float8Linear":
+        """New module sharing ``mod``'s Parameters; reads no weight values (works on the meta device)."""
+        config = config if config is not None else Float8LinearConfig()
+        if config.emulate:
+            raise NotImplementedError(
+                "emulate=True selects a CPU-emulated matmul upstream; this library only has the native gfx950 path"
+            )
+        with torch.device("meta"):
+            new = cls(mod.in_features, mod.out_features, bias=False, config=config)
+        new.weight = mod.weight
+        new.bias = mod.bias
+        return new
+
+
+def _swap(
+    module: nn.Module,
+    make: Callable[[nn.Linear], nn.Module],
+    module_filter_fn: Optional[Callable[[nn.Module, str], bool]],
+) -> nn.Module:
+    """Post-order walk replacing every ``nn.Linear`` the filter accepts; the filter sees only Linears."""
+    if isinstance(module, nn.Linear) and (module_filter_fn is None or module_filter_fn(module, "")):
+        if len(list(module.children())) > 0:
+            raise AssertionError(f"Does not support a root nn.Linear with children: {module}")
+        return make(module)
+
+    visited = set()
+
+    def walk(m: nn.Module, fqn: str, parent: Optional[nn.Module], name: Optional[str]) -> None:
+        if id(m) in visited:
+            return
+        visited.add(id(m))
+        for child_name, child in list(m.named_children()):
+            walk(child, f"{fqn}.{child_name}" if fqn else child_name, m, child_name)
+        if parent is not None and isinstance(m, nn.Linear) and not isinstance(m, Float8Linear):
+            if module_filter_fn is None or module_filter_fn(m, fqn):
+                setattr(parent, name, make(m))
+
+    walk(module, "", None, None)
+    return module
+
+
+def convert_to_float8_training(
+    module: nn.Module,
+    *,
+    module_filter_fn: Optional[Callable[[nn.Module, str], bool]] = None,
+    config: Optional[Float8LinearConfig] = None,
+) -> nn.Module:
+    """
+    Swap ``nn.Linear`` modules for :class:`Float8Linear` in place and return the (possibly new) root.
+    ``module_filter_fn(mod, fqn)`` is consulted for Linear modules only; returning False keeps the module.
+    """
+    config = config if config is not None else Float8LinearConfig()
+    return _swap(module, lambda m: Float8Linear.from_float(m, config), module_filter_fn)

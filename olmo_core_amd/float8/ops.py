@@ -1,0 +1,238 @@
+"""
+Torch-level wrappers over the C ABI: quantised operands and the scaled GEMM.
+
+torch is used here for device memory and streams only: every wrapper allocates its outputs with
+``torch.empty`` on the input's device, passes raw pointers plus the current HIP stream to
+``libmi8.so``, and returns tensors.  Nothing here computes on the host and nothing falls back to
+PyTorch arithmetic.
+"""
+
+from __future__ import annotations
+
+from typing import Optional, Tuple
+
+import torch
+
+from .. import _C
+
+_FP8_CODE = {torch.float8_e4m3fn: _C.MI8_E4M3, torch.float8_e5m2: _C.MI8_E5M2}
+_HP_CODE = {torch.bfloat16: _C.MI8_BF16, torch.float32: _C.MI8_F32}
+
+# Debug/testing switch: convert with the integer-arithmetic path instead of v_cvt_pk_*.
+FORCE_SW_CVT = False
+
+
+def _stream(t: torch.Tensor) -> int:
+    return torch.cuda.current_stream(t.device).cuda_stream
+
+
+def _flags(pow2: bool) -> int:
+    return (_C.FLAG_POW2_SCALE if pow2 else 0) | (_C.FLAG_SW_CVT if FORCE_SW_CVT else 0)
+
+
+def _require_gpu(t: torch.Tensor, what: str) -> None:
+    if not t.is_cuda:
+        raise RuntimeError(f"{what}: expected a tensor on the GPU, got device '{t.device}' (there is no CPU path)")
+
+
+def _hp2d(x: torch.Tensor, what: str) -> torch.Tensor:
+    _require_gpu(x, what)
+    if x.dim() != 2:
+        raise ValueError(f"{what}: expected a 2-D tensor, got shape {tuple(x.shape)}")
+    if x.dtype not in _HP_CODE:
+        raise TypeError(f"{what}: unsupported dtype {x.dtype} (bfloat16 or float32)")
+    if not x.is_contiguous() or x.data_ptr() % 16:
+        x = x.contiguous()
+        if x.data_ptr() % 16:
+            x = x.clone()
+    return x
+
+
+def pad16(n: int) -> int:
+    return (n + 15) // 16 * 16
+
+
+def amax_partials(x: torch.Tensor) -> Tuple[torch.Tensor, int]:
+    """Per-workgroup partial maxima of |x| (as float32 bit patterns); returns (slots, n_used)."""
+    _require_gpu(x, "amax_partials")
+    xc = x if x.is_contiguous() else x.contiguous()
+    slots = torch.empty(_C.AMAX_SLOTS, dtype=torch.int32, device=x.device)
+    used = _C.c_int32(0)
+    _C.check(
+        _C.lib().mi8_amax_partials(xc.data_ptr(), _HP_CODE[xc.dtype], xc.numel(), slots.data_ptr(), used, _stream(x)),
+        "mi8_amax_partials",
+    )
+    return slots, used.value
+
+
+def scale_from_partials(slots: torch.Tensor, n_slots: int, fp8_dtype: torch.dtype, pow2: bool = False) -> torch.Tensor:
+    """Returns a float32 tensor [2] = (scale, amax)."""
+    out = torch.empty(2, dtype=torch.float32, device=slots.device)
+    _C.check(
+        _C.lib().mi8_scale_from_partials(
+            slots.data_ptr(), n_slots, _FP8_CODE[fp8_dtype], _flags(pow2), out.data_ptr(), _stream(slots)
+        ),
+        "mi8_scale_from_partials",
+    )
+    return out
+
+
+def tensor_to_scale(x: torch.Tensor, fp8_dtype: torch.dtype, pow2: bool = False) -> torch.Tensor:
+    """Tensorwise dynamic scale of ``x`` (0-d float32 tensor on x's device)."""
+    slots, used = amax_partials(x)
+    return scale_from_partials(slots, used, fp8_dtype, pow2)[0]
+
+
+def cast_tensorwise(
+    x: torch.Tensor,
+    fp8_dtype: torch.dtype,
+    *,
+    pow2: bool = False,
+    want_rowmajor: bool = True,
+    want_transposed: bool = False,
+    slots: Optional[Tuple[torch.Tensor, int]] = None,
+    scale: Optional[torch.Tensor] = None,
+) -> Tuple[Optional[torch.Tensor], Optional[torch.Tensor], torch.Tensor]:
+    """
+    Quantise ``x [rows, cols]`` with one scale.  Returns ``(q, q_t, scale)``: ``q`` fp8 ``[rows, cols]``,
+    ``q_t`` fp8 ``[cols, pad16(rows)]`` (zero padded), ``scale`` float32 ``[1]``.  The scale comes from
+    ``scale`` if given, else from amax partials (``slots`` if already computed by a producer kernel).
+    """
+    x = _hp2d(x, "cast_tensorwise")
+    rows, cols = x.shape
+    dev = x.device
+    if scale is None and slots is None:
+        slots = amax_partials(x)
+    q = torch.empty((rows, cols), dtype=fp8_dtype, device=dev) if want_rowmajor else None
+    ld_t = pad16(rows)
+    q_t = torch.empty((cols, ld_t), dtype=fp8_dtype, device=dev) if want_transposed else None
+    scale_out = torch.empty(1, dtype=torch.float32, device=dev)
+    if scale is not None:
+        scale = scale.reshape(1).to(torch.float32)
+    _C.check(
+        _C.lib().mi8_cast_tensorwise(
+            x.data_ptr(), _HP_CODE[x.dtype], rows, cols,
+            slots[0].data_ptr() if scale is None else None, slots[1] if scale is None else 0,
+            scale.data_ptr() if scale is not None else None,
+            _FP8_CODE[fp8_dtype], _flags(pow2),
+            q.data_ptr() if q is not None else None,
+            q_t.data_ptr() if q_t is not None else None, ld_t,
+            scale_out.data_ptr(), _stream(x),
+        ),
+        "mi8_cast_tensorwise",
+    )
+    return q, q_t, scale_out
+
+
+def cast_rowwise(x: torch.Tensor, fp8_dtype: torch.dtype, *, pow2: bool = False) -> Tuple[torch.Tensor, torch.Tensor]:
+    """One scale per row: returns (q fp8 [rows, cols], scale float32 [rows])."""
+    x = _hp2d(x, "cast_rowwise")
+    rows, cols = x.shape
+    q = torch.empty((rows, cols), dtype=fp8_dtype, device=x.device)
+    s = torch.empty(rows, dtype=torch.float32, device=x.device)
+    _C.check(
+        _C.lib().mi8_cast_rowwise(
+            x.data_ptr(), _HP_CODE[x.dtype], rows, cols, _FP8_CODE[fp8_dtype], _flags(pow2), q.data_ptr(),
+            s.data_ptr(), _stream(x),
+        ),
+        "mi8_cast_rowwise",
+    )
+    return q, s
+
+
+def cast_colwise_t(x: torch.Tensor, fp8_dtype: torch.dtype, *, pow2: bool = False) -> Tuple[torch.Tensor, torch.Tensor]:
+    """One scale per column, transposed output: returns (q_t fp8 [cols, pad16(rows)], scale float32 [cols])."""
+    x = _hp2d(x, "cast_colwise_t")
+    rows, cols = x.shape
+    ld_t = pad16(rows)
+    q_t = torch.empty((cols, ld_t), dtype=fp8_dtype, device=x.device)
+    s = torch.empty(cols, dtype=torch.float32, device=x.device)
+    ws = torch.empty(_C.lib().mi8_colamax_workspace_slots(rows, cols), dtype=torch.int32, device=x.device)
+    _C.check(
+        _C.lib().mi8_cast_colwise_t(
+            x.data_ptr(), _HP_CODE[x.dtype], rows, cols, _FP8_CODE[fp8_dtype], _flags(pow2), ws.data_ptr(),
+            q_t.data_ptr(), ld_t, s.data_ptr(), _stream(x),
+        ),
+        "mi8_cast_colwise_t",
+    )
+    return q_t, s
+
+
+def gemm_fp8(
+    a: torch.Tensor,
+    sa: torch.Tensor,
+    b: torch.Tensor,
+    sb: torch.Tensor,
+    *,
+    k: Optional[int] = None,
+    out_dtype: torch.dtype = torch.bfloat16,
+    variant: int = -1,
+) -> torch.Tensor:
+    """
+    ``out[M, N] = (a[M, :k] @ b[N, :k].T) / sa / sb`` with fp32 accumulation on the fp8 matrix cores.
+    ``a`` and ``b`` are fp8 tensors whose rows are K-contiguous; ``sa`` / ``sb`` hold one scale or one per row.
+    """
+    _require_gpu(a, "gemm_fp8")
+    if a.dim() != 2 or b.dim() != 2 or a.stride(1) != 1 or b.stride(1) != 1:
+        raise ValueError("gemm_fp8: operands must be 2-D with contiguous rows")
+    if a.dtype not in _FP8_CODE or b.dtype not in _FP8_CODE:
+        raise TypeError(f"gemm_fp8: operands must be float8, got {a.dtype} and {b.dtype}")
+    if out_dtype not in _HP_CODE:
+        raise TypeError(f"gemm_fp8: unsupported output dtype {out_dtype}")
+    M, N = a.shape[0], b.shape[0]
+    K = min(a.shape[1], b.shape[1]) if k is None else k
+    if sa.numel() not in (1, M) or sb.numel() not in (1, N):
+        raise ValueError(f"gemm_fp8: scale sizes {sa.numel()}, {sb.numel()} do not match M={M}, N={N}")
+    out = torch.empty((M, N), dtype=out_dtype, device=a.device)
+    _C.check(
+        _C.lib().mi8_gemm_fp8(
+            a.data_ptr(), _FP8_CODE[a.dtype], a.stride(0), b.data_ptr(), _FP8_CODE[b.dtype], b.stride(0), M, N, K,
+            sa.data_ptr(), int(sa.numel() != 1),
+            sb.data_ptr(), int(sb.numel() != 1),
+            out.data_ptr(), _HP_CODE[out_dtype], out.stride(0), variant, _stream(a),
+        ),
+        "mi8_gemm_fp8",
+    )
+    return out
+
+
+def gemm_variants() -> list:
+    L = _C.lib()
+    return [L.mi8_gemm_variant_name(i).decode() for i in range(L.mi8_gemm_num_variants())]
+
+
+def swiglu_fwd(x1: torch.Tensor, x3: torch.Tensor, want_amax: bool = True):
+    """h = silu(x1) * x3 (bf16); optionally the amax partials of h for the cast that follows."""
+    _require_gpu(x1, "swiglu_fwd")
+    if x1.dtype != torch.bfloat16 or x3.dtype != torch.bfloat16 or x1.shape != x3.shape:
+        raise TypeError("swiglu_fwd: expects two bfloat16 tensors of the same shape")
+    x1, x3 = x1.contiguous(), x3.contiguous()
+    h = torch.empty_like(x1)
+    slots = torch.empty(_C.AMAX_SLOTS, dtype=torch.int32, device=x1.device) if want_amax else None
+    n = x1.numel()
+    _C.check(
+        _C.lib().mi8_swiglu_fwd(
+            x1.data_ptr(), x3.data_ptr(), h.data_ptr(), n, slots.data_ptr() if want_amax else None, _stream(x1)
+        ),
+        "mi8_swiglu_fwd",
+    )
+    return h, ((slots, _C.lib().mi8_amax_slots_for(n)) if want_amax else None)
+
+
+def swiglu_bwd(x1: torch.Tensor, x3: torch.Tensor, gh: torch.Tensor, want_amax: bool = True):
+    """Gradients of h = silu(x1) * x3 w.r.t. x1 and x3 (bf16) and optionally their amax partials."""
+    _require_gpu(x1, "swiglu_bwd")
+    x1, x3, gh = x1.contiguous(), x3.contiguous(), gh.contiguous()
+    g1, g3 = torch.empty_like(x1), torch.empty_like(x1)
+    n = x1.numel()
+    s1 = torch.empty(_C.AMAX_SLOTS, dtype=torch.int32, device=x1.device) if want_amax else None
+    s3 = torch.empty(_C.AMAX_SLOTS, dtype=torch.int32, device=x1.device) if want_amax else None
+    _C.check(
+        _C.lib().mi8_swiglu_bwd(
+            x1.data_ptr(), x3.data_ptr(), gh.data_ptr(), g1.data_ptr(), g3.data_ptr(), n,
+            s1.data_ptr() if want_amax else None, s3.data_ptr() if want_amax else None, _stream(x1),
+        ),
+        "mi8_swiglu_bwd",
+    )
+    used = _C.lib().mi8_amax_slots_for(n)
+    return g1, g3, ((s1, used) if want_amax else None), ((s3, used) if want_amax else None)

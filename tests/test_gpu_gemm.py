@@ -1,0 +1,136 @@
+"""Parity of the scaled fp8 GEMM with the oracle's emulated matmul (tolerance stated in helpers.py) and
+exactness on integer-valued operands."""
+
+import pytest
+import torch
+
+from helpers import E4M3, E5M2, assert_gemm_close, seeded
+from oracle import float8_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+from olmo_core_amd.float8 import ops  # noqa: E402
+
+
+def _variants():
+    return list(range(len(ops.gemm_variants())))
+
+
+def _int_operand(shape, seed, dtype):
+    g = torch.Generator().manual_seed(seed)
+    return torch.randint(-2, 3, shape, generator=g).float().to(dtype)
+
+
+EXACT_SHAPES = [(32, 32, 64), (1, 16, 16), (33, 48, 144), (256, 256, 128), (300, 272, 1040), (257, 513, 4096), (512, 768, 16)]
+
+
+@pytest.mark.parametrize("mnk", EXACT_SHAPES, ids=lambda s: "x".join(map(str, s)))
+def test_integer_operands_exact(dev, mnk):
+    """Operands in {-2..2}: every product and partial sum is an integer below 2^24, so fp32 accumulation in any
+    order is exact and the output must equal the integer matmul exactly - any wrong index, dropped k-chunk or
+    mis-mapped accumulator register changes the result."""
+    M, N, K = mnk
+    one = torch.ones(1, device=dev)
+    for da, db in ((E4M3, E4M3), (E5M2, E4M3), (E4M3, E5M2), (E5M2, E5M2)):
+        a = _int_operand((M, K), 1, da)
+        b = _int_operand((N, K), 2, db)
+        ref = a.float() @ b.float().t()
+        for v in _variants():
+            out = ops.gemm_fp8(a.to(dev), one, b.to(dev), one, out_dtype=torch.float32, variant=v)
+            assert torch.equal(out.cpu(), ref), f"variant {ops.gemm_variants()[v]} {da} x {db}: max diff {(out.cpu() - ref).abs().max()}"
+
+
+def test_integer_operands_exact_padded_pitch(dev):
+    """Row pitch larger than K (the zero-padded transposed copies): only the first K bytes of a row count."""
+    M, N, K, ld = 100, 80, 112, 128
+    a = torch.zeros(M, ld, dtype=E4M3); a[:, :K] = _int_operand((M, K), 3, E4M3); a[:, K:] = 1.0
+    b = torch.zeros(N, ld, dtype=E4M3); b[:, :K] = _int_operand((N, K), 4, E4M3); b[:, K:] = 1.0
+    ref = a[:, :K].float() @ b[:, :K].float().t()
+    one = torch.ones(1, device=dev)
+    for v in _variants():
+        out = ops.gemm_fp8(a.to(dev), one, b.to(dev), one, k=K, out_dtype=torch.float32, variant=v)
+        assert torch.equal(out.cpu(), ref)
+
+
+PARITY_SHAPES = [(64, 96, 128), (2048, 1024, 512), (300, 272, 1040), (128, 4096, 4096), (1000, 11008, 256)]
+
+
+@pytest.mark.parametrize("mnk", PARITY_SHAPES, ids=lambda s: "x".join(map(str, s)))
+@pytest.mark.parametrize("gran", ["tensorwise", "axiswise"])
+def test_against_emulated_mm(dev, mnk, gran):
+    M, N, K = mnk
+    x = seeded((M, K), seed=M + K, std=1.0)
+    w = seeded((N, K), seed=N + 1, std=0.02)
+    if gran == "tensorwise":
+        a8, sa = O.cast(x, E4M3)
+        b8, sb = O.cast(w, E4M3)
+        ref = O.emulated_mm_f32(a8, sa, b8.t(), sb)
+        sa_d, sb_d = sa.reshape(1).to(dev), sb.reshape(1).to(dev)
+    else:
+        a8, sa = O.cast(x, E4M3, O.AXISWISE, -1, True)
+        b8, sb = O.cast(w, E4M3, O.AXISWISE, -1, True)
+        ref = O.emulated_mm_f32(a8, sa, b8.t(), sb.t())
+        sa_d, sb_d = sa.reshape(-1).to(dev), sb.reshape(-1).to(dev)
+    for v in _variants():
+        out = ops.gemm_fp8(a8.to(dev), sa_d, b8.to(dev), sb_d, variant=v)
+        assert out.dtype == torch.bfloat16
+        assert_gemm_close(out, ref, f"variant {v}")
+        out32 = ops.gemm_fp8(a8.to(dev), sa_d, b8.to(dev), sb_d, out_dtype=torch.float32, variant=v)
+        assert_gemm_close(out32, ref, f"variant {v} f32")
+        # bf16 output is the rounding of the fp32 output
+        assert torch.equal(out32.bfloat16(), out)
+
+
+def test_scaled_mm_library_crosscheck(dev):
+    """Tensorwise case against torch-CPU's own _scaled_mm (library routine)."""
+    x = seeded((96, 256), 1)
+    w = seeded((160, 256), 2, std=0.02)
+    a8, sa = O.cast(x, E4M3)
+    b8, sb = O.cast(w, E4M3)
+    ref = torch._scaled_mm(a8, b8.t(), scale_a=sa.reciprocal(), scale_b=sb.reciprocal(), out_dtype=torch.float32)
+    out = ops.gemm_fp8(a8.to(dev), sa.reshape(1).to(dev), b8.to(dev), sb.reshape(1).to(dev), out_dtype=torch.float32)
+    assert_gemm_close(out, ref)
+
+
+def test_mixed_dtypes_gradient_shapes(dev):
+    """e5m2 x e4m3 with a long, padded K: the grad_weight call shape."""
+    M_tok, N, K = 1000, 272, 144
+    go = seeded((M_tok, N), 5, std=1e-3)
+    x = seeded((M_tok, K), 6)
+    go8, sg = O.cast(go, E5M2)
+    x8, sx = O.cast(x, E4M3)
+    ref = O.emulated_mm_f32(go8.t(), sg, x8, sx)
+    ld = ops.pad16(M_tok)
+    a = torch.zeros(N, ld, dtype=E5M2); a[:, :M_tok] = go8.t()
+    b = torch.zeros(K, ld, dtype=E4M3); b[:, :M_tok] = x8.t()
+    out = ops.gemm_fp8(a.to(dev), sg.reshape(1).to(dev), b.to(dev), sx.reshape(1).to(dev), out_dtype=torch.float32)
+    assert_gemm_close(out, ref)
+
+
+def test_full_size_row_sample(dev):
+    """7B MLP up-projection at full size (16384 x 11008 x 4096): a sample of output rows against the oracle."""
+    M, N, K = 16384, 11008, 4096
+    x = seeded((M, K), 1002)
+    w = seeded((N, K), 1003, std=0.02)
+    xq, _, sx = ops.cast_tensorwise(x.to(dev), E4M3)
+    wq, _, sw = ops.cast_tensorwise(w.to(dev), E4M3)
+    out = ops.gemm_fp8(xq, sx, wq, sw)
+    rows = torch.arange(5, M, 1021)
+    ref = O.emulated_mm_f32(xq[rows.to(dev)].cpu(), sx.cpu()[0], wq.cpu().t(), sw.cpu()[0])
+    assert_gemm_close(out[rows.to(dev)], ref, "row sample")
+    # linearity in the scales: doubling a scale halves the output exactly (power of two)
+    out2 = ops.gemm_fp8(xq, sx * 2, wq, sw)
+    assert torch.equal(out2[rows.to(dev)].float() * 2, out[rows.to(dev)].float())
+
+
+def test_argument_errors(dev):
+    from olmo_core_amd.exceptions import MI8KernelError
+
+    a = torch.zeros(16, 24, dtype=E4M3, device=dev)
+    one = torch.ones(1, device=dev)
+    with pytest.raises(MI8KernelError):
+        ops.gemm_fp8(a, one, a, one)  # K not a multiple of 16
+    with pytest.raises(TypeError):
+        ops.gemm_fp8(a.view(torch.uint8), one, a, one)
+    with pytest.raises(ValueError):
+        ops.gemm_fp8(torch.zeros(16, 32, dtype=E4M3, device=dev), torch.ones(3, device=dev), a, one)

