@@ -1,0 +1,174 @@
+"""
+Benchmark of the float8 linear hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+A "step" is one forward+backward pass of the OLMo-2-7B-shape SwiGLU feed-forward block
+(d_model 4096, hidden 11008, tokens M = 16384 = batch 4 x seq 4096) with all three projections float8
+tensorwise (e4m3 forward operands, e5m2 grad_output), synthetic seeded inputs resident in HBM.
+Prints ONE JSON line: whole-step throughput in TFLOP/s (2*M*N*K per GEMM, 9 GEMMs per step), the
+roofline of the dominant kernel (the fp8 GEMM, timed with HIP events on its launch stream during the
+timed region) and the CPU baseline (the oracle's emulated float8 path on the host cores, on a bounded
+sample of the same workload).
+"""
+
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+import torch
+
+D_MODEL, HIDDEN, TOKENS = 4096, 11008, 16384
+FP8_MFMA_PEAK_TFLOPS = 5000.0  # MI355X dense fp8 matrix peak
+GEMMS_PER_STEP = 9
+
+
+def build_mlp(dev):
+    from olmo_core_amd.float8 import AOFloat8LinearRecipe, Float8Config
+    from olmo_core_amd.nn import FeedForward
+
+    g = torch.Generator().manual_seed(1002)
+    mlp = FeedForward(d_model=D_MODEL, hidden_size=HIDDEN, bias=False, dtype=torch.bfloat16)
+    with torch.no_grad():
+        for p in mlp.parameters():
+            p.copy_((torch.randn(p.shape, generator=g) * 0.02).to(torch.bfloat16))
+    mlp = mlp.to(dev)
+    Float8Config(ao_recipe=AOFloat8LinearRecipe.tensorwise).apply_float8_linear(mlp)
+    x = torch.randn(TOKENS, D_MODEL, generator=g).to(torch.bfloat16).to(dev).requires_grad_(True)
+    go = (torch.randn(TOKENS, D_MODEL, generator=g) * 1e-3).to(torch.bfloat16).to(dev)
+    return mlp, x, go
+
+
+def step(mlp, x, go):
+    x.grad = None
+    for p in mlp.parameters():
+        p.grad = None
+    y = mlp(x)
+    y.backward(go)
+
+
+def cpu_baseline(target_seconds: float = 15.0):
+    """The oracle's emulated path (fp32 matmul on dequantised fp8 operands) on the host cores, MLP fwd+bwd at
+    a reduced token count chosen to take about `target_seconds`."""
+    sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
+    from oracle import float8_oracle as O
+
+    cores = int(os.environ.get("OMP_NUM_THREADS", 0)) or os.cpu_count() or 1
+    cores = min(cores, os.cpu_count() or cores)
+    torch.set_num_threads(cores)
+    g = torch.Generator().manual_seed(1002)
+    w1 = (torch.randn(HIDDEN, D_MODEL, generator=g) * 0.02).bfloat16()
+    w2 = (torch.randn(D_MODEL, HIDDEN, generator=g) * 0.02).bfloat16()
+    w3 = (torch.randn(HIDDEN, D_MODEL, generator=g) * 0.02).bfloat16()
+    spec = O.recipe("tensorwise")
+
+    def run(m):
+        x = torch.randn(m, D_MODEL, generator=g).bfloat16()
+        go = (torch.randn(m, D_MODEL, generator=g) * 1e-3).bfloat16()
+        t0 = time.perf_counter()
+        O.mlp_fwd_bwd(x, w1, w2, w3, go, spec)
+        return time.perf_counter() - t0
+
+    probe_m = 256
+    run(probe_m)  # warm the thread pool
+    t_probe = run(probe_m)
+    m = int(min(TOKENS, max(probe_m, probe_m * target_seconds / max(t_probe, 1e-3))))
+    m = max(256, (m // 256) * 256)
+    t = run(m)
+    flops = GEMMS_PER_STEP * 2.0 * m * D_MODEL * HIDDEN
+    return {
+        "value": round(flops / t / 1e12, 4),
+        "unit": "TFLOP/s",
+        "cores": cores,
+        "kind": "port",
+        "sample": f"oracle emulated float8 MLP fwd+bwd (fp32 torch-CPU matmul), {m} of {TOKENS} tokens, {t:.1f} s, same weights shape",
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ns = ap.parse_args()
+    if ns.gpus != 1:
+        print("bench.py: this build measures the float8 linear path on ONE GPU; --gpus must be 1", file=sys.stderr)
+        sys.exit(2)
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible; the float8 path has no CPU implementation", file=sys.stderr)
+        sys.exit(2)
+
+    from olmo_core_amd.float8 import ops
+
+    dev = torch.device("cuda:0")
+    mlp, x, go = build_mlp(dev)
+
+    for _ in range(ns.warmup):
+        step(mlp, x, go)
+    torch.cuda.synchronize()
+
+    events = []
+    ops.GEMM_EVENT_SINK = events  # every GEMM launch is bracketed by HIP events on its stream
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(ns.steps):
+        step(mlp, x, go)
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    ops.GEMM_EVENT_SINK = None
+
+    ms_per_step = elapsed / ns.steps * 1e3
+    flops_per_step = GEMMS_PER_STEP * 2.0 * TOKENS * D_MODEL * HIDDEN
+    tflops = flops_per_step / (ms_per_step * 1e-3) / 1e12
+
+    gemm_ms = [s.elapsed_time(e) for s, e, _ in events]
+    assert len(gemm_ms) == GEMMS_PER_STEP * ns.steps, (len(gemm_ms), ns.steps)
+    avg_gemm_s = sum(gemm_ms) / len(gemm_ms) * 1e-3
+    flops_per_launch = 2.0 * TOKENS * D_MODEL * HIDDEN
+    achieved = flops_per_launch / avg_gemm_s / 1e12
+
+    result = {
+        "metric": "Float8Linear fwd+bwd TFLOP/s at 7B MLP shape",
+        "value": round(tflops, 2),
+        "unit": "TFLOP/s",
+        "n_gpus": 1,
+        "steps": ns.steps,
+        "warmup": ns.warmup,
+        "ms_per_step": round(ms_per_step, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "fp8 (e4m3/e5m2 operands, fp32 accumulate, bf16 out)",
+        "data": "synthetic (seeded N(0,1) activations, N(0,0.02) weights, N(0,1e-3) grad_output)",
+        "config": {
+            "workload": "OLMo-2-7B SwiGLU MLP fwd+bwd, w1/w3 4096->11008, w2 11008->4096, tokens 16384, float8 tensorwise",
+            "tokens": TOKENS,
+            "d_model": D_MODEL,
+            "hidden": HIDDEN,
+            "recipe": "tensorwise",
+        },
+        "pct_fp8_mfma_peak": round(100.0 * tflops / FP8_MFMA_PEAK_TFLOPS, 2),
+        "roofline": {
+            "kernel": "gemm_fp8_kernel (9 launches per step, 2*16384*4096*11008 flop each)",
+            "bound": "mfma",
+            "achieved": round(achieved, 2),
+            "peak": FP8_MFMA_PEAK_TFLOPS,
+            "unit": "TFLOP/s",
+            "frac": round(achieved / FP8_MFMA_PEAK_TFLOPS, 4),
+            "traffic": None,
+            "avg_launch_us": round(avg_gemm_s * 1e6, 2),
+            "gemm_share_of_step": round(sum(gemm_ms) / ns.steps / ms_per_step, 4),
+        },
+    }
+    if not ns.no_cpu_baseline:
+        result["cpu_baseline"] = cpu_baseline()
+    print(json.dumps(result), flush=True)
+
+
+if __name__ == "__main__":
+    main()

@@ -222,6 +222,7 @@ class Float8Linear(nn.Linear):
             raise NotImplementedError(
                 "emulate=True selects a CPU-emulated matmul upstream; this library only has the native gfx950 path"
             )
+        config.check_gemm_operands()
         with torch.device("meta"):
             new = cls(mod.in_features, mod.out_features, bias=False, config=config)
         new.weight = mod.weight

@@ -21,6 +21,10 @@ _HP_CODE = {torch.bfloat16: _C.MI8_BF16, torch.float32: _C.MI8_F32}
 # Debug/testing switch: convert with the integer-arithmetic path instead of v_cvt_pk_*.
 FORCE_SW_CVT = False
 
+# Measurement hook: when set to a list, every GEMM launch appends (start_event, end_event, (M, N, K)) recorded
+# on the launch stream.
+GEMM_EVENT_SINK = None
+
 
 def _stream(t: torch.Tensor) -> int:
     return torch.cuda.current_stream(t.device).cuda_stream
@@ -184,6 +188,10 @@ def gemm_fp8(
     if sa.numel() not in (1, M) or sb.numel() not in (1, N):
         raise ValueError(f"gemm_fp8: scale sizes {sa.numel()}, {sb.numel()} do not match M={M}, N={N}")
     out = torch.empty((M, N), dtype=out_dtype, device=a.device)
+    sink = GEMM_EVENT_SINK
+    if sink is not None:
+        ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        ev0.record()
     _C.check(
         _C.lib().mi8_gemm_fp8(
             a.data_ptr(), _FP8_CODE[a.dtype], a.stride(0), b.data_ptr(), _FP8_CODE[b.dtype], b.stride(0), M, N, K,
@@ -193,6 +201,9 @@ def gemm_fp8(
         ),
         "mi8_gemm_fp8",
     )
+    if sink is not None:
+        ev1.record()
+        sink.append((ev0, ev1, (M, N, K)))
     return out
 
 

@@ -32,10 +32,12 @@ def bits32(t: torch.Tensor) -> torch.Tensor:
     return t.detach().contiguous().view(torch.int32).cpu()
 
 
-def assert_bytes_equal(got: torch.Tensor, ref: torch.Tensor, what: str = ""):
+def assert_bytes_equal(got: torch.Tensor, ref: torch.Tensor, what: str = "", fp8: torch.dtype = None):
     """Bit-exact comparison of fp8 bytes; where both sides hold a NaN code only NaN-ness must match
     (the sign/payload of a NaN produced by a multiply differs between x86 and the GPU)."""
-    nan_floor = 0x7D if ref.dtype == torch.float8_e5m2 else 0x7F  # e5m2 NaN codes 0x7D..0x7F; e4m3fn NaN 0x7F
+    fp8 = fp8 if fp8 is not None else (ref.dtype if ref.dtype in (E4M3, E5M2) else got.dtype)
+    assert fp8 in (E4M3, E5M2), "cannot tell which float8 encoding is being compared"
+    nan_floor = 0x7D if fp8 == E5M2 else 0x7F  # e5m2 NaN codes 0x7D..0x7F; e4m3fn NaN 0x7F
     got, ref = u8(got), u8(ref)
     assert got.shape == ref.shape, f"{what}: shape {tuple(got.shape)} vs {tuple(ref.shape)}"
     neq = got != ref

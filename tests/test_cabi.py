@@ -1,0 +1,48 @@
+"""The C-ABI library loads and exports every symbol include/mi8.h declares (no GPU work is launched)."""
+
+import ctypes
+import re
+from pathlib import Path
+
+import pytest
+
+from olmo_core_amd import _C
+
+ROOT = Path(__file__).resolve().parent.parent
+
+
+def _declared_symbols():
+    text = (ROOT / "include" / "mi8.h").read_text()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(mi8_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_header_and_binding_agree():
+    assert _declared_symbols() == sorted(_C.EXPORTED_SYMBOLS)
+
+
+def test_library_exports_every_declared_symbol():
+    assert _C.is_built(), "libmi8.so is not built: run `python -m olmo_core_amd.build`"
+    handle = ctypes.CDLL(str(_C.LIB_PATH))
+    for name in _declared_symbols():
+        assert hasattr(handle, name), f"libmi8.so does not export {name}"
+
+
+def test_host_only_entry_points():
+    L = _C.lib()
+    assert L.mi8_version() == 100
+    assert L.mi8_gemm_num_variants() >= 1
+    assert L.mi8_gemm_variant_name(0)
+    assert L.mi8_gemm_variant_name(999) is None
+    assert L.mi8_amax_slots_for(1) == 1
+    assert L.mi8_amax_slots_for(1 << 40) == _C.AMAX_SLOTS
+    assert L.mi8_colamax_workspace_slots(16384, 4096) % 4096 == 0
+
+
+def test_argument_validation_happens_before_any_gpu_call():
+    L = _C.lib()
+    assert L.mi8_cast_rowwise(None, 0, 4, 16, 0, 0, None, None, None) == -1
+    assert "null" in _C.last_error()
+    assert L.mi8_gemm_fp8(None, 0, 16, None, 0, 16, 1, 1, 16, None, 0, None, 0, None, 0, 16, -1, None) == -1
+    with pytest.raises(Exception):
+        _C.check(-2, "x")
