@@ -1,0 +1,68 @@
+// Shared pieces of the fp8 GEMM kernels (argument block, LDS swizzle, tile order).
+#pragma once
+#include "mi8_common.h"
+
+namespace mi8 {
+namespace gemm {
+
+typedef int v8i __attribute__((ext_vector_type(8)));
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef float v16f __attribute__((ext_vector_type(16)));
+
+constexpr int BK = 128;  // bytes of K per LDS stage
+
+struct GemmArgs {
+    const uint8_t* A;
+    const uint8_t* B;
+    void* C;
+    int c_f32;
+    int64_t lda, ldb, ldc;
+    int M, N, K;
+    const float* sa;
+    const float* sb;
+    int sa_vec, sb_vec;
+    int tiles_m, tiles_n;
+};
+
+__device__ __forceinline__ int swz(int r) { return (r ^ (r >> 3)) & 7; }
+
+__device__ __forceinline__ uint16_t f32_to_bf16_bits(float f)
+{
+    __bf16 h = (__bf16)f;  // round-to-nearest-even; v_cvt_pk_bf16_f32 on gfx950
+    return __builtin_bit_cast(uint16_t, h);
+}
+
+// Linear tile index -> tile coordinates: tiles are walked in groups of 8 tile-rows (all columns of the group
+// before the next group) so that tiles with neighbouring indices share A and B panels.
+__device__ __forceinline__ void tile_coords(const GemmArgs& g, int t, int& tm, int& tn)
+{
+    constexpr int GROUP = 8;
+    const int span = GROUP * g.tiles_n;
+    const int first_m = (t / span) * GROUP;
+    const int gsz = (g.tiles_m - first_m < GROUP) ? g.tiles_m - first_m : GROUP;
+    const int in = t % span;
+    tm = first_m + in % gsz;
+    tn = in / gsz;
+}
+
+// Workgroup id -> output tile.  Consecutive workgroup ids are spread round-robin over the 8 XCDs, each with
+// its own L2; give every XCD a contiguous range of tiles so that the workgroups resident on one XCD share A
+// and B panels in its L2.
+__device__ __forceinline__ bool tile_of_block(const GemmArgs& g, int& tm, int& tn)
+{
+    constexpr int XCDS = 8;
+    const int total = g.tiles_m * g.tiles_n;
+    const int per_xcd = (total + XCDS - 1) / XCDS;
+    const int b = (int)blockIdx.x;
+    const int t = (b % XCDS) * per_xcd + b / XCDS;
+    if (t >= total) return false;
+    tile_coords(g, t, tm, tn);
+    return true;
+}
+
+// pipelined persistent kernel (mi8_gemm_pipe.hip); requires M, N >= 256, K % 128 == 0, N % 8 == 0, ldc % 8 == 0
+// and a 16-byte aligned output
+int launch_pipelined(GemmArgs& g, int a_dtype, int b_dtype, hipStream_t st);
+
+}  // namespace gemm
+}  // namespace mi8

@@ -7,57 +7,11 @@
 // LDS stage layout: [row][128 bytes]; the 16-byte chunk c of row r sits at chunk position c ^ swz(r),
 // swz(r) = (r ^ (r >> 3)) & 7, so that the 16-byte fragment reads of 32 different rows spread over all banks
 // while the stores (8 lanes per row) stay contiguous.
-#include "mi8_common.h"
+#include "mi8_gemm.h"
 
 namespace mi8 {
+using namespace gemm;
 namespace {
-
-typedef int v8i __attribute__((ext_vector_type(8)));
-typedef int v4i __attribute__((ext_vector_type(4)));
-typedef float v16f __attribute__((ext_vector_type(16)));
-
-constexpr int BK = 128;  // bytes of K per LDS stage
-
-struct GemmArgs {
-    const uint8_t* A;
-    const uint8_t* B;
-    void* C;
-    int c_f32;
-    int64_t lda, ldb, ldc;
-    int M, N, K;
-    const float* sa;
-    const float* sb;
-    int sa_vec, sb_vec;
-    int tiles_m, tiles_n;
-};
-
-__device__ __forceinline__ int swz(int r) { return (r ^ (r >> 3)) & 7; }
-
-__device__ __forceinline__ uint16_t f32_to_bf16_bits(float f)
-{
-    __bf16 h = (__bf16)f;  // round-to-nearest-even; v_cvt_pk_bf16_f32 on gfx950
-    return __builtin_bit_cast(uint16_t, h);
-}
-
-// Workgroup id -> output tile.  Consecutive workgroup ids are spread round-robin over the 8 XCDs, each with
-// its own L2; give every XCD a contiguous range of tiles and walk that range in groups of 8 tile-rows so that
-// the workgroups resident on one XCD share A and B panels in its L2.
-__device__ __forceinline__ bool tile_of_block(const GemmArgs& g, int& tm, int& tn)
-{
-    constexpr int XCDS = 8, GROUP = 8;
-    const int total = g.tiles_m * g.tiles_n;
-    const int per_xcd = (total + XCDS - 1) / XCDS;
-    const int b = (int)blockIdx.x;
-    const int t = (b % XCDS) * per_xcd + b / XCDS;
-    if (t >= total) return false;
-    const int span = GROUP * g.tiles_n;
-    const int first_m = (t / span) * GROUP;
-    const int gsz = (g.tiles_m - first_m < GROUP) ? g.tiles_m - first_m : GROUP;
-    const int in = t % span;
-    tm = first_m + in % gsz;
-    tn = in / gsz;
-    return true;
-}
 
 template <int BM, int BN, int WM, int WN, int CBSZ, int BLGP>
 __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_fp8_kernel(GemmArgs g)
@@ -227,7 +181,9 @@ constexpr Variant kVariants[] = {
     {"128x128_w2x2", 128, 128, 256},
     {"256x128_w2x2", 256, 128, 256},
     {"128x256_w2x2", 128, 256, 256},
+    {"256x256_pipelined_persistent", 256, 256, 256},
 };
+constexpr int kPipelined = 5;
 constexpr int kNumVariants = sizeof(kVariants) / sizeof(kVariants[0]);
 
 template <int BM, int BN, int WM, int WN, int CBSZ, int BLGP>
@@ -302,8 +258,16 @@ extern "C" int mi8_gemm_fp8(const void* a, int a_dtype, int64_t lda, const void*
                 out_dtype);
     GemmArgs g{(const uint8_t*)a, (const uint8_t*)b, out, out_dtype == MI8_F32 ? 1 : 0, lda, ldb, ldc, (int)M, (int)N, (int)K,
                sa, sb, sa_is_vector ? 1 : 0, sb_is_vector ? 1 : 0, 0, 0};
-    if (variant < 0) variant = 0;
     hipStream_t st = (hipStream_t)stream;
+    const bool pipe_ok = (K % BK == 0) && M >= 256 && N >= 256 && N % 8 == 0 && ldc % 8 == 0 && aligned16(out);
+    if (variant < 0) variant = pipe_ok ? kPipelined : 1;
+    if (variant == kPipelined) {
+        MI8_REQUIRE(pipe_ok, MI8_ERR_UNSUPPORTED,
+                    "mi8_gemm_fp8: the pipelined variant needs M, N >= 256, K %% 128 == 0, N %% 8 == 0, ldc %% 8 == 0 "
+                    "and a 16-byte aligned output (M=%lld N=%lld K=%lld ldc=%lld)",
+                    (long long)M, (long long)N, (long long)K, (long long)ldc);
+        return launch_pipelined(g, a_dtype, b_dtype, st);
+    }
     if (a_dtype == MI8_E4M3)
         return b_dtype == MI8_E4M3 ? launch_variant<0, 0>(variant, g, st) : launch_variant<0, 1>(variant, g, st);
     return b_dtype == MI8_E4M3 ? launch_variant<1, 0>(variant, g, st) : launch_variant<1, 1>(variant, g, st);
