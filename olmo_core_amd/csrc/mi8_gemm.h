@@ -60,9 +60,11 @@ __device__ __forceinline__ bool tile_of_block(const GemmArgs& g, int& tm, int& t
     return true;
 }
 
-// pipelined persistent kernel (mi8_gemm_pipe.hip); requires M, N >= 256, K % 128 == 0, N % 8 == 0, ldc % 8 == 0
-// and a 16-byte aligned output
-int launch_pipelined(GemmArgs& g, int a_dtype, int b_dtype, hipStream_t st);
+// persistent direct-to-LDS kernel (mi8_gemm_dma.hip); requires M, N >= 256, K % 64 == 0, N % 8 == 0, ldc % 8 == 0,
+// a 16-byte aligned bf16 output
+int launch_dma(GemmArgs& g, int a_dtype, int b_dtype, hipStream_t st);
+// same, 8 waves per workgroup and full 128-byte rows; additionally K % 128 == 0 (mi8_gemm_dma8.hip)
+int launch_dma8(GemmArgs& g, int a_dtype, int b_dtype, hipStream_t st);
 
 }  // namespace gemm
 }  // namespace mi8

@@ -181,9 +181,10 @@ constexpr Variant kVariants[] = {
     {"128x128_w2x2", 128, 128, 256},
     {"256x128_w2x2", 256, 128, 256},
     {"128x256_w2x2", 128, 256, 256},
-    {"256x256_pipelined_persistent", 256, 256, 256},
+    {"256x256_dma_w4_k64x4", 256, 256, 256},
+    {"256x256_dma_w8_k128x2", 256, 256, 512},
 };
-constexpr int kPipelined = 5;
+constexpr int kDma = 5, kDma8 = 6;
 constexpr int kNumVariants = sizeof(kVariants) / sizeof(kVariants[0]);
 
 template <int BM, int BN, int WM, int WN, int CBSZ, int BLGP>
@@ -259,14 +260,16 @@ extern "C" int mi8_gemm_fp8(const void* a, int a_dtype, int64_t lda, const void*
     GemmArgs g{(const uint8_t*)a, (const uint8_t*)b, out, out_dtype == MI8_F32 ? 1 : 0, lda, ldb, ldc, (int)M, (int)N, (int)K,
                sa, sb, sa_is_vector ? 1 : 0, sb_is_vector ? 1 : 0, 0, 0};
     hipStream_t st = (hipStream_t)stream;
-    const bool pipe_ok = (K % BK == 0) && M >= 256 && N >= 256 && N % 8 == 0 && ldc % 8 == 0 && aligned16(out);
-    if (variant < 0) variant = pipe_ok ? kPipelined : 1;
-    if (variant == kPipelined) {
-        MI8_REQUIRE(pipe_ok, MI8_ERR_UNSUPPORTED,
-                    "mi8_gemm_fp8: the pipelined variant needs M, N >= 256, K %% 128 == 0, N %% 8 == 0, ldc %% 8 == 0 "
-                    "and a 16-byte aligned output (M=%lld N=%lld K=%lld ldc=%lld)",
+    const bool dma_ok = (K % 64 == 0) && M >= 256 && N >= 256 && N % 8 == 0 && ldc % 8 == 0 && aligned16(out) &&
+                        out_dtype == MI8_BF16;
+    if (variant < 0) variant = dma_ok ? (K % 128 == 0 ? kDma8 : kDma) : 1;
+    if (variant == kDma8 && dma_ok && K % 128 == 0) return launch_dma8(g, a_dtype, b_dtype, st);
+    if (variant == kDma || variant == kDma8) {
+        MI8_REQUIRE(dma_ok && variant == kDma, MI8_ERR_UNSUPPORTED,
+                    "mi8_gemm_fp8: the direct-to-LDS variant needs M, N >= 256, K %% 64 == 0 (8 waves: 128), N %% 8 == 0, ldc %% 8 == 0 "
+                    "and a 16-byte aligned bf16 output (M=%lld N=%lld K=%lld ldc=%lld)",
                     (long long)M, (long long)N, (long long)K, (long long)ldc);
-        return launch_pipelined(g, a_dtype, b_dtype, st);
+        return launch_dma(g, a_dtype, b_dtype, st);
     }
     if (a_dtype == MI8_E4M3)
         return b_dtype == MI8_E4M3 ? launch_variant<0, 0>(variant, g, st) : launch_variant<0, 1>(variant, g, st);

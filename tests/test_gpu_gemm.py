@@ -23,7 +23,7 @@ def _gemm(a, sa, b, sb, variant, **kw):
     try:
         return ops.gemm_fp8(a, sa, b, sb, variant=variant, **kw)
     except MI8KernelError as e:
-        if "pipelined variant needs" in str(e):
+        if "direct-to-LDS variant needs" in str(e):
             return None
         raise
 
@@ -94,6 +94,8 @@ def test_against_emulated_mm(dev, mnk, gran):
         assert out.dtype == torch.bfloat16
         assert_gemm_close(out, ref, f"variant {v}")
         out32 = _gemm(a8.to(dev), sa_d, b8.to(dev), sb_d, v, out_dtype=torch.float32)
+        if out32 is None:  # this variant only writes bf16
+            continue
         assert_gemm_close(out32, ref, f"variant {v} f32")
         # bf16 output is the rounding of the fp32 output
         assert torch.equal(out32.bfloat16(), out)
