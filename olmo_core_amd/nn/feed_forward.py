@@ -2,7 +2,13 @@
 SwiGLU feed-forward block: the host of the float8 linears in the dense models
 (reference: src/olmo_core/nn/feed_forward.py:142-171, ``w2(silu(w1(x)) * w3(x))``; flops convention
 :206-209).  The three projections are ordinary ``nn.Linear`` modules so that
-``Float8Config.apply_float8_linear`` swaps them; the gate runs in one HIP kernel per direction.
+``Float8Config.apply_float8_linear`` swaps them.
+
+When all three are tensorwise ``Float8Linear`` modules without bias the block runs as one autograd function
+that performs exactly the casts and GEMMs the three modules would perform one by one (same bytes, same scales,
+same outputs), but quantises ``x`` once for ``w1`` and ``w3``, takes the amax of ``h`` and of the two gate
+gradients inside the SwiGLU kernels that produce them (no separate pass over the largest tensors), and saves
+fp8 copies instead of the bf16 activations ``x`` and ``h``.
 """
 
 from __future__ import annotations
@@ -11,6 +17,7 @@ import torch
 import torch.nn as nn
 
 from ..float8 import ops
+from ..float8.linear import Float8Linear, _is_tensorwise, _shared_tensorwise
 
 __all__ = ["FeedForward", "swiglu"]
 
@@ -34,6 +41,92 @@ def swiglu(x1: torch.Tensor, x3: torch.Tensor) -> torch.Tensor:
     return _SwiGLU.apply(x1, x3)
 
 
+class _Float8SwiGLUMLP(torch.autograd.Function):
+    """y = (silu(x W1^T) * (x W3^T)) W2^T with tensorwise float8 GEMMs; x [M, D], W1/W3 [H, D], W2 [D, H]."""
+
+    @staticmethod
+    def forward(ctx, x, w1, w2, w3, config):
+        c = config
+        pow2 = c.round_scales_to_power_of_2
+        in_dt, w_dt, go_dt = (
+            c.cast_config_input.target_dtype,
+            c.cast_config_weight.target_dtype,
+            c.cast_config_grad_output.target_dtype,
+        )
+        need = ctx.needs_input_grad
+        any_grad = any(need[:4])
+        xq, xq_t, sx = ops.cast_tensorwise(x, in_dt, pow2=pow2, want_transposed=need[1] or need[3])
+        w1q, w1q_t, s1 = ops.cast_tensorwise(w1, w_dt, pow2=pow2, want_transposed=need[0])
+        w3q, w3q_t, s3 = ops.cast_tensorwise(w3, w_dt, pow2=pow2, want_transposed=need[0])
+        w2q, w2q_t, s2 = ops.cast_tensorwise(w2, w_dt, pow2=pow2, want_transposed=any_grad)
+        x1 = ops.gemm_fp8(xq, sx, w1q, s1, out_dtype=x.dtype)
+        x3 = ops.gemm_fp8(xq, sx, w3q, s3, out_dtype=x.dtype)
+        h, h_slots = ops.swiglu_fwd(x1, x3, want_amax=True)
+        hq, hq_t, sh = ops.cast_tensorwise(h, in_dt, pow2=pow2, want_transposed=need[2], slots=h_slots)
+        y = ops.gemm_fp8(hq, sh, w2q, s2, out_dtype=x.dtype)
+        ctx.config = c
+        ctx.dtypes = (x.dtype, w1.dtype, w2.dtype, w3.dtype, go_dt)
+        ctx.dims = (x.shape[0], x.shape[1], w1.shape[0])
+        none = x.new_empty(0)
+        ctx.save_for_backward(
+            xq_t if xq_t is not None else none, sx, x1, x3, hq_t if hq_t is not None else none, sh,
+            w1q_t if w1q_t is not None else none, s1, w2q_t if w2q_t is not None else none, s2,
+            w3q_t if w3q_t is not None else none, s3,
+        )
+        return y
+
+    @staticmethod
+    def backward(ctx, gy):
+        xq_t, sx, x1, x3, hq_t, sh, w1q_t, s1, w2q_t, s2, w3q_t, s3 = ctx.saved_tensors
+        c = ctx.config
+        pow2 = c.round_scales_to_power_of_2
+        x_dt, w1_dt, w2_dt, w3_dt, go_dt = ctx.dtypes
+        M, D, H = ctx.dims
+        need_x, need_w1, need_w2, need_w3 = ctx.needs_input_grad[:4]
+        gy = gy.reshape(M, D)
+        if gy.dtype != x_dt:
+            gy = gy.to(x_dt)
+        need_gh = need_x or need_w1 or need_w3
+        gyq, gyq_t, sgy = ops.cast_tensorwise(gy, go_dt, pow2=pow2, want_rowmajor=need_gh, want_transposed=need_w2)
+        gw2 = ops.gemm_fp8(gyq_t, sgy, hq_t, sh, out_dtype=x_dt) if need_w2 else None
+        gx = gw1 = gw3 = None
+        if need_gh:
+            gh = ops.gemm_fp8(gyq, sgy, w2q_t, s2, k=D, out_dtype=x_dt)
+            g1, g3, slots1, slots3 = ops.swiglu_bwd(x1, x3, gh, want_amax=True)
+            del gh
+            need_t = need_w1 or need_w3
+            g1q, g1q_t, sg1 = ops.cast_tensorwise(g1, go_dt, pow2=pow2, want_rowmajor=need_x, want_transposed=need_t, slots=slots1)
+            g3q, g3q_t, sg3 = ops.cast_tensorwise(g3, go_dt, pow2=pow2, want_rowmajor=need_x, want_transposed=need_t, slots=slots3)
+            del g1, g3
+            if need_x:
+                gx = ops.gemm_fp8(g1q, sg1, w1q_t, s1, k=H, out_dtype=x_dt)
+                gx = gx + ops.gemm_fp8(g3q, sg3, w3q_t, s3, k=H, out_dtype=x_dt)
+            if need_w1:
+                gw1 = ops.gemm_fp8(g1q_t, sg1, xq_t, sx, out_dtype=x_dt)
+            if need_w3:
+                gw3 = ops.gemm_fp8(g3q_t, sg3, xq_t, sx, out_dtype=x_dt)
+
+        def as_param(g, dt):
+            return g if g is None or g.dtype == dt else g.to(dt)
+
+        return gx, as_param(gw1, w1_dt), as_param(gw2, w2_dt), as_param(gw3, w3_dt), None
+
+
+def _fusable(ff: "FeedForward", x: torch.Tensor) -> bool:
+    mods = (ff.w1, ff.w2, ff.w3)
+    if not all(isinstance(m, Float8Linear) and m.bias is None for m in mods):
+        return False
+    c = ff.w1.config
+    if ff.w2.config is not c and ff.w2.config != c or ff.w3.config is not c and ff.w3.config != c:
+        return False
+    same = (
+        _shared_tensorwise(c.cast_config_input, c.cast_config_input_for_grad_weight)
+        and _shared_tensorwise(c.cast_config_weight, c.cast_config_weight_for_grad_input)
+        and _shared_tensorwise(c.cast_config_grad_output, c.cast_config_grad_output_for_grad_weight)
+    )
+    return same and x.is_cuda and x.dtype == torch.bfloat16 and not torch.is_autocast_enabled()
+
+
 class FeedForward(nn.Module):
     """Gated feed-forward with SiLU activation: ``w2(silu(w1 x) * w3 x)``."""
 
@@ -45,15 +138,21 @@ class FeedForward(nn.Module):
         bias: bool = True,
         dtype: torch.dtype = torch.float32,
         init_device: str = "cpu",
+        fuse_float8: bool = True,
     ):
         super().__init__()
         self.d_model = d_model
         self.hidden_size = hidden_size
+        self.fuse_float8 = fuse_float8
         self.w1 = nn.Linear(d_model, hidden_size, bias=bias, dtype=dtype, device=init_device)
         self.w2 = nn.Linear(hidden_size, d_model, bias=bias, dtype=dtype, device=init_device)
         self.w3 = nn.Linear(d_model, hidden_size, bias=bias, dtype=dtype, device=init_device)
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
+        if self.fuse_float8 and _fusable(self, x):
+            x2 = x.reshape(-1, x.shape[-1])
+            y = _Float8SwiGLUMLP.apply(x2, self.w1.weight, self.w2.weight, self.w3.weight, self.w1.config)
+            return y.reshape(*x.shape[:-1], self.w2.weight.shape[0])
         x1, x3 = self.w1(x), self.w3(x)
         if x1.is_cuda and x1.dtype == torch.bfloat16:
             h = swiglu(x1, x3)
