@@ -121,6 +121,43 @@ int mi8_gemm_num_variants(void);
 const char* mi8_gemm_variant_name(int variant);
 
 /* ---------------------------------------------------------------------------------------------
+ * Ragged grouped operations for the dropless-MoE expert layer.  The reference runs this layer in bf16 through
+ * grouped_gemm.ops.gmm(x, w, batch_sizes, trans_b) or a per-expert loop (src/olmo_core/nn/moe/mlp.py:256-270);
+ * these entry points are its float8 counterpart with the axiswise recipe applied to every expert's slice
+ * independently.  Rows of the activation matrix form consecutive groups; group_sizes is an int64 device array
+ * (as DroplessMoEMLP.forward receives it, mlp.py:272-280) that is never copied to the host.
+ * ------------------------------------------------------------------------------------------- */
+
+/* Upper bound of the padded token axis used by the grouped transposed layouts: every group's segment starts at a
+ * multiple of 128. */
+int64_t mi8_grouped_padded_rows(int64_t T, int32_t num_groups);
+
+/* Per-group, per-column dynamic cast with transposed output: for group e (rows R_e of x[T, cols]) the scale of
+ * column c is taken over R_e only; out_t[c, 128 * tiles_before(e) + (r - first row of e)] holds the bytes, the
+ * rest of each 128-aligned segment is zero.  amax_ws: uint32 [num_groups * cols], ZERO on entry.
+ * scale_out: float32 [num_groups, cols] (rows of empty groups are not written).
+ * ld_t >= mi8_grouped_padded_rows(T, num_groups), ld_t % 16 == 0.  With equal group sizes that are multiples of
+ * 128 this is a batched transpose-cast (used for the expert weights). */
+int mi8_grouped_cast_colwise_t(const void* x, int hp_dtype, int64_t T, int64_t cols, const int64_t* group_sizes,
+                               int32_t num_groups, int fp8_dtype, uint32_t flags, uint32_t* amax_ws, void* out_t,
+                               int64_t ld_t, float* scale_out, void* stream);
+
+/* out[R_e, :N] = (A[R_e, :K] . B_e[:N, :K]^T) / sa[r] / sb_e[n]   for every group e.
+ *   A fp8 [T, lda]; B_e = b + e * b_group_stride (bytes), N rows of pitch ldb; sa float32 [T];
+ *   sb_e = sb + e * sb_group_stride (floats), N values; out [T, ldc] of out_dtype. */
+int mi8_grouped_gemm_fp8(const void* a, int a_dtype, int64_t lda, const void* b, int b_dtype, int64_t ldb,
+                         int64_t b_group_stride, const int64_t* group_sizes, int32_t num_groups, int64_t T, int64_t N,
+                         int64_t K, const float* sa, const float* sb, int64_t sb_group_stride, void* out,
+                         int out_dtype, int64_t ldc, void* stream);
+
+/* out[e, :N, :Kl] = (A_t[:N, S_e] . B_t[:Kl, S_e]^T) / sa[e, n] / sb[e, k]: the contraction runs over group e's
+ * 128-aligned segment S_e of the padded token axis (layout written by mi8_grouped_cast_colwise_t; both operands
+ * have pitch ld_t).  Empty groups produce zeros.  out is [num_groups, N, Kl] contiguous. */
+int mi8_grouped_wgrad_fp8(const void* a_t, int a_dtype, const void* b_t, int b_dtype, int64_t ld_t,
+                          const int64_t* group_sizes, int32_t num_groups, int64_t T, int64_t N, int64_t Kl,
+                          const float* sa, const float* sb, void* out, int out_dtype, void* stream);
+
+/* ---------------------------------------------------------------------------------------------
  * SwiGLU pointwise kernels between the projections of the feed-forward block
  * (reference: src/olmo_core/nn/feed_forward.py:171  w2(silu(w1 x) * w3 x)).
  *   forward : h = bf16(bf16(silu(x1)) * x3), optionally also the amax partials of h.

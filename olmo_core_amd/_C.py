@@ -52,6 +52,22 @@ _SIGNATURES = {
         c_int,
         [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_void_p, c_void_p, c_void_p],
     ),
+    "mi8_grouped_padded_rows": (c_int64, [c_int64, c_int32]),
+    "mi8_grouped_cast_colwise_t": (
+        c_int,
+        [c_void_p, c_int, c_int64, c_int64, c_void_p, c_int32, c_int, c_uint32, c_void_p, c_void_p, c_int64, c_void_p,
+         c_void_p],
+    ),
+    "mi8_grouped_gemm_fp8": (
+        c_int,
+        [c_void_p, c_int, c_int64, c_void_p, c_int, c_int64, c_int64, c_void_p, c_int32, c_int64, c_int64, c_int64,
+         c_void_p, c_void_p, c_int64, c_void_p, c_int, c_int64, c_void_p],
+    ),
+    "mi8_grouped_wgrad_fp8": (
+        c_int,
+        [c_void_p, c_int, c_void_p, c_int, c_int64, c_void_p, c_int32, c_int64, c_int64, c_int64, c_void_p, c_void_p,
+         c_void_p, c_int, c_void_p],
+    ),
 }
 
 EXPORTED_SYMBOLS = tuple(_SIGNATURES)

@@ -138,6 +138,72 @@ __device__ __forceinline__ int tile_lds_chunk(int col, int part /* 0..7: which 1
     return (col >> 1) * 16 + ((((col & 1) << 3) | part) ^ key);
 }
 
+// Quantise one 128 x 128 tile with the eight per-column scales of this lane (all equal for a tensorwise cast):
+// rows [row0, row0 + 128) of x (rows >= row_end read as zero and produce zero bytes), columns [col0, col0 + 128).
+// Row-major bytes go to out[r, c]; the transposed bytes go to out_t[c, dst0 + (r - row0)] as 16-byte chunks,
+// chunks at or beyond dst_end are not written.
+template <int HP, int FP8, bool SW>
+__device__ __forceinline__ void tile_cast_body(const void* x, int64_t row_end, int64_t cols, int64_t row0, int64_t col0,
+                                               const float (&sc)[8], uint8_t* out, uint8_t* out_t, int64_t ld_t,
+                                               int64_t dst0, int64_t dst_end, uint32_t* lds_t)
+{
+    const int tid = threadIdx.x;
+    const int wave = tid >> 6, lane = tid & 63;
+    const int cl = lane & 15, g = lane >> 4;
+    const int64_t c8 = col0 + 8 * cl;
+    const bool col_ok = c8 < cols;
+    const char* xb = reinterpret_cast<const char*>(x);
+
+    float f[2][4][8];
+#pragma unroll
+    for (int it = 0; it < 2; ++it)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int64_t r = row0 + 32 * wave + 16 * it + 4 * g + j;
+            const bool ok = col_ok && r < row_end;
+            HpVec<HP>::load8(xb + (r * cols + c8) * HpVec<HP>::kBytes, ok, f[it][j]);
+        }
+
+#pragma unroll
+    for (int it = 0; it < 2; ++it) {
+        uint32_t lo[4], hi[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int64_t r = row0 + 32 * wave + 16 * it + 4 * g + j;
+            const bool ok = col_ok && r < row_end;
+            const float* v = f[it][j];
+            lo[j] = quant4<FP8, SW>(v[0], v[1], v[2], v[3], sc[0], sc[1], sc[2], sc[3]);
+            hi[j] = quant4<FP8, SW>(v[4], v[5], v[6], v[7], sc[4], sc[5], sc[6], sc[7]);
+            if (!ok) lo[j] = hi[j] = 0;  // padding is zero bytes whatever the scale is (0 * NaN is NaN)
+            if (out && ok) *reinterpret_cast<uint2*>(out + r * cols + c8) = make_uint2(lo[j], hi[j]);
+        }
+        if (out_t) {
+            uint32_t t[8];
+            transpose4x4_bytes(lo[0], lo[1], lo[2], lo[3], t[0], t[1], t[2], t[3]);
+            transpose4x4_bytes(hi[0], hi[1], hi[2], hi[3], t[4], t[5], t[6], t[7]);
+            const int rd = 8 * wave + 4 * it + g;  // which dword of the column's 32 row-dwords
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const int col = 8 * cl + i;
+                lds_t[tile_lds_chunk(col, rd >> 2) * 4 + (rd & 3)] = t[i];
+            }
+        }
+    }
+
+    if (out_t) {
+        __syncthreads();
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int q = tid + kThreads * i;
+            const int col = q >> 3, part = q & 7;
+            const uint4 v = reinterpret_cast<const uint4*>(lds_t)[tile_lds_chunk(col, part)];
+            const int64_t c = col0 + col;
+            const int64_t d = dst0 + 16 * part;
+            if (c < cols && d < dst_end) *reinterpret_cast<uint4*>(out_t + c * ld_t + d) = v;
+        }
+    }
+}
+
 template <int HP, int FP8, bool SW, int MODE>
 __global__ __launch_bounds__(kThreads) void tile_cast_kernel(TileCastArgs a)
 {
@@ -184,59 +250,7 @@ __global__ __launch_bounds__(kThreads) void tile_cast_kernel(TileCastArgs a)
         for (int i = 0; i < 8; ++i) sc[i] = s;
     }
 
-    // ---- load, quantise, write row-major, stage transposed ----------------------------------
-    const int64_t c8 = col0 + 8 * cl;
-    const bool col_ok = c8 < a.cols;
-    const char* xb = reinterpret_cast<const char*>(a.x);
-
-    float f[2][4][8];
-#pragma unroll
-    for (int it = 0; it < 2; ++it)
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            const int64_t r = row0 + 32 * wave + 16 * it + 4 * g + j;
-            const bool ok = col_ok && r < a.rows;
-            HpVec<HP>::load8(xb + (r * a.cols + c8) * HpVec<HP>::kBytes, ok, f[it][j]);
-        }
-
-#pragma unroll
-    for (int it = 0; it < 2; ++it) {
-        uint32_t lo[4], hi[4];
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            const int64_t r = row0 + 32 * wave + 16 * it + 4 * g + j;
-            const bool ok = col_ok && r < a.rows;
-            const float* v = f[it][j];
-            lo[j] = quant4<FP8, SW>(v[0], v[1], v[2], v[3], sc[0], sc[1], sc[2], sc[3]);
-            hi[j] = quant4<FP8, SW>(v[4], v[5], v[6], v[7], sc[4], sc[5], sc[6], sc[7]);
-            if (!ok) lo[j] = hi[j] = 0;  // padding is zero bytes whatever the scale is (0 * NaN is NaN)
-            if (a.out && ok) *reinterpret_cast<uint2*>(a.out + r * a.cols + c8) = make_uint2(lo[j], hi[j]);
-        }
-        if (a.out_t) {
-            uint32_t t[8];
-            transpose4x4_bytes(lo[0], lo[1], lo[2], lo[3], t[0], t[1], t[2], t[3]);
-            transpose4x4_bytes(hi[0], hi[1], hi[2], hi[3], t[4], t[5], t[6], t[7]);
-            const int rd = 8 * wave + 4 * it + g;  // which dword of the column's 32 row-dwords
-#pragma unroll
-            for (int i = 0; i < 8; ++i) {
-                const int col = 8 * cl + i;
-                lds_t[tile_lds_chunk(col, rd >> 2) * 4 + (rd & 3)] = t[i];
-            }
-        }
-    }
-
-    if (a.out_t) {
-        __syncthreads();
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const int q = tid + kThreads * i;
-            const int col = q >> 3, part = q & 7;
-            const uint4 v = reinterpret_cast<const uint4*>(lds_t)[tile_lds_chunk(col, part)];
-            const int64_t c = col0 + col;
-            const int64_t r = row0 + 16 * part;
-            if (c < a.cols && r < a.ld_t) *reinterpret_cast<uint4*>(a.out_t + c * a.ld_t + r) = v;
-        }
-    }
+    tile_cast_body<HP, FP8, SW>(a.x, a.rows, a.cols, row0, col0, sc, a.out, a.out_t, a.ld_t, row0, a.ld_t, lds_t);
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -353,6 +367,127 @@ __global__ __launch_bounds__(kThreads) void rowwise_cast_kernel(const void* __re
             *reinterpret_cast<uint2*>(orow + (int64_t)v * 8) = make_uint2(lo, hi);
         }
     }
+}
+
+// ------------------------------------------------------------------------------------------------
+// grouped per-column cast: rows of x are split into consecutive groups (dropless-MoE experts); every
+// group gets its own per-column scales and its transposed bytes start at a multiple of 128 in out_t
+// ------------------------------------------------------------------------------------------------
+
+struct GroupedCastArgs {
+    const void* x;
+    int64_t T, cols;
+    const int64_t* sizes;
+    int E;
+    bool pow2;
+    uint32_t* amax;  // [E, cols], zero on entry
+    uint8_t* out_t;  // [cols, ld_t]
+    int64_t ld_t;
+    float* scale_out;  // [E, cols]
+};
+
+// Tile p of the padded row space (128 rows each; group e owns ceil(m_e / 128) consecutive tiles) -> its group,
+// its rows [row0, row_end) in x (row_end = the group's end) and its destination column 128 p in out_t.
+// Sizes are clamped so that nothing past row T is ever read.
+__device__ __forceinline__ bool locate_padded_tile(const int64_t* sizes, int E, int64_t T, int p, int& e,
+                                                   int64_t& row0, int64_t& row_end)
+{
+    int64_t rows_before = 0;
+    int tiles_before = 0;
+    for (e = 0; e < E; ++e) {
+        int64_t m = sizes[e];
+        m = m < 0 ? 0 : m;
+        m = (rows_before + m > T) ? T - rows_before : m;
+        const int t = (int)((m + kTile - 1) / kTile);
+        if (p < tiles_before + t) {
+            row0 = rows_before + (int64_t)kTile * (p - tiles_before);
+            row_end = rows_before + m;
+            return true;
+        }
+        tiles_before += t;
+        rows_before += m;
+    }
+    return false;
+}
+
+template <int HP>
+__global__ __launch_bounds__(kThreads) void grouped_colamax_kernel(GroupedCastArgs a)
+{
+    __shared__ uint32_t red[16][kTile + 1];
+    int e;
+    int64_t row0, row_end;
+    if (!locate_padded_tile(a.sizes, a.E, a.T, (int)blockIdx.y, e, row0, row_end)) return;
+    const int tid = threadIdx.x;
+    const int cl = tid & 15, rg = tid >> 4;
+    const int64_t col0 = (int64_t)blockIdx.x * kTile;
+    const int64_t c8 = col0 + 8 * cl;
+    const char* xb = reinterpret_cast<const char*>(a.x);
+    constexpr int NV = HpVec<HP>::kBytes == 2 ? 1 : 2;
+    uint32_t acc[NV][4];
+#pragma unroll
+    for (int v = 0; v < NV; ++v)
+#pragma unroll
+        for (int k = 0; k < 4; ++k) acc[v][k] = 0;
+    if (c8 < a.cols) {
+#pragma unroll
+        for (int i = 0; i < kTile / 16; ++i) {
+            const int64_t r = row0 + rg + 16 * i;
+            if (r < row_end) {
+#pragma unroll
+                for (int k = 0; k < NV; ++k)
+                    absmax_accumulate<HP>(
+                        reinterpret_cast<const uint4*>(xb + (r * a.cols + c8) * HpVec<HP>::kBytes)[k], acc[k]);
+            }
+        }
+    }
+    if constexpr (HP == MI8_BF16) {
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            red[rg][8 * cl + 2 * k] = (acc[0][k] & 0xFFFFu) << 16;
+            red[rg][8 * cl + 2 * k + 1] = acc[0][k] & 0xFFFF0000u;
+        }
+    } else {
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            red[rg][8 * cl + k] = acc[0][k];
+            red[rg][8 * cl + 4 + k] = acc[NV - 1][k];
+        }
+    }
+    __syncthreads();
+    if (tid < kTile && col0 + tid < a.cols) {
+        uint32_t m = 0;
+#pragma unroll
+        for (int k = 0; k < 16; ++k) m = umax32(m, red[k][tid]);
+        atomicMax(&a.amax[(int64_t)e * a.cols + col0 + tid], m);  // integer max: order-independent, deterministic
+    }
+}
+
+template <int HP, int FP8, bool SW>
+__global__ __launch_bounds__(kThreads) void grouped_tile_cast_kernel(GroupedCastArgs a)
+{
+    __shared__ __attribute__((aligned(16))) uint32_t lds_t[kTile * kTile / 4];
+    __shared__ float s_scale[kTile];
+    int e;
+    int64_t row0, row_end;
+    if (!locate_padded_tile(a.sizes, a.E, a.T, (int)blockIdx.y, e, row0, row_end)) return;
+    const int tid = threadIdx.x;
+    const int cl = tid & 15;
+    const int64_t col0 = (int64_t)blockIdx.x * kTile;
+    if (tid < kTile) {
+        const int64_t c = col0 + tid;
+        float s = 0.0f;
+        if (c < a.cols) {
+            s = scale_from_amax_bits<FP8>(a.amax[(int64_t)e * a.cols + c], a.pow2);
+            a.scale_out[(int64_t)e * a.cols + c] = s;  // every tile of the group writes the same value
+        }
+        s_scale[tid] = s;
+    }
+    __syncthreads();
+    float sc[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) sc[i] = s_scale[8 * cl + i];
+    const int64_t dst0 = (int64_t)kTile * blockIdx.y;
+    tile_cast_body<HP, FP8, SW>(a.x, row_end, a.cols, row0, col0, sc, nullptr, a.out_t, a.ld_t, dst0, a.ld_t, lds_t);
 }
 
 // ---- dispatch helpers ------------------------------------------------------------------------------
@@ -562,4 +697,53 @@ extern "C" int mi8_cast_colwise_t(const void* x, int hp_dtype, int64_t rows, int
                    nullptr, (uint8_t*)out_t, ld_t, scale_out};
     dispatch_tile_cast(hp_dtype, fp8_dtype, (flags & MI8_FLAG_SW_CVT) != 0, kPerColumnFromWorkspace, a, st);
     return launch_status("mi8_cast_colwise_t(cast)");
+}
+
+extern "C" int64_t mi8_grouped_padded_rows(int64_t T, int32_t num_groups)
+{
+    if (T < 0 || num_groups < 0) return 0;
+    return round_up(T, kTile) + (int64_t)kTile * num_groups;
+}
+
+extern "C" int mi8_grouped_cast_colwise_t(const void* x, int hp_dtype, int64_t T, int64_t cols,
+                                          const int64_t* group_sizes, int32_t num_groups, int fp8_dtype,
+                                          uint32_t flags, uint32_t* amax_ws, void* out_t, int64_t ld_t,
+                                          float* scale_out, void* stream)
+{
+    MI8_REQUIRE(x && group_sizes && amax_ws && out_t && scale_out, MI8_ERR_ARG, "mi8_grouped_cast_colwise_t: null pointer");
+    MI8_REQUIRE(valid_hp(hp_dtype) && valid_fp8(fp8_dtype), MI8_ERR_ARG, "mi8_grouped_cast_colwise_t: unknown dtype");
+    MI8_REQUIRE(T > 0 && cols > 0 && num_groups > 0, MI8_ERR_ARG, "mi8_grouped_cast_colwise_t: empty input");
+    MI8_REQUIRE(cols % 16 == 0, MI8_ERR_UNSUPPORTED, "mi8_grouped_cast_colwise_t: cols (%lld) must be a multiple of 16",
+                (long long)cols);
+    MI8_REQUIRE(ld_t % 16 == 0 && ld_t >= mi8_grouped_padded_rows(T, num_groups), MI8_ERR_UNSUPPORTED,
+                "mi8_grouped_cast_colwise_t: ld_t (%lld) must be a multiple of 16 and at least mi8_grouped_padded_rows() = %lld",
+                (long long)ld_t, (long long)mi8_grouped_padded_rows(T, num_groups));
+    MI8_REQUIRE(aligned16(x) && aligned16(out_t), MI8_ERR_UNSUPPORTED,
+                "mi8_grouped_cast_colwise_t: pointers must be 16-byte aligned");
+    const int64_t ptiles = ceil_div(T, kTile) + num_groups;
+    MI8_REQUIRE(ptiles <= 65535, MI8_ERR_UNSUPPORTED, "mi8_grouped_cast_colwise_t: too many row tiles (%lld)",
+                (long long)ptiles);
+    GroupedCastArgs a{x, T, cols, group_sizes, num_groups, (flags & MI8_FLAG_POW2_SCALE) != 0,
+                      amax_ws, (uint8_t*)out_t, ld_t, scale_out};
+    hipStream_t st = (hipStream_t)stream;
+    dim3 grid((unsigned)ceil_div(cols, kTile), (unsigned)ptiles);
+    if (hp_dtype == MI8_BF16)
+        hipLaunchKernelGGL((grouped_colamax_kernel<MI8_BF16>), grid, dim3(kThreads), 0, st, a);
+    else
+        hipLaunchKernelGGL((grouped_colamax_kernel<MI8_F32>), grid, dim3(kThreads), 0, st, a);
+    int rc = launch_status("mi8_grouped_cast_colwise_t(amax)");
+    if (rc != MI8_OK) return rc;
+    const bool sw = flags & MI8_FLAG_SW_CVT;
+#define MI8_GC(HP_, FP8_)                                                                                   \
+    if (sw)                                                                                                 \
+        hipLaunchKernelGGL((grouped_tile_cast_kernel<HP_, FP8_, true>), grid, dim3(kThreads), 0, st, a);    \
+    else                                                                                                    \
+        hipLaunchKernelGGL((grouped_tile_cast_kernel<HP_, FP8_, false>), grid, dim3(kThreads), 0, st, a)
+    if (hp_dtype == MI8_BF16) {
+        if (fp8_dtype == MI8_E4M3) { MI8_GC(MI8_BF16, MI8_E4M3); } else { MI8_GC(MI8_BF16, MI8_E5M2); }
+    } else {
+        if (fp8_dtype == MI8_E4M3) { MI8_GC(MI8_F32, MI8_E4M3); } else { MI8_GC(MI8_F32, MI8_E5M2); }
+    }
+#undef MI8_GC
+    return launch_status("mi8_grouped_cast_colwise_t(cast)");
 }

@@ -247,3 +247,105 @@ def swiglu_bwd(x1: torch.Tensor, x3: torch.Tensor, gh: torch.Tensor, want_amax: 
     )
     used = _C.lib().mi8_amax_slots_for(n)
     return g1, g3, ((s1, used) if want_amax else None), ((s3, used) if want_amax else None)
+
+
+# ---- ragged grouped operations (dropless-MoE expert layer) -------------------------------------------
+
+
+def grouped_padded_rows(T: int, num_groups: int) -> int:
+    return _C.lib().mi8_grouped_padded_rows(T, num_groups)
+
+
+def _sizes_i64(group_sizes: torch.Tensor, dev) -> torch.Tensor:
+    if group_sizes.dim() != 1:
+        raise ValueError("group sizes must be a 1-D tensor")
+    if group_sizes.device != dev or group_sizes.dtype != torch.int64 or not group_sizes.is_contiguous():
+        group_sizes = group_sizes.to(device=dev, dtype=torch.int64).contiguous()
+    return group_sizes
+
+
+def grouped_cast_colwise_t(
+    x: torch.Tensor, group_sizes: torch.Tensor, fp8_dtype: torch.dtype, *, pow2: bool = False
+) -> Tuple[torch.Tensor, torch.Tensor]:
+    """
+    Per-group, per-column cast with transposed output.  ``x [T, cols]``, rows grouped consecutively by
+    ``group_sizes [E]`` (int64, on the device).  Returns ``(q_t [cols, ld_t], scale [E, cols])`` where group e's
+    bytes start at column ``128 * (number of 128-row tiles of the groups before it)`` and the padding is zero.
+    """
+    x = _hp2d(x, "grouped_cast_colwise_t")
+    T, cols = x.shape
+    sizes = _sizes_i64(group_sizes, x.device)
+    E = sizes.numel()
+    ld_t = grouped_padded_rows(T, E)
+    q_t = torch.empty((cols, ld_t), dtype=fp8_dtype, device=x.device)
+    scale = torch.empty((E, cols), dtype=torch.float32, device=x.device)
+    ws = torch.zeros(E * cols, dtype=torch.int32, device=x.device)
+    _C.check(
+        _C.lib().mi8_grouped_cast_colwise_t(
+            x.data_ptr(), _HP_CODE[x.dtype], T, cols, sizes.data_ptr(), E, _FP8_CODE[fp8_dtype], _flags(pow2),
+            ws.data_ptr(), q_t.data_ptr(), ld_t, scale.data_ptr(), _stream(x),
+        ),
+        "mi8_grouped_cast_colwise_t",
+    )
+    return q_t, scale
+
+
+def grouped_gemm_fp8(
+    a: torch.Tensor,
+    sa: torch.Tensor,
+    b: torch.Tensor,
+    sb: torch.Tensor,
+    group_sizes: torch.Tensor,
+    *,
+    n: int,
+    k: int,
+    b_group_stride: int,
+    sb_group_stride: int,
+    out_dtype: torch.dtype = torch.bfloat16,
+) -> torch.Tensor:
+    """
+    ``out[rows of group e] = a[rows of group e, :k] @ B_e[:n, :k].T / sa / sb_e`` where ``B_e`` starts
+    ``e * b_group_stride`` bytes into ``b`` (row pitch ``b.stride(0)``) and its scales ``e * sb_group_stride``
+    floats into ``sb``.
+    """
+    _require_gpu(a, "grouped_gemm_fp8")
+    T = a.shape[0]
+    sizes = _sizes_i64(group_sizes, a.device)
+    out = torch.empty((T, n), dtype=out_dtype, device=a.device)
+    _C.check(
+        _C.lib().mi8_grouped_gemm_fp8(
+            a.data_ptr(), _FP8_CODE[a.dtype], a.stride(0), b.data_ptr(), _FP8_CODE[b.dtype], b.stride(0),
+            b_group_stride, sizes.data_ptr(), sizes.numel(), T, n, k, sa.data_ptr(), sb.data_ptr(), sb_group_stride,
+            out.data_ptr(), _HP_CODE[out_dtype], out.stride(0), _stream(a),
+        ),
+        "mi8_grouped_gemm_fp8",
+    )
+    return out
+
+
+def grouped_wgrad_fp8(
+    a_t: torch.Tensor,
+    sa: torch.Tensor,
+    b_t: torch.Tensor,
+    sb: torch.Tensor,
+    group_sizes: torch.Tensor,
+    *,
+    tokens: int,
+    out_dtype: torch.dtype = torch.bfloat16,
+) -> torch.Tensor:
+    """``out[e] = a_t[:, seg_e] @ b_t[:, seg_e].T / sa[e] / sb[e]`` -> ``[E, a_t.shape[0], b_t.shape[0]]``."""
+    _require_gpu(a_t, "grouped_wgrad_fp8")
+    sizes = _sizes_i64(group_sizes, a_t.device)
+    E, N, Kl = sizes.numel(), a_t.shape[0], b_t.shape[0]
+    if a_t.stride(0) != b_t.stride(0):
+        raise ValueError("grouped_wgrad_fp8: both operands must share the padded token pitch")
+    out = torch.empty((E, N, Kl), dtype=out_dtype, device=a_t.device)
+    _C.check(
+        _C.lib().mi8_grouped_wgrad_fp8(
+            a_t.data_ptr(), _FP8_CODE[a_t.dtype], b_t.data_ptr(), _FP8_CODE[b_t.dtype], a_t.stride(0),
+            sizes.data_ptr(), E, tokens, N, Kl, sa.data_ptr(), sb.data_ptr(), out.data_ptr(), _HP_CODE[out_dtype],
+            _stream(a_t),
+        ),
+        "mi8_grouped_wgrad_fp8",
+    )
+    return out

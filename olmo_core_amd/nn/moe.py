@@ -1,0 +1,139 @@
+"""
+Dropless-MoE expert MLP with float8 grouped GEMMs.
+
+Same parameters and call signature as the reference's ``DroplessMoEMLP`` (reference:
+src/olmo_core/nn/moe/mlp.py:198-292): ``w1, w2, w3`` of shape ``[num_experts * hidden_size, d_model]``,
+``forward(x [T, d_model], batch_size_per_expert [E])`` with the rows of ``x`` already permuted so that each
+expert's tokens are consecutive, ``w1``/``w3`` used transposed and ``w2`` as stored, ``h = silu(x1) * x2``.
+The reference runs the expert GEMMs in bf16 (its float8 conversion never touches these raw Parameters); here
+every expert's slice goes through the axiswise float8 recipe (per-row scales for activations, per-channel
+scales per expert for weights, per-group column scales for the weight gradients, e4m3 everywhere, power-of-two
+scales) on ragged grouped kernels.  Group sizes stay on the device: there is no host synchronisation.
+"""
+
+from __future__ import annotations
+
+import math
+
+import torch
+import torch.nn as nn
+
+from ..float8 import ops
+
+__all__ = ["DroplessMoEMLP", "float8_dropless_mlp"]
+
+_E4M3 = torch.float8_e4m3fn
+
+
+class _Float8DroplessMLP(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, x, w1, w2, w3, sizes, num_experts, pow2):
+        E = num_experts
+        T, D = x.shape
+        H = w1.shape[0] // E
+        dev = x.device
+        equal = torch.full((E,), H, dtype=torch.int64, device=dev)  # the experts' weights as equal-size groups
+
+        xq, sx = ops.cast_rowwise(x, _E4M3, pow2=pow2)
+        w1q, s1 = ops.cast_rowwise(w1, _E4M3, pow2=pow2)  # per output channel (row of w[e])
+        w3q, s3 = ops.cast_rowwise(w3, _E4M3, pow2=pow2)
+        x1 = ops.grouped_gemm_fp8(xq, sx, w1q, s1, sizes, n=H, k=D, b_group_stride=H * w1q.stride(0), sb_group_stride=H)
+        x2 = ops.grouped_gemm_fp8(xq, sx, w3q, s3, sizes, n=H, k=D, b_group_stride=H * w3q.stride(0), sb_group_stride=H)
+        h, _ = ops.swiglu_fwd(x1, x2, want_amax=False)
+        hq, sh = ops.cast_rowwise(h, _E4M3, pow2=pow2)
+        # w2[e] is [H, D] and is used as-is (h_e @ w2[e]): its output channel is the column -> transposed copy
+        # [D, E*H] with one scale per (expert, column)
+        w2t, s2 = ops.grouped_cast_colwise_t(w2, equal, _E4M3, pow2=pow2)
+        y = ops.grouped_gemm_fp8(hq, sh, w2t, s2, sizes, n=D, k=H, b_group_stride=H, sb_group_stride=D)
+        ctx.save_for_backward(x, w1, w2, w3, x1, x2, h, sizes, equal)
+        ctx.meta = (E, T, D, H, pow2)
+        return y
+
+    @staticmethod
+    def backward(ctx, gy):
+        x, w1, w2, w3, x1, x2, h, sizes, equal = ctx.saved_tensors
+        E, T, D, H, pow2 = ctx.meta
+        gy = gy.reshape(T, D).contiguous()
+        need_x, need_w1, need_w2, need_w3 = ctx.needs_input_grad[:4]
+
+        gyq, sgy = ops.cast_rowwise(gy, _E4M3, pow2=pow2)
+        # gh_e = gy_e @ w2[e]^T : contraction over D, the right operand is w2[e] itself with one scale per row
+        w2q, s2r = ops.cast_rowwise(w2, _E4M3, pow2=pow2)
+        gh = ops.grouped_gemm_fp8(gyq, sgy, w2q, s2r, sizes, n=H, k=D, b_group_stride=H * w2q.stride(0), sb_group_stride=H)
+        gw2 = None
+        if need_w2:
+            # gw2[e] [H, D] = h_e^T @ gy_e : contraction over the group's tokens
+            ht, shc = ops.grouped_cast_colwise_t(h, sizes, _E4M3, pow2=pow2)
+            gyt, sgyc = ops.grouped_cast_colwise_t(gy, sizes, _E4M3, pow2=pow2)
+            gw2 = ops.grouped_wgrad_fp8(ht, shc, gyt, sgyc, sizes, tokens=T, out_dtype=gy.dtype).reshape(E * H, D)
+        g1, g2, _, _ = ops.swiglu_bwd(x1, x2, gh, want_amax=False)
+        del gh
+        gx = gw1 = gw3 = None
+        if need_x:
+            # gx_e = g_e @ w[e] : contraction over H, the right operand is w[e]^T [D, H] with one scale per input channel
+            g1q, sg1 = ops.cast_rowwise(g1, _E4M3, pow2=pow2)
+            g2q, sg2 = ops.cast_rowwise(g2, _E4M3, pow2=pow2)
+            w1t, s1c = ops.grouped_cast_colwise_t(w1, equal, _E4M3, pow2=pow2)
+            w3t, s3c = ops.grouped_cast_colwise_t(w3, equal, _E4M3, pow2=pow2)
+            gx = ops.grouped_gemm_fp8(g1q, sg1, w1t, s1c, sizes, n=D, k=H, b_group_stride=H, sb_group_stride=D)
+            gx = gx + ops.grouped_gemm_fp8(g2q, sg2, w3t, s3c, sizes, n=D, k=H, b_group_stride=H, sb_group_stride=D)
+        if need_w1 or need_w3:
+            xt, sxc = ops.grouped_cast_colwise_t(x, sizes, _E4M3, pow2=pow2)
+            if need_w1:
+                g1t, sg1c = ops.grouped_cast_colwise_t(g1, sizes, _E4M3, pow2=pow2)
+                gw1 = ops.grouped_wgrad_fp8(g1t, sg1c, xt, sxc, sizes, tokens=T, out_dtype=gy.dtype).reshape(E * H, D)
+            if need_w3:
+                g2t, sg2c = ops.grouped_cast_colwise_t(g2, sizes, _E4M3, pow2=pow2)
+                gw3 = ops.grouped_wgrad_fp8(g2t, sg2c, xt, sxc, sizes, tokens=T, out_dtype=gy.dtype).reshape(E * H, D)
+
+        def as_param(g, ref):
+            return g if g is None or g.dtype == ref.dtype else g.to(ref.dtype)
+
+        return gx, as_param(gw1, w1), as_param(gw2, w2), as_param(gw3, w3), None, None, None
+
+
+def float8_dropless_mlp(x, w1, w2, w3, batch_size_per_expert, num_experts: int, pow2: bool = True):
+    """``gmm(silu(gmm(x, w1^T)) * gmm(x, w3^T), w2)`` with float8 grouped GEMMs; ``x`` is ``[T, d_model]`` bf16."""
+    return _Float8DroplessMLP.apply(x, w1, w2, w3, batch_size_per_expert, num_experts, pow2)
+
+
+class DroplessMoEMLP(nn.Module):
+    """A dropless expert MLP module with SwiGLU activation and float8 grouped GEMMs."""
+
+    def __init__(
+        self,
+        *,
+        d_model: int,
+        hidden_size: int,
+        num_experts: int,
+        dtype: torch.dtype = torch.float32,
+        init_device: str = "cpu",
+    ):
+        super().__init__()
+        if d_model % 16 or hidden_size % 16:
+            raise ValueError("float8 grouped GEMMs need d_model and hidden_size to be multiples of 16")
+        self.d_model = d_model
+        self.hidden_size = hidden_size
+        self.num_experts = num_experts
+        shape = (num_experts * hidden_size, d_model)
+        self.w1 = nn.Parameter(torch.empty(*shape, device=init_device, dtype=dtype))
+        self.w2 = nn.Parameter(torch.empty(*shape, device=init_device, dtype=dtype))
+        self.w3 = nn.Parameter(torch.empty(*shape, device=init_device, dtype=dtype))
+        self.reset_parameters()
+
+    def reset_parameters(self) -> None:
+        for w in (self.w1, self.w2, self.w3):
+            if not w.is_meta:
+                nn.init.kaiming_uniform_(w, a=math.sqrt(5))
+
+    def forward(self, x: torch.Tensor, batch_size_per_expert: torch.Tensor) -> torch.Tensor:
+        """
+        :param x: the expert inputs of shape ``(*, d_model)``, rows ordered by expert.
+        :param batch_size_per_expert: how many rows go to each expert, a 1-D ``LongTensor``.
+        """
+        lead = x.shape[:-1]
+        x2 = x.reshape(-1, self.d_model)
+        if x2.dtype != torch.bfloat16:
+            x2 = x2.to(torch.bfloat16)
+        y = float8_dropless_mlp(x2, self.w1, self.w2, self.w3, batch_size_per_expert, self.num_experts)
+        return y.reshape(*lead, self.d_model).to(x.dtype)
