@@ -43,6 +43,116 @@ def build_mlp(dev):
     return mlp, x, go
 
 
+# ---- the other BASELINE configurations (parity-test shapes; measured with --config N for the design notes) ----
+
+
+def build_config(n, dev):
+    """Returns (step_fn, flops_per_step, gemms_per_step, flops_per_gemm_launch or None, description)."""
+    from olmo_core_amd.float8 import AOFloat8LinearRecipe, Float8Config
+    from olmo_core_amd.nn import DroplessMoEMLP, FeedForward
+
+    def rand(shape, g, std=1.0):
+        return (torch.randn(shape, generator=g) * std).to(torch.bfloat16)
+
+    if n == 1:
+        g = torch.Generator().manual_seed(0)
+        x = rand((2048, 4096), g).to(dev)
+        lin = torch.nn.Linear(4096, 11008, bias=False, dtype=torch.bfloat16)
+        with torch.no_grad():
+            lin.weight.copy_(rand((11008, 4096), g, 0.02))
+        seq = torch.nn.Sequential(lin).to(dev)
+        Float8Config(ao_recipe=AOFloat8LinearRecipe.tensorwise).apply_float8_linear(seq)
+
+        def fn():
+            with torch.no_grad():
+                seq(x)
+
+        f = 2.0 * 2048 * 4096 * 11008
+        return fn, f, 1, f, "config 1: one Float8Linear forward 2048x4096 -> 11008, tensorwise"
+    if n in (2, 4):
+        d, h, m, seed = (4096, 11008, 16384, 1002) if n == 2 else (5120, 27648, 8192, 1004)
+        g = torch.Generator().manual_seed(seed)
+        mlp = FeedForward(d_model=d, hidden_size=h, bias=False, dtype=torch.bfloat16)
+        with torch.no_grad():
+            for p in mlp.parameters():
+                p.copy_(rand(p.shape, g, 0.02))
+        mlp = mlp.to(dev)
+        Float8Config(ao_recipe=AOFloat8LinearRecipe.tensorwise).apply_float8_linear(mlp)
+        x = torch.randn(m, d, generator=g)
+        if n == 4:  # 0.1 % of the entries x100
+            pos = torch.randperm(m * d, generator=g)[: m * d // 1000]
+            x.view(-1)[pos] *= 100
+        x = x.to(torch.bfloat16).to(dev).requires_grad_(True)
+        go = rand((m, d), g, 1e-3).to(dev)
+        f = 2.0 * m * d * h
+        name = "OLMo-2-7B" if n == 2 else "OLMo-2-32B (0.1 % outliers x100)"
+        return (lambda: step(mlp, x, go)), 9 * f, 9, f, f"config {n}: {name} SwiGLU MLP fwd+bwd, tokens {m}, tensorwise"
+    if n == 3:
+        g = torch.Generator().manual_seed(1003)
+        m, d = 16384, 4096
+        mods = torch.nn.ModuleList([torch.nn.Linear(d, d, bias=False, dtype=torch.bfloat16) for _ in range(4)])
+        with torch.no_grad():
+            for p in mods.parameters():
+                p.copy_(rand(p.shape, g, 0.02))
+        mods = mods.to(dev)
+        Float8Config(ao_recipe=AOFloat8LinearRecipe.rowwise).apply_float8_linear(mods)
+        x = rand((m, d), g).to(dev).requires_grad_(True)
+        go = rand((m, d), g, 1e-3).to(dev)
+
+        def fn():
+            x.grad = None
+            for lin in mods:
+                lin.weight.grad = None
+                lin(x).backward(go)
+
+        f = 2.0 * m * d * d
+        return fn, 12 * f, 12, f, "config 3: OLMo-3-7B q/k/v/o projections fwd+bwd, tokens 16384, rowwise recipe"
+    if n == 5:
+        g = torch.Generator().manual_seed(1005)
+        E, d, h, T, top_k = 64, 2048, 1024, 16384, 8
+        rank = torch.arange(1, E + 1, dtype=torch.float64)
+        pmf = rank ** -1.1
+        pmf = pmf / pmf.sum()
+        logits = torch.randn(T, E, generator=g) + (1.75 * torch.log(pmf)).float()  # Zipf(s=1.1) bias: 7 of 64 experts get no token
+        idx = logits.float().softmax(-1).topk(top_k, dim=-1).indices.reshape(-1)
+        sizes = torch.bincount(idx, minlength=E)
+        mlp = DroplessMoEMLP(d_model=d, hidden_size=h, num_experts=E, dtype=torch.bfloat16)
+        with torch.no_grad():
+            for p in mlp.parameters():
+                p.copy_(rand(p.shape, g, 0.02))
+        mlp = mlp.to(dev)
+        x = rand((T * top_k, d), g).to(dev).requires_grad_(True)
+        go = rand((T * top_k, d), g, 1e-3).to(dev)
+        sizes_d = sizes.to(dev)
+
+        def fn():
+            x.grad = None
+            for p in mlp.parameters():
+                p.grad = None
+            mlp(x, sizes_d).backward(go)
+
+        f = float(T * top_k) * 18 * d * h
+        desc = (f"config 5: dropless MoE experts fwd+bwd, 64 experts, {T * top_k} rows, group sizes min {int(sizes.min())} "
+                f"max {int(sizes.max())} empty {int((sizes == 0).sum())}, grouped rowwise")
+        return fn, f, 9, None, desc
+    raise ValueError(n)
+
+
+def run_other_config(n, steps, warmup):
+    dev = torch.device("cuda:0")
+    fn, flops, _, _, desc = build_config(n, dev)
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        fn()
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) / steps * 1e3
+    print(json.dumps({"config": desc, "ms_per_step": round(ms, 4), "TFLOP/s": round(flops / ms / 1e9, 1),
+                      "pct_fp8_mfma_peak": round(100 * flops / ms / 1e9 / FP8_MFMA_PEAK_TFLOPS, 2), "steps": steps}), flush=True)
+
+
 def step(mlp, x, go):
     x.grad = None
     for p in mlp.parameters():
@@ -73,12 +183,12 @@ def cpu_baseline(target_seconds: float = 15.0):
         O.mlp_fwd_bwd(x, w1, w2, w3, go, spec)
         return time.perf_counter() - t0
 
-    probe_m = 256
-    run(probe_m)  # warm the thread pool
+    probe_m = 1024
+    run(256)  # warm the thread pool
     t_probe = run(probe_m)
     m = int(min(TOKENS, max(probe_m, probe_m * target_seconds / max(t_probe, 1e-3))))
     m = max(256, (m // 256) * 256)
-    t = run(m)
+    t = run(m) if m != probe_m else t_probe
     flops = GEMMS_PER_STEP * 2.0 * m * D_MODEL * HIDDEN
     return {
         "value": round(flops / t / 1e12, 4),
@@ -95,6 +205,7 @@ def main():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--config", type=int, default=2, help="BASELINE configuration 1..5 (2 is the benchmark line)")
     ns = ap.parse_args()
     if ns.gpus != 1:
         print("bench.py: this build measures the float8 linear path on ONE GPU; --gpus must be 1", file=sys.stderr)
@@ -104,6 +215,10 @@ def main():
         sys.exit(2)
 
     from olmo_core_amd.float8 import ops
+
+    if ns.config != 2:
+        run_other_config(ns.config, ns.steps, ns.warmup)
+        return
 
     dev = torch.device("cuda:0")
     mlp, x, go = build_mlp(dev)
