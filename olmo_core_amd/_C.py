@@ -14,7 +14,10 @@ from typing import Optional
 
 from .exceptions import MI8KernelError
 
-LIB_PATH = Path(__file__).resolve().parent / "lib" / "libmi8.so"
+import os
+
+# MI8_LIBRARY overrides the in-tree location (e.g. to try a differently built library)
+LIB_PATH = Path(os.environ.get("MI8_LIBRARY") or (Path(__file__).resolve().parent / "lib" / "libmi8.so"))
 
 MI8_E4M3, MI8_E5M2 = 0, 1
 MI8_BF16, MI8_F32 = 0, 1

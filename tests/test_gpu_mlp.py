@@ -52,12 +52,12 @@ def test_mlp_against_oracle(dev, recipe):
     ref = O.mlp_fwd_bwd(x, w1, w2, w3, go, O.recipe(recipe))
     y, gx, gw1, gw2, gw3 = _run(ff, x.to(dev), go.to(dev))
     assert_gemm_close(y, ref.y, "y")
-    assert_gemm_close(gw2, ref.grad_w2, "grad_w2")
-    # The 1e-2 / 0.9999 bar is for one GEMM on identical operands.  These three gradients are compositions:
+    # The 1e-2 / 0.9999 bar is for one GEMM on identical operands.  The gradients are compositions:
     # the device's bf16 intermediates (h, the gate gradients) differ from the host's in the last bf16 ulp on a
     # few elements (different exp), and a re-quantisation to e5m2 (2 mantissa bits) can turn such an ulp into
     # one fp8 step.  The cosine bar is kept, the max-error bar is doubled for the compositions.
-    for name, got, want in (("grad_x", gx, ref.grad_x), ("grad_w1", gw1, ref.grad_w1), ("grad_w3", gw3, ref.grad_w3)):
+    for name, got, want in (("grad_x", gx, ref.grad_x), ("grad_w1", gw1, ref.grad_w1), ("grad_w2", gw2, ref.grad_w2),
+                            ("grad_w3", gw3, ref.grad_w3)):
         rel, cos = gemm_errors(got, want)
         assert rel <= 2e-2 and cos >= 0.9999, (name, rel, cos)
 
