@@ -25,6 +25,9 @@ import torch
 D_MODEL, HIDDEN, TOKENS = 4096, 11008, 16384
 FP8_MFMA_PEAK_TFLOPS = 5000.0  # MI355X dense fp8 matrix peak
 GEMMS_PER_STEP = 9
+# HBM-side bytes per GEMM launch (L2 fill reads + writes), mean over the 9 launches of a step, from the
+# FETCH_SIZE / WRITE_SIZE counter runs summarised in profiles/gemm_fp8_dma8_kernel__mlp7b_traffic_pmc.txt
+GEMM_TRAFFIC_BYTES_PER_LAUNCH = 1.558e9
 
 
 def build_mlp(dev):
@@ -153,6 +156,36 @@ def run_other_config(n, steps, warmup):
                       "pct_fp8_mfma_peak": round(100 * flops / ms / 1e9 / FP8_MFMA_PEAK_TFLOPS, 2), "steps": steps}), flush=True)
 
 
+def traffic_probe():
+    """Workload for the rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs: a plain 256 MiB device copy (the
+    calibration: 268435456 bytes read and written), then the three GEMM shapes of the benchmark step and the
+    amax + cast of the 16384 x 4096 activation, a few launches each, nothing timed."""
+    from olmo_core_amd.float8 import ops
+
+    dev = torch.device("cuda:0")
+    e4m3, e5m2 = torch.float8_e4m3fn, torch.float8_e5m2
+    src = torch.randint(0, 255, (1 << 28,), dtype=torch.uint8, device=dev)
+    dst = torch.empty_like(src)
+    for _ in range(3):
+        dst.copy_(src)
+    torch.cuda.synchronize()
+    one = torch.ones(1, device=dev)
+    shapes = [(TOKENS, HIDDEN, D_MODEL, e4m3), (TOKENS, D_MODEL, HIDDEN, e5m2), (HIDDEN, D_MODEL, TOKENS, e5m2)]
+    for M, N, K, da in shapes:
+        a = torch.randn(M, K, device=dev).to(da)
+        b = torch.randn(N, K, device=dev).to(e4m3)
+        for _ in range(3):
+            ops.gemm_fp8(a, one, b, one)
+        torch.cuda.synchronize()
+        del a, b
+    x = torch.randn(TOKENS, D_MODEL, device=dev, dtype=torch.bfloat16)
+    for _ in range(3):
+        slots = ops.amax_partials(x)
+        ops.cast_tensorwise(x, e4m3, want_transposed=True, slots=slots)
+    torch.cuda.synchronize()
+    print("traffic probe done", flush=True)
+
+
 def step(mlp, x, go):
     x.grad = None
     for p in mlp.parameters():
@@ -206,6 +239,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--config", type=int, default=2, help="BASELINE configuration 1..5 (2 is the benchmark line)")
+    ap.add_argument("--traffic-probe", action="store_true", help="workload for the FETCH_SIZE/WRITE_SIZE counter runs")
     ns = ap.parse_args()
     if ns.gpus != 1:
         print("bench.py: this build measures the float8 linear path on ONE GPU; --gpus must be 1", file=sys.stderr)
@@ -216,6 +250,9 @@ def main():
 
     from olmo_core_amd.float8 import ops
 
+    if ns.traffic_probe:
+        traffic_probe()
+        return
     if ns.config != 2:
         run_other_config(ns.config, ns.steps, ns.warmup)
         return
@@ -275,7 +312,7 @@ def main():
             "peak": FP8_MFMA_PEAK_TFLOPS,
             "unit": "TFLOP/s",
             "frac": round(achieved / FP8_MFMA_PEAK_TFLOPS, 4),
-            "traffic": None,
+            "traffic": GEMM_TRAFFIC_BYTES_PER_LAUNCH,
             "avg_launch_us": round(avg_gemm_s * 1e6, 2),
             "gemm_share_of_step": round(sum(gemm_ms) / ns.steps / ms_per_step, 4),
         },

@@ -133,27 +133,34 @@ __device__ __forceinline__ void gemm_tile_body(const GemmArgs& g, const int m0, 
     }
 
     // ---- epilogue: scale, round to bf16, store ------------------------------------------------------
-    // accumulator element e of lane l is C[row = 8*(e/4) + 4*(l/32) + e%4][col = l%32] of its 32x32 tile
-    const float isb_scalar = g.sb_vec ? 0.0f : 1.0f / g.sb[0];
-    const float isa_scalar = g.sa_vec ? 0.0f : 1.0f / g.sa[0];
+    // accumulator element e of lane l is C[row = 8*(e/4) + 4*(l/32) + e%4][col = l%32] of its 32x32 tile.
+    // Scalar scales are inverted with an IEEE division; per-row / per-column scale vectors with v_rcp_f32
+    // (exact for the power-of-two scales of the axiswise recipes, within 1 ulp otherwise).
+    float isb[TN];
+    bool col_ok[TN];
 #pragma unroll
     for (int j = 0; j < TN; ++j) {
         const int col = n0 + wn * WTN + j * 32 + l32;
-        const bool col_ok = col < g.N;
-        const float isb = g.sb_vec ? (col_ok ? 1.0f / g.sb[col] : 0.0f) : isb_scalar;
+        col_ok[j] = col < g.N;
+        isb[j] = g.sb_vec ? (col_ok[j] ? __builtin_amdgcn_rcpf(g.sb[col]) : 0.0f) : 1.0f / g.sb[0];
+    }
+    const float isa_scalar = g.sa_vec ? 0.0f : 1.0f / g.sa[0];
 #pragma unroll
-        for (int i = 0; i < TM; ++i) {
+    for (int i = 0; i < TM; ++i) {
 #pragma unroll
-            for (int e = 0; e < 16; ++e) {
-                const int row = m0 + wm * WTM + i * 32 + 8 * (e >> 2) + 4 * half + (e & 3);
-                if (col_ok && row < g.M) {
-                    const float isa = g.sa_vec ? 1.0f / g.sa[row] : isa_scalar;
-                    const float v = acc[i][j][e] * isa * isb;
-                    if (g.c_f32)
-                        reinterpret_cast<float*>(g.C)[(int64_t)row * g.ldc + col] = v;
-                    else
-                        reinterpret_cast<uint16_t*>(g.C)[(int64_t)row * g.ldc + col] = f32_to_bf16_bits(v);
-                }
+        for (int e = 0; e < 16; ++e) {
+            const int row = m0 + wm * WTM + i * 32 + 8 * (e >> 2) + 4 * half + (e & 3);
+            if (row >= g.M) continue;
+            const float isa = g.sa_vec ? __builtin_amdgcn_rcpf(g.sa[row]) : isa_scalar;
+#pragma unroll
+            for (int j = 0; j < TN; ++j) {
+                if (!col_ok[j]) continue;
+                const int col = n0 + wn * WTN + j * 32 + l32;
+                const float v = acc[i][j][e] * isa * isb[j];
+                if (g.c_f32)
+                    reinterpret_cast<float*>(g.C)[(int64_t)row * g.ldc + col] = v;
+                else
+                    reinterpret_cast<uint16_t*>(g.C)[(int64_t)row * g.ldc + col] = f32_to_bf16_bits(v);
             }
         }
     }

@@ -13,8 +13,9 @@ namespace mi8 {
 using namespace gemm;
 namespace {
 
-constexpr int GBM = 128, GBN = 128;
-constexpr int kGroupedThreads = 256;
+constexpr int GBM = 256, GBN = 256;  // 8 waves of 128 x 64: the best general-shape configuration measured
+constexpr int GWM = 2, GWN = 4;
+constexpr int kGroupedThreads = GWM * GWN * 64;
 constexpr int kGroupedLds = 2 * (GBM + GBN) * BK;
 
 struct GroupedArgs {
@@ -71,7 +72,7 @@ __global__ __launch_bounds__(kGroupedThreads, 1) void grouped_gemm_kernel(Groupe
     g.sb_vec = 1;
     g.tiles_m = 0;
     g.tiles_n = a.tiles_n;
-    gemm_tile_body<GBM, GBN, 2, 2, CBSZ, BLGP>(g, (mt - tiles_before) * GBM, nt * GBN, lds);
+    gemm_tile_body<GBM, GBN, GWM, GWN, CBSZ, BLGP>(g, (mt - tiles_before) * GBM, nt * GBN, lds);
 }
 
 struct GroupedWgradArgs {
@@ -132,7 +133,7 @@ __global__ __launch_bounds__(kGroupedThreads, 1) void grouped_wgrad_kernel(Group
     g.sb_vec = seg ? 1 : 0;
     g.tiles_m = 0;
     g.tiles_n = a.tiles_k;
-    gemm_tile_body<GBM, GBN, 2, 2, CBSZ, BLGP>(g, tn * GBM, tk * GBN, lds);
+    gemm_tile_body<GBM, GBN, GWM, GWN, CBSZ, BLGP>(g, tn * GBM, tk * GBN, lds);
 }
 
 template <typename K>
