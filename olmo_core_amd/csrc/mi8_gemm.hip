@@ -115,13 +115,14 @@ extern "C" int mi8_gemm_fp8(const void* a, int a_dtype, int64_t lda, const void*
                sa, sb, sa_is_vector ? 1 : 0, sb_is_vector ? 1 : 0, 0, 0};
     hipStream_t st = (hipStream_t)stream;
     const bool dma_ok = (K % 64 == 0) && M >= 256 && N >= 256 && N % 8 == 0 && ldc % 8 == 0 && aligned16(out) &&
-                        out_dtype == MI8_BF16;
+                        out_dtype == MI8_BF16 && (!sb_is_vector || aligned16(sb)) &&
+                        (sa_is_vector != 0) == (sb_is_vector != 0);
     if (variant < 0) variant = dma_ok ? (K % 128 == 0 ? kDma8 : kDma) : 1;
     if (variant == kDma8 && dma_ok && K % 128 == 0) return launch_dma8(g, a_dtype, b_dtype, st);
     if (variant == kDma || variant == kDma8) {
         MI8_REQUIRE(dma_ok && variant == kDma, MI8_ERR_UNSUPPORTED,
-                    "mi8_gemm_fp8: the direct-to-LDS variant needs M, N >= 256, K %% 64 == 0 (8 waves: 128), N %% 8 == 0, ldc %% 8 == 0 "
-                    "and a 16-byte aligned bf16 output (M=%lld N=%lld K=%lld ldc=%lld)",
+                    "mi8_gemm_fp8: the direct-to-LDS variant needs M, N >= 256, K %% 64 == 0 (8 waves: 128), N %% 8 == 0, ldc %% 8 == 0, "
+                    "scales that are both single values or both vectors, and a 16-byte aligned bf16 output (M=%lld N=%lld K=%lld ldc=%lld)",
                     (long long)M, (long long)N, (long long)K, (long long)ldc);
         return launch_dma(g, a_dtype, b_dtype, st);
     }

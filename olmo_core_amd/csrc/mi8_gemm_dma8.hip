@@ -1,5 +1,5 @@
 // Persistent fp8 GEMM, 8 waves per workgroup, direct global->LDS loads of full 128-byte rows.
-// For full 256 x 256 tiles, K % 128 == 0 and bf16 output.
+// For full 256 x 256 tiles, K % 128 == 0, bf16 output, and scales that are both single values or both vectors.
 //
 // Why 8 waves: the load bandwidth one CU can pull out of L2 grows with the number of waves that issue loads
 // (measured on MI355X with 1 KB global_load_lds_dwordx4 instructions: 4 waves ~54 GB/s, 8 waves ~81 GB/s per
@@ -42,8 +42,194 @@ struct Frags {
 __device__ __forceinline__ constexpr int frag_a(int i) { return i == 0 ? 0 : 4 + 2 * i; }
 __device__ __forceinline__ constexpr int frag_b(int j) { return 2 + 2 * j; }
 
-template <int CBSZ_A, int BLGP_B>
-__global__ __launch_bounds__(NT, 1) void gemm_fp8_dma8_kernel(GemmArgs g)
+
+// ---- what a workgroup needs to know about one output tile ---------------------------------------------
+struct TileDesc {
+    const uint8_t* a;  // first A row of the tile (K offset 0 of the tile's contraction range)
+    const uint8_t* b;  // first B row of the tile
+    int nk;            // 128-byte K steps (0: the tile is all zeros)
+    const float* sa;   // scale of the tile's first row (or the single scale)
+    const float* sb;   // scale of the tile's first column (or the single scale)
+    uint16_t* c;       // C element (first row, first column) of the tile
+    int row_lo, row_hi;  // rows [row_lo, row_hi) of the 256 are stored
+};
+
+// Dense problem: C[M, N] = A[M, K] . B[N, K]^T.  The last tile row / column is shifted back so that every tile
+// is full (M, N >= 256): the overlap is recomputed with the same K order and rewritten with identical values.
+template <bool VEC>
+struct DenseProblem {
+    GemmArgs g;
+    int64_t lda, ldb, ldc;
+    static constexpr bool kVecScales = VEC;  // both scales are vectors (per row / per column) or both single
+    static constexpr bool kMaskRows = false, kXcdRanges = true;
+    __device__ __forceinline__ int total_tiles() const { return g.tiles_m * g.tiles_n; }
+    __device__ __forceinline__ TileDesc tile(int t) const
+    {
+        int tm, tn;
+        tile_coords(g, t, tm, tn);
+        const int m0 = (tm * BM + BM <= g.M) ? tm * BM : g.M - BM;
+        const int n0 = (tn * BN + BN <= g.N) ? tn * BN : g.N - BN;
+        TileDesc d;
+        d.a = g.A + (int64_t)m0 * g.lda;
+        d.b = g.B + (int64_t)n0 * g.ldb;
+        d.nk = g.K / BK;
+        d.sa = g.sa + (VEC ? m0 : 0);
+        d.sb = g.sb + (VEC ? n0 : 0);
+        d.c = reinterpret_cast<uint16_t*>(g.C) + (int64_t)m0 * g.ldc + n0;
+        d.row_lo = 0;
+        d.row_hi = BM;
+        return d;
+    }
+};
+
+// ---- locating a group in the device-resident size list ---------------------------------------------------
+// Groups are consecutive row ranges; sizes are clamped so that their running sum never passes T.  A group of
+// m rows owns ceil(m / U) "units" (row tiles).  The 64 lanes of a wave each take one group of a 64-group chunk
+// and prefix-sum rows and units with shuffles, so a lookup costs one load latency instead of E dependent
+// ones.  Must be called by all lanes of the wave together; the result is wave-uniform.
+struct GroupSpan {
+    int e;                 // group index (E if the key is past the end)
+    int64_t rows_before;   // rows of the groups before it
+    int64_t m;             // its clamped size
+    int64_t units_before;  // units of the groups before it (all units if the key is past the end)
+};
+
+__device__ __forceinline__ int64_t uniform64(int64_t v)
+{
+    const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v);
+    const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)((uint64_t)v >> 32));
+    return (int64_t)(((uint64_t)hi << 32) | lo);
+}
+
+__device__ __forceinline__ int64_t wave_inclusive_sum(int64_t v, int lane)
+{
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+        const int64_t o = __shfl_up(v, d, 64);
+        if (lane >= d) v += o;
+    }
+    return v;
+}
+
+// BY_UNIT: key is a unit index, find the group that owns it; otherwise key is the group index itself.
+template <int U, bool BY_UNIT>
+__device__ __forceinline__ GroupSpan locate_group(const int64_t* sizes, int E, int64_t T, int64_t key)
+{
+    const int lane = (int)threadIdx.x & 63;
+    int64_t rows_c = 0, units_c = 0;
+    for (int base = 0; base < E; base += 64) {
+        const int e = base + lane;
+        int64_t m = (e < E) ? sizes[e] : 0;
+        m = m < 0 ? 0 : (m > T ? T : m);
+        int64_t end = rows_c + wave_inclusive_sum(m, lane);
+        int64_t start = end - m;
+        end = end < T ? end : T;
+        start = start < T ? start : T;
+        const int64_t me = end - start;
+        const int64_t un = (me + U - 1) / U;
+        const int64_t uend = units_c + wave_inclusive_sum(un, lane);
+        const bool hit = (e < E) && (BY_UNIT ? key < uend : key == e);
+        const uint64_t mask = __ballot(hit);
+        if (mask) {
+            const int src = __ffsll((unsigned long long)mask) - 1;
+            GroupSpan r;
+            r.e = base + src;
+            r.rows_before = uniform64(__shfl(start, src, 64));
+            r.m = uniform64(__shfl(me, src, 64));
+            r.units_before = uniform64(__shfl(uend - un, src, 64));
+            return r;
+        }
+        rows_c = uniform64(__shfl(end, 63, 64));
+        units_c = uniform64(__shfl(uend, 63, 64));
+    }
+    return GroupSpan{E, rows_c, 0, units_c};
+}
+
+// Ragged-M grouped problem (dropless-MoE forward / grad_input): rows of A form consecutive groups, group e
+// multiplies B_e = B + e * b_group_stride.  A tile covers up to 256 rows of ONE group; it always loads a full
+// 256-row window (shifted back at the end of the matrix, T >= 256) and stores only its group's rows.
+struct GroupedProblem {
+    const uint8_t* A;
+    const uint8_t* B;
+    uint16_t* C;
+    int64_t lda, ldb, ldc, b_group_stride, sb_group_stride;
+    const int64_t* sizes;
+    int E;
+    int64_t T;
+    int N, K, tiles_n;
+    const float* sa;
+    const float* sb;
+    static constexpr bool kVecScales = true, kMaskRows = true, kXcdRanges = true;
+    __device__ __forceinline__ int total_tiles() const
+    {
+        const GroupSpan s = locate_group<BM, true>(sizes, E, T, (int64_t)1 << 60);
+        return (int)s.units_before * tiles_n;
+    }
+    __device__ __forceinline__ TileDesc tile(int t) const
+    {
+        const int mt = t / tiles_n, nt = t % tiles_n;
+        const GroupSpan s = locate_group<BM, true>(sizes, E, T, mt);
+        const int64_t want0 = s.rows_before + (mt - s.units_before) * BM;  // first row this tile is responsible for
+        int64_t want1 = want0 + BM;
+        const int64_t group_end = s.rows_before + s.m;
+        want1 = want1 < group_end ? want1 : group_end;                     // ... up to the group's end
+        const int64_t m0 = (want0 + BM <= T) ? want0 : T - BM;             // loaded window
+        const int n0 = (nt * BN + BN <= N) ? nt * BN : N - BN;
+        TileDesc d;
+        d.a = A + m0 * lda;
+        d.b = B + (int64_t)s.e * b_group_stride + (int64_t)n0 * ldb;
+        d.nk = K / BK;
+        d.sa = sa + m0;
+        d.sb = sb + (int64_t)s.e * sb_group_stride + n0;
+        d.c = C + m0 * ldc + n0;
+        d.row_lo = (int)(want0 - m0);
+        d.row_hi = (int)(want1 - m0);
+        return d;
+    }
+};
+
+// Ragged-K grouped problem (dropless-MoE grad_weight): out[e] = A_t[:, S_e] . B_t[:, S_e]^T over group e's
+// 128-aligned segment S_e of the padded token axis; N, Kl >= 256.  An empty group gives nk = 0: its tiles are
+// written as zeros and its scales (never produced) are ignored.
+struct GroupedWgradProblem {
+    const uint8_t* At;
+    const uint8_t* Bt;
+    uint16_t* C;
+    int64_t lda, ldb, ldc;  // lda = ldb = padded token pitch, ldc = Kl
+    const int64_t* sizes;
+    int E;
+    int64_t T;
+    int N, Kl, tiles_n, tiles_k;
+    const float* sa;  // [E, N]
+    const float* sb;  // [E, Kl]
+    static constexpr bool kVecScales = true, kMaskRows = false, kXcdRanges = false;
+    __device__ __forceinline__ int total_tiles() const { return E * tiles_n * tiles_k; }
+    __device__ __forceinline__ TileDesc tile(int t) const
+    {
+        const int per_group = tiles_n * tiles_k;
+        const int e = t / per_group, rem = t % per_group;
+        const int tn = rem / tiles_k, tk = rem % tiles_k;
+        const GroupSpan s = locate_group<128, false>(sizes, E, T, e);
+        const int64_t seg0 = 128 * s.units_before;
+        int64_t seg = 128 * ((s.m + 127) / 128);
+        if (seg0 + seg > lda) seg = 0;
+        const int n0 = (tn * BM + BM <= N) ? tn * BM : N - BM;
+        const int k0 = (tk * BN + BN <= Kl) ? tk * BN : Kl - BN;
+        TileDesc d;
+        d.a = At + (int64_t)n0 * lda + seg0;
+        d.b = Bt + (int64_t)k0 * ldb + seg0;
+        d.nk = (int)(seg / BK);
+        d.sa = sa + (int64_t)e * N + n0;
+        d.sb = sb + (int64_t)e * Kl + k0;
+        d.c = C + ((int64_t)e * N + n0) * ldc + k0;
+        d.row_lo = 0;
+        d.row_hi = BM;
+        return d;
+    }
+};
+
+template <typename Problem, int CBSZ_A, int BLGP_B>
+__global__ __launch_bounds__(NT, 1) void gemm_fp8_dma8_kernel(Problem pb)
 {
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
 
@@ -79,58 +265,79 @@ __global__ __launch_bounds__(NT, 1) void gemm_fp8_dma8_kernel(GemmArgs g)
     // lane -> row 32 w + 8 p + lr (lr = lane / 8), position lane % 8; swz(row) = (lr ^ (4 w + p)) & 7
     const int lr = lane >> 3;
     const uint32_t c0 = (uint32_t)((lane & 7) ^ lr);
-    const uint32_t rowoff_a = (uint32_t)((int64_t)(wave * 32 + lr) * g.lda);
-    const uint32_t rowoff_b = (uint32_t)((int64_t)(wave * 32 + lr) * g.ldb);
+    const uint32_t rowoff_a = (uint32_t)((int64_t)(wave * 32 + lr) * pb.lda);
+    const uint32_t rowoff_b = (uint32_t)((int64_t)(wave * 32 + lr) * pb.ldb);
     // x in 0..7: 0..3 -> A rows 8 x, 4..7 -> B rows 8 (x - 4)
     auto dma_one = [&](const uint8_t* a_origin, const uint8_t* b_origin, int stage, int x) __attribute__((always_inline)) {
         const int p = x & 3;
-        const uint32_t chunk = (c0 ^ (uint32_t)((4 * wave + p) & 7)) << 4;
-        const uint8_t* src = x < 4 ? a_origin + (int64_t)(8 * p) * g.lda + (rowoff_a + chunk)
-                                   : b_origin + (int64_t)(8 * p) * g.ldb + (rowoff_b + chunk);
+        // uniform 64-bit base + 32-bit lane offset.  The empty asm makes the lane's chunk index opaque at every
+        // use: the offset is then rebuilt with two cheap vector instructions next to the load (and folded into
+        // its scalar-base addressing) instead of living in eight hoisted 64-bit lane addresses.
+        uint32_t c = c0;
+        asm volatile("" : "+v"(c));
+        const uint32_t voff = (x < 4 ? rowoff_a : rowoff_b) + ((c ^ (uint32_t)((4 * wave + p) & 7)) << 4);
+        const uint8_t* src = (x < 4 ? a_origin + (int64_t)(8 * p) * pb.lda : b_origin + (int64_t)(8 * p) * pb.ldb) + voff;
         uint8_t* dst = lds + stage * STAGE + (x < 4 ? 0 : BM * BK) + (wave * 32 + 8 * p) * BK;
         __builtin_amdgcn_global_load_lds((gptr_t)src, (lptr_t)dst, 16, 0, 0);
     };
 
     // ---- this workgroup's tiles: XCD-contiguous ranges, persistent over the `slots` workgroups of its XCD
-    const int total = g.tiles_m * g.tiles_n;
-    const int per_xcd = (total + 7) / 8;
-    const int xcd = (int)blockIdx.x & 7;
-    const int slot = (int)blockIdx.x >> 3;
-    const int slots = ((int)gridDim.x + 7 - xcd) >> 3;
-    const int first = xcd * per_xcd;
-    int last = first + per_xcd;
-    last = last < total ? last : total;
-    const int my_tiles = (first + slot < last) ? (last - first - slot + slots - 1) / slots : 0;
+    // Workgroups are dealt round-robin to the 8 XCDs (blockIdx % 8).  Tiles of equal cost: every XCD takes a
+    // contiguous range of the tile order (its L2 then sees neighbouring tiles) and the `slots` workgroups of the
+    // XCD stride through it.  Tiles of unequal cost: plain striding over all workgroups, so that the heavy
+    // groups are spread over all XCDs.
+    const int total = pb.total_tiles();
+    int first_tile, tile_stride, my_tiles;
+    if constexpr (Problem::kXcdRanges) {
+        const int per_xcd = (total + 7) / 8;
+        const int xcd = (int)blockIdx.x & 7;
+        const int slot = (int)blockIdx.x >> 3;
+        const int slots = ((int)gridDim.x + 7 - xcd) >> 3;
+        const int first = xcd * per_xcd;
+        int last = first + per_xcd;
+        last = last < total ? last : total;
+        first_tile = first + slot;
+        tile_stride = slots;
+        my_tiles = (first_tile < last) ? (last - first_tile + slots - 1) / slots : 0;
+    } else {
+        first_tile = (int)blockIdx.x;
+        tile_stride = (int)gridDim.x;
+        my_tiles = (first_tile < total) ? (total - first_tile + tile_stride - 1) / tile_stride : 0;
+    }
     if (my_tiles == 0) return;
-    const int nk = g.K / BK;
+    auto my_tile = [&](int idx) __attribute__((always_inline)) { return pb.tile(first_tile + idx * tile_stride); };
 
-    auto tile_origin = [&](int idx, int& m0, int& n0) __attribute__((always_inline)) {
-        int tm, tn;
-        tile_coords(g, first + slot + idx * slots, tm, tn);
-        // the last tile row / column is shifted back so that every tile is full (M, N >= 256): the overlap is
-        // recomputed with the same K order and rewritten with identical values
-        m0 = (tm * BM + BM <= g.M) ? tm * BM : g.M - BM;
-        n0 = (tn * BN + BN <= g.N) ? tn * BN : g.N - BN;
+    // load cursor: the K step whose stage is fetched next (two steps ahead of the compute cursor); it skips
+    // tiles without K steps and, past the last tile, keeps fetching valid data nobody reads
+    int ld_tile = -1, ld_kt = 0, ld_nk = 0;
+    const uint8_t* ld_a = nullptr;
+    const uint8_t* ld_b = nullptr;
+    auto next_load_tile = [&]() __attribute__((always_inline)) {
+        while (ld_tile + 1 < my_tiles) {
+            ++ld_tile;
+            const TileDesc d = my_tile(ld_tile);
+            if (d.nk > 0) {
+                ld_a = d.a;
+                ld_b = d.b;
+                ld_nk = d.nk;
+                ld_kt = 0;
+                return;
+            }
+        }
+        // no further tile with work: rewind to the start of the current one (or stay null if there never was one)
+        if (ld_a) {
+            ld_a -= (int64_t)ld_kt * BK;
+            ld_b -= (int64_t)ld_kt * BK;
+            ld_kt = 0;
+        }
     };
-
-    // load cursor: the K step whose stage is fetched next (two steps ahead of the compute cursor)
-    int ld_tile = 0, ld_kt = 0, ld_m0, ld_n0;
-    tile_origin(0, ld_m0, ld_n0);
-    const uint8_t* ld_a = g.A + (int64_t)ld_m0 * g.lda;
-    const uint8_t* ld_b = g.B + (int64_t)ld_n0 * g.ldb;
     auto advance_load_cursor = [&]() __attribute__((always_inline)) {
         ++ld_kt;
         ld_a += BK;
         ld_b += BK;
-        if (ld_kt == nk) {
-            ld_kt = 0;
-            // past the last tile the cursor stays on it: the extra loads fetch valid data nobody reads
-            if (ld_tile + 1 < my_tiles) ++ld_tile;
-            tile_origin(ld_tile, ld_m0, ld_n0);
-            ld_a = g.A + (int64_t)ld_m0 * g.lda;
-            ld_b = g.B + (int64_t)ld_n0 * g.ldb;
-        }
+        if (ld_kt >= ld_nk) next_load_tile();
     };
+    next_load_tile();
 
     v16f acc[TM][TN];
     auto clear_acc = [&]() __attribute__((always_inline)) {
@@ -150,11 +357,14 @@ __global__ __launch_bounds__(NT, 1) void gemm_fp8_dma8_kernel(GemmArgs g)
     };
 
     // ---- prologue: stages of steps 0 and 1, fragments of step 0 ----------------------------------------
+    const bool any_work = ld_a != nullptr;  // uniform
+    if (any_work) {
 #pragma unroll
-    for (int s = 0; s < 2; ++s) {
+        for (int s = 0; s < 2; ++s) {
 #pragma unroll
-        for (int x = 0; x < 8; ++x) dma_one(ld_a, ld_b, s, x);
-        advance_load_cursor();
+            for (int x = 0; x < 8; ++x) dma_one(ld_a, ld_b, s, x);
+            advance_load_cursor();
+        }
     }
     clear_acc();
     Frags f0, f1;
@@ -163,12 +373,10 @@ __global__ __launch_bounds__(NT, 1) void gemm_fp8_dma8_kernel(GemmArgs g)
 #pragma unroll
     for (int x = 0; x < NH; ++x) read_one(f0, lds, 0, x);
 
-    const float isb_scalar = 1.0f / g.sb[0];
     int step = 0;
     for (int cp_tile = 0; cp_tile < my_tiles; ++cp_tile) {
-        int m0, n0;
-        tile_origin(cp_tile, m0, n0);
-        for (int kt = 0; kt < nk; ++kt, ++step) {
+        const TileDesc td = my_tile(cp_tile);
+        for (int kt = 0; kt < td.nk; ++kt, ++step) {
             const int cur = step & 1;
             const uint8_t* st_cur = lds + cur * STAGE;
             const uint8_t* st_nxt = lds + (cur ^ 1) * STAGE;
@@ -201,26 +409,30 @@ __global__ __launch_bounds__(NT, 1) void gemm_fp8_dma8_kernel(GemmArgs g)
         }
 
         // ---- tile finished: epilogue -------------------------------------------------------------------
-        // acc[i][j][e] of lane l is C[row = m(i, l%32)][col = n(j) + 8*(e/4) + 4*(l/32) + e%4]
+        // acc[i][j][e] of lane l is C[row = 32 i + l%32][col = 32 j + 8*(e/4) + 4*(l/32) + e%4] of the wave tile.
+        // A single scale is inverted with an IEEE division, scale vectors with v_rcp_f32 (exact for the
+        // power-of-two scales of the axiswise recipes, within 1 ulp otherwise).
         uint8_t* stg = lds + 2 * STAGE + wave * (32 * WTN * 2);  // wave-private 4 KB: 32 rows x 128 bytes
+        const bool zero_tile = td.nk == 0;  // nothing accumulated; the scales may be unset
         float isb[TN][4][4];
-        if (g.sb_vec) {
+        if constexpr (Problem::kVecScales) {
 #pragma unroll
             for (int j = 0; j < TN; ++j)
 #pragma unroll
                 for (int q = 0; q < 4; ++q) {
-                    const float4 s4 = *reinterpret_cast<const float4*>(g.sb + n0 + wn * WTN + j * 32 + 8 * q + 4 * half);
-                    isb[j][q][0] = __builtin_amdgcn_rcpf(s4.x);
-                    isb[j][q][1] = __builtin_amdgcn_rcpf(s4.y);
-                    isb[j][q][2] = __builtin_amdgcn_rcpf(s4.z);
-                    isb[j][q][3] = __builtin_amdgcn_rcpf(s4.w);
+                    const float4 s4 = *reinterpret_cast<const float4*>(td.sb + wn * WTN + j * 32 + 8 * q + 4 * half);
+                    isb[j][q][0] = zero_tile ? 0.0f : __builtin_amdgcn_rcpf(s4.x);
+                    isb[j][q][1] = zero_tile ? 0.0f : __builtin_amdgcn_rcpf(s4.y);
+                    isb[j][q][2] = zero_tile ? 0.0f : __builtin_amdgcn_rcpf(s4.z);
+                    isb[j][q][3] = zero_tile ? 0.0f : __builtin_amdgcn_rcpf(s4.w);
                 }
         }
+        const float isb_scalar = Problem::kVecScales ? 1.0f : 1.0f / td.sb[0];
 #pragma unroll
         for (int i = 0; i < TM; ++i) {
-            const int row = m0 + wm * WTM + i * 32 + l32;
-            float mult = 1.0f / g.sa[g.sa_vec ? row : 0];
-            if (!g.sb_vec) mult *= isb_scalar;
+            const int rt = wm * WTM + i * 32;  // first tile row of this pass
+            float mult = Problem::kVecScales ? __builtin_amdgcn_rcpf(td.sa[rt + l32]) : 1.0f / td.sa[0];
+            mult = zero_tile ? 0.0f : mult * isb_scalar;
             // 32 rows x 64 bf16 through the wave's staging area: pitch 128 bytes, the 16-byte chunk index XORed
             // with (row >> 1) & 7 so that 16 consecutive rows cover all banks
 #pragma unroll
@@ -232,7 +444,7 @@ __global__ __launch_bounds__(NT, 1) void gemm_fp8_dma8_kernel(GemmArgs g)
 #pragma unroll
                     for (int e = 0; e < 4; ++e) {
                         v[e] = acc[i][j][4 * q + e] * mult;
-                        if (g.sb_vec) v[e] *= isb[j][q][e];
+                        if constexpr (Problem::kVecScales) v[e] *= isb[j][q][e];
                     }
                     uint2 o;
                     o.x = (uint32_t)f32_to_bf16_bits(v[0]) | ((uint32_t)f32_to_bf16_bits(v[1]) << 16);
@@ -242,14 +454,21 @@ __global__ __launch_bounds__(NT, 1) void gemm_fp8_dma8_kernel(GemmArgs g)
                 }
             __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): the wave's own LDS writes have landed
             __builtin_amdgcn_wave_barrier();
+            uint4 staged[4];
 #pragma unroll
             for (int it = 0; it < 4; ++it) {
                 const int rw = it * 8 + (lane >> 3);
-                const int c8 = lane & 7;
-                const uint4 v = *reinterpret_cast<const uint4*>(stg + rw * 128 + ((c8 ^ ((rw >> 1) & 7)) << 4));
-                const int orow = m0 + wm * WTM + i * 32 + rw;
-                const int ocol = n0 + wn * WTN + c8 * 8;
-                *reinterpret_cast<uint4*>(reinterpret_cast<uint16_t*>(g.C) + (int64_t)orow * g.ldc + ocol) = v;
+                staged[it] = *reinterpret_cast<const uint4*>(stg + rw * 128 + (((lane & 7) ^ ((rw >> 1) & 7)) << 4));
+            }
+#pragma unroll
+            for (int it = 0; it < 4; ++it) {
+                const int trow = rt + it * 8 + (lane >> 3);
+                uint4* dst = reinterpret_cast<uint4*>(td.c + (int64_t)trow * pb.ldc + wn * WTN + (lane & 7) * 8);
+                if constexpr (Problem::kMaskRows) {
+                    if (trow >= td.row_lo && trow < td.row_hi) *dst = staged[it];
+                } else {
+                    *dst = staged[it];
+                }
             }
             __builtin_amdgcn_s_waitcnt(0xc07f);  // the reads are done before the next pass overwrites
             __builtin_amdgcn_wave_barrier();
@@ -274,35 +493,69 @@ int num_cus()
     return cached;
 }
 
-template <int CBSZ_A, int BLGP_B>
-int launch(GemmArgs& g, hipStream_t st)
+// persistent: one workgroup per CU walks a static share of the tiles (right when all tiles cost the same);
+// otherwise one workgroup per tile, handed to free CUs by the hardware dispatcher (tiles of unequal cost).
+template <typename Problem, int CBSZ_A, int BLGP_B>
+int launch(const Problem& pb, int max_tiles, bool persistent, hipStream_t st)
 {
-    auto kern = gemm_fp8_dma8_kernel<CBSZ_A, BLGP_B>;
+    auto kern = gemm_fp8_dma8_kernel<Problem, CBSZ_A, BLGP_B>;
     static bool configured = false;
     if (!configured) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES);
         if (e != hipSuccess) {
-            set_error("mi8_gemm_fp8: cannot reserve %d bytes of LDS: %s", LDS_BYTES, hipGetErrorString(e));
+            set_error("mi8 direct-to-LDS GEMM: cannot reserve %d bytes of LDS: %s", LDS_BYTES, hipGetErrorString(e));
             return MI8_ERR_LAUNCH;
         }
         configured = true;
     }
-    g.tiles_m = (g.M + BM - 1) / BM;
-    g.tiles_n = (g.N + BN - 1) / BN;
-    const int total = g.tiles_m * g.tiles_n;
-    int blocks = num_cus();
-    if (blocks > total) blocks = total;
-    hipLaunchKernelGGL(kern, dim3(blocks), dim3(NT), LDS_BYTES, st, g);
-    return launch_status("mi8_gemm_fp8(direct-to-LDS, 8 waves)");
+    int blocks = persistent ? num_cus() : max_tiles;
+    if (blocks > max_tiles) blocks = max_tiles;
+    hipLaunchKernelGGL(kern, dim3(blocks), dim3(NT), LDS_BYTES, st, pb);
+    return launch_status("mi8 direct-to-LDS GEMM (8 waves)");
+}
+
+template <typename Problem>
+int launch_typed(const Problem& pb, int max_tiles, bool persistent, int a_dtype, int b_dtype, hipStream_t st)
+{
+    if (a_dtype == MI8_E4M3)
+        return b_dtype == MI8_E4M3 ? launch<Problem, 0, 0>(pb, max_tiles, persistent, st)
+                                   : launch<Problem, 0, 1>(pb, max_tiles, persistent, st);
+    return b_dtype == MI8_E4M3 ? launch<Problem, 1, 0>(pb, max_tiles, persistent, st)
+                               : launch<Problem, 1, 1>(pb, max_tiles, persistent, st);
 }
 
 }  // namespace
 
 int launch_dma8(GemmArgs& g, int a_dtype, int b_dtype, hipStream_t st)
 {
-    if (a_dtype == MI8_E4M3) return b_dtype == MI8_E4M3 ? launch<0, 0>(g, st) : launch<0, 1>(g, st);
-    return b_dtype == MI8_E4M3 ? launch<1, 0>(g, st) : launch<1, 1>(g, st);
+    g.tiles_m = (g.M + BM - 1) / BM;
+    g.tiles_n = (g.N + BN - 1) / BN;
+    if (g.sa_vec) {
+        DenseProblem<true> pb{g, g.lda, g.ldb, g.ldc};
+        return launch_typed(pb, g.tiles_m * g.tiles_n, true, a_dtype, b_dtype, st);
+    }
+    DenseProblem<false> pb{g, g.lda, g.ldb, g.ldc};
+    return launch_typed(pb, g.tiles_m * g.tiles_n, true, a_dtype, b_dtype, st);
+}
+
+int launch_dma8_grouped(const uint8_t* a, int a_dtype, int64_t lda, const uint8_t* b, int b_dtype, int64_t ldb,
+                        int64_t b_group_stride, const int64_t* sizes, int E, int64_t T, int N, int K, const float* sa,
+                        const float* sb, int64_t sb_group_stride, uint16_t* out, int64_t ldc, hipStream_t st)
+{
+    const int tiles_n = (N + BN - 1) / BN;
+    GroupedProblem pb{a, b, out, lda, ldb, ldc, b_group_stride, sb_group_stride, sizes, E, T, N, K, tiles_n, sa, sb};
+    const int64_t max_tiles = ((T + BM - 1) / BM + E) * tiles_n;
+    return launch_typed(pb, max_tiles > (1 << 30) ? (1 << 30) : (int)max_tiles, true, a_dtype, b_dtype, st);
+}
+
+int launch_dma8_grouped_wgrad(const uint8_t* a_t, int a_dtype, const uint8_t* b_t, int b_dtype, int64_t ld_t,
+                              const int64_t* sizes, int E, int64_t T, int N, int Kl, const float* sa, const float* sb,
+                              uint16_t* out, hipStream_t st)
+{
+    const int tiles_n = (N + BM - 1) / BM, tiles_k = (Kl + BN - 1) / BN;
+    GroupedWgradProblem pb{a_t, b_t, out, ld_t, ld_t, Kl, sizes, E, T, N, Kl, tiles_n, tiles_k, sa, sb};
+    return launch_typed(pb, E * tiles_n * tiles_k, false, a_dtype, b_dtype, st);
 }
 
 }  // namespace gemm

@@ -205,6 +205,12 @@ extern "C" int mi8_grouped_gemm_fp8(const void* a, int a_dtype, int64_t lda, con
                   b_group_stride, sb_group_stride, group_sizes, num_groups, T, (int)N, (int)K, sa, sb, tiles_n};
     const int blocks = (int)(m_tiles * tiles_n);
     hipStream_t st = (hipStream_t)stream;
+    // full-tile shapes with bf16 output run on the persistent direct-to-LDS kernel
+    if (out_dtype == MI8_BF16 && T >= 256 && N >= 256 && K % 128 == 0 && N % 8 == 0 && ldc % 8 == 0 && aligned16(out) &&
+        sb_group_stride % 4 == 0 && aligned16(sb) && lda < (1 << 23) && ldb < (1 << 23))
+        return launch_dma8_grouped((const uint8_t*)a, a_dtype, lda, (const uint8_t*)b, b_dtype, ldb, b_group_stride,
+                                   group_sizes, num_groups, T, (int)N, (int)K, sa, sb, sb_group_stride, (uint16_t*)out,
+                                   ldc, st);
     if (a_dtype == MI8_E4M3)
         return b_dtype == MI8_E4M3 ? launch_grouped<0, 0>(g, blocks, st) : launch_grouped<0, 1>(g, blocks, st);
     return b_dtype == MI8_E4M3 ? launch_grouped<1, 0>(g, blocks, st) : launch_grouped<1, 1>(g, blocks, st);
@@ -229,6 +235,10 @@ extern "C" int mi8_grouped_wgrad_fp8(const void* a_t, int a_dtype, const void* b
                        sa, sb, out, out_dtype == MI8_F32 ? 1 : 0, tiles_n, tiles_k};
     const int blocks = num_groups * tiles_n * tiles_k;
     hipStream_t st = (hipStream_t)stream;
+    if (out_dtype == MI8_BF16 && N >= 256 && Kl >= 256 && Kl % 8 == 0 && aligned16(out) && aligned16(sb) &&
+        ld_t % 128 == 0 && ld_t < (1 << 23))
+        return launch_dma8_grouped_wgrad((const uint8_t*)a_t, a_dtype, (const uint8_t*)b_t, b_dtype, ld_t, group_sizes,
+                                         num_groups, T, (int)N, (int)Kl, sa, sb, (uint16_t*)out, st);
     if (a_dtype == MI8_E4M3)
         return b_dtype == MI8_E4M3 ? launch_wgrad<0, 0>(g, blocks, st) : launch_wgrad<0, 1>(g, blocks, st);
     return b_dtype == MI8_E4M3 ? launch_wgrad<1, 0>(g, blocks, st) : launch_wgrad<1, 1>(g, blocks, st);
