@@ -54,6 +54,8 @@ struct TileDesc {
     int row_lo, row_hi;  // rows [row_lo, row_hi) of the 256 are stored
 };
 
+struct NoCache {};
+
 // Dense problem: C[M, N] = A[M, K] . B[N, K]^T.  The last tile row / column is shifted back so that every tile
 // is full (M, N >= 256): the overlap is recomputed with the same K order and rewritten with identical values.
 template <bool VEC>
@@ -62,8 +64,10 @@ struct DenseProblem {
     int64_t lda, ldb, ldc;
     static constexpr bool kVecScales = VEC;  // both scales are vectors (per row / per column) or both single
     static constexpr bool kMaskRows = false, kXcdRanges = true;
-    __device__ __forceinline__ int total_tiles() const { return g.tiles_m * g.tiles_n; }
-    __device__ __forceinline__ TileDesc tile(int t) const
+    using Cache = NoCache;
+    __device__ __forceinline__ Cache prepare() const { return Cache{}; }
+    __device__ __forceinline__ int total_tiles(const Cache&) const { return g.tiles_m * g.tiles_n; }
+    __device__ __forceinline__ TileDesc tile(int t, const Cache&) const
     {
         int tm, tn;
         tile_coords(g, t, tm, tn);
@@ -145,6 +149,56 @@ __device__ __forceinline__ GroupSpan locate_group(const int64_t* sizes, int E, i
     return GroupSpan{E, rows_c, 0, units_c};
 }
 
+// Up to 64 groups: the prefix sums live in four registers of every wave for the whole kernel (lane e holds
+// group e), and a lookup is a ballot and three lane reads, with no memory access inside the K loop.
+struct GroupCache {
+    int start, m, ubefore, uend;  // per lane: first row, clamped size, units before, units up to and including
+    bool valid;                   // wave-uniform: E <= 64 (otherwise lookups go to memory)
+};
+
+template <int U>
+__device__ __forceinline__ GroupCache build_group_cache(const int64_t* sizes, int E, int64_t T)
+{
+    GroupCache c{0, 0, 0, 0, E <= 64};
+    if (!c.valid) return c;
+    const int lane = (int)threadIdx.x & 63;
+    int64_t m = (lane < E) ? sizes[lane] : 0;
+    m = m < 0 ? 0 : (m > T ? T : m);
+    int64_t end = wave_inclusive_sum(m, lane);
+    int64_t start = end - m;
+    end = end < T ? end : T;
+    start = start < T ? start : T;
+    const int64_t me = end - start;
+    const int64_t un = (me + U - 1) / U;
+    const int64_t uend = wave_inclusive_sum(un, lane);
+    c.start = (int)start;  // T < 2^30 is checked on the host
+    c.m = (int)me;
+    c.ubefore = (int)(uend - un);
+    c.uend = (int)uend;
+    return c;
+}
+
+template <int U, bool BY_UNIT>
+__device__ __forceinline__ GroupSpan locate_group_cached(const GroupCache& c, const int64_t* sizes, int E, int64_t T,
+                                                         int64_t key)
+{
+    if (!c.valid) return locate_group<U, BY_UNIT>(sizes, E, T, key);
+    int src;
+    if constexpr (BY_UNIT) {
+        const uint64_t mask = __ballot((int64_t)c.uend > key);
+        if (mask == 0) return GroupSpan{E, T, 0, __builtin_amdgcn_readlane(c.uend, 63)};
+        src = __ffsll((unsigned long long)mask) - 1;
+    } else {
+        src = (int)key;
+    }
+    GroupSpan r;
+    r.e = src;
+    r.rows_before = __builtin_amdgcn_readlane(c.start, src);
+    r.m = __builtin_amdgcn_readlane(c.m, src);
+    r.units_before = __builtin_amdgcn_readlane(c.ubefore, src);
+    return r;
+}
+
 // Ragged-M grouped problem (dropless-MoE forward / grad_input): rows of A form consecutive groups, group e
 // multiplies B_e = B + e * b_group_stride.  A tile covers up to 256 rows of ONE group; it always loads a full
 // 256-row window (shifted back at the end of the matrix, T >= 256) and stores only its group's rows.
@@ -160,15 +214,17 @@ struct GroupedProblem {
     const float* sa;
     const float* sb;
     static constexpr bool kVecScales = true, kMaskRows = true, kXcdRanges = true;
-    __device__ __forceinline__ int total_tiles() const
+    using Cache = GroupCache;
+    __device__ __forceinline__ Cache prepare() const { return build_group_cache<BM>(sizes, E, T); }
+    __device__ __forceinline__ int total_tiles(const Cache& c) const
     {
-        const GroupSpan s = locate_group<BM, true>(sizes, E, T, (int64_t)1 << 60);
+        const GroupSpan s = locate_group_cached<BM, true>(c, sizes, E, T, (int64_t)1 << 60);
         return (int)s.units_before * tiles_n;
     }
-    __device__ __forceinline__ TileDesc tile(int t) const
+    __device__ __forceinline__ TileDesc tile(int t, const Cache& c) const
     {
         const int mt = t / tiles_n, nt = t % tiles_n;
-        const GroupSpan s = locate_group<BM, true>(sizes, E, T, mt);
+        const GroupSpan s = locate_group_cached<BM, true>(c, sizes, E, T, mt);
         const int64_t want0 = s.rows_before + (mt - s.units_before) * BM;  // first row this tile is responsible for
         int64_t want1 = want0 + BM;
         const int64_t group_end = s.rows_before + s.m;
@@ -203,13 +259,15 @@ struct GroupedWgradProblem {
     const float* sa;  // [E, N]
     const float* sb;  // [E, Kl]
     static constexpr bool kVecScales = true, kMaskRows = false, kXcdRanges = false;
-    __device__ __forceinline__ int total_tiles() const { return E * tiles_n * tiles_k; }
-    __device__ __forceinline__ TileDesc tile(int t) const
+    using Cache = GroupCache;
+    __device__ __forceinline__ Cache prepare() const { return build_group_cache<128>(sizes, E, T); }
+    __device__ __forceinline__ int total_tiles(const Cache&) const { return E * tiles_n * tiles_k; }
+    __device__ __forceinline__ TileDesc tile(int t, const Cache& c) const
     {
         const int per_group = tiles_n * tiles_k;
         const int e = t / per_group, rem = t % per_group;
         const int tn = rem / tiles_k, tk = rem % tiles_k;
-        const GroupSpan s = locate_group<128, false>(sizes, E, T, e);
+        const GroupSpan s = locate_group_cached<128, false>(c, sizes, E, T, e);
         const int64_t seg0 = 128 * s.units_before;
         int64_t seg = 128 * ((s.m + 127) / 128);
         if (seg0 + seg > lda) seg = 0;
@@ -239,26 +297,22 @@ __global__ __launch_bounds__(NT, 1) void gemm_fp8_dma8_kernel(Problem pb)
     const int wm = wave >> 2, wn = wave & 3;
     const int l32 = lane & 31, half = lane >> 5;
 
-    // ---- fragment read offsets: rows r0 + 32 i; chunk (4 s + 2 half + q) ^ swz(r0 + 32 i)
-    //      = (4 (s ^ (i & 1)) + 2 half + q) ^ swz(r0)   [r0 a multiple of 64 plus l32]
-    uint32_t xa[2][2], xb[2][2];
-    {
-        const int ra0 = wm * WTM + l32, rb0 = wn * WTN + l32;
-#pragma unroll
-        for (int t = 0; t < 2; ++t)
-#pragma unroll
-            for (int q = 0; q < 2; ++q) {
-                xa[t][q] = (uint32_t)(ra0 * BK + (((4 * t + 2 * half + q) ^ swz(ra0)) << 4));
-                xb[t][q] = (uint32_t)(BM * BK + rb0 * BK + (((4 * t + 2 * half + q) ^ swz(rb0)) << 4));
-            }
-    }
-    // slot x of Frags: 0,1 = A0; 2..5 = B0,B1; 6..11 = A1..A3
-    auto read_one = [&](Frags& f, const uint8_t* st, int s, int x) __attribute__((always_inline)) {
+    // ---- fragment read offsets.  MFMA tile `tile` of a wave reads rows r0 + 32 tile (r0 = wave origin + l32, the
+    // wave origin a multiple of 64), 16-byte chunk (4 s + 2 half + q) ^ swz(row) of K sub-step s.  Adding 32 to
+    // the row flips bit 2 of swz, and 4 s, 2 half, q occupy disjoint bits, so
+    //     chunk = ((2 half) ^ swz(r0)) ^ (4 (s ^ (tile & 1)) | q).
+    // One register per operand holds the lane's byte offset for (s, q, tile) = 0; the stage base is added once
+    // per phase (no carries into the chunk bits) and every read XORs a literal into it.  Keeping only two
+    // registers instead of eight precomputed addresses matters: the kernel runs at the 256-register limit.
+    const uint32_t xa00 = (uint32_t)((wm * WTM + l32) * BK + (((2 * half) ^ swz(wm * WTM + l32)) << 4));
+    const uint32_t xb00 = (uint32_t)(BM * BK + (wn * WTN + l32) * BK + (((2 * half) ^ swz(wn * WTN + l32)) << 4));
+    // slot x of Frags: 0,1 = A0; 2..5 = B0,B1; 6..11 = A1..A3.  pa / pb: xa00 / xb00 plus the stage's byte offset.
+    auto read_one = [&](Frags& f, uint32_t pa, uint32_t pb_, int s, int x) __attribute__((always_inline)) {
         const bool is_a = (x < 2) || (x >= 6);
         const int tile = x < 2 ? 0 : (x < 6 ? (x - 2) >> 1 : (x - 4) >> 1);
         const int q = x & 1;
-        const uint32_t off = (is_a ? xa[s ^ (tile & 1)][q] : xb[s ^ (tile & 1)][q]) + tile * 32 * BK;
-        f.h[x] = *reinterpret_cast<const v4i*>(st + off);
+        const uint32_t off = ((is_a ? pa : pb_) ^ (uint32_t)(((4 * (s ^ (tile & 1))) | q) << 4)) + tile * 32 * BK;
+        f.h[x] = *reinterpret_cast<const v4i*>(lds + off);
     };
 
     // ---- direct loads: wave w fills rows [32 w + 8 p, +8) of each operand, p = 0..3;
@@ -286,7 +340,8 @@ __global__ __launch_bounds__(NT, 1) void gemm_fp8_dma8_kernel(Problem pb)
     // contiguous range of the tile order (its L2 then sees neighbouring tiles) and the `slots` workgroups of the
     // XCD stride through it.  Tiles of unequal cost: plain striding over all workgroups, so that the heavy
     // groups are spread over all XCDs.
-    const int total = pb.total_tiles();
+    const typename Problem::Cache cache = pb.prepare();
+    const int total = pb.total_tiles(cache);
     int first_tile, tile_stride, my_tiles;
     if constexpr (Problem::kXcdRanges) {
         const int per_xcd = (total + 7) / 8;
@@ -305,7 +360,7 @@ __global__ __launch_bounds__(NT, 1) void gemm_fp8_dma8_kernel(Problem pb)
         my_tiles = (first_tile < total) ? (total - first_tile + tile_stride - 1) / tile_stride : 0;
     }
     if (my_tiles == 0) return;
-    auto my_tile = [&](int idx) __attribute__((always_inline)) { return pb.tile(first_tile + idx * tile_stride); };
+    auto my_tile = [&](int idx) __attribute__((always_inline)) { return pb.tile(first_tile + idx * tile_stride, cache); };
 
     // load cursor: the K step whose stage is fetched next (two steps ahead of the compute cursor); it skips
     // tiles without K steps and, past the last tile, keeps fetching valid data nobody reads
@@ -371,22 +426,22 @@ __global__ __launch_bounds__(NT, 1) void gemm_fp8_dma8_kernel(Problem pb)
     __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wave's direct loads have landed
     __syncthreads();
 #pragma unroll
-    for (int x = 0; x < NH; ++x) read_one(f0, lds, 0, x);
+    for (int x = 0; x < NH; ++x) read_one(f0, xa00, xb00, 0, x);
 
     int step = 0;
     for (int cp_tile = 0; cp_tile < my_tiles; ++cp_tile) {
         const TileDesc td = my_tile(cp_tile);
         for (int kt = 0; kt < td.nk; ++kt, ++step) {
             const int cur = step & 1;
-            const uint8_t* st_cur = lds + cur * STAGE;
-            const uint8_t* st_nxt = lds + (cur ^ 1) * STAGE;
+            const uint32_t pa_cur = xa00 + cur * STAGE, pb_cur = xb00 + cur * STAGE;
+            const uint32_t pa_nxt = xa00 + (cur ^ 1) * STAGE, pb_nxt = xb00 + (cur ^ 1) * STAGE;
             // phase A
 #pragma unroll
             for (int x = 0; x < 8; ++x) {
                 mma_one(f0, x);
-                if (x < 6) {
-                    read_one(f1, st_cur, 1, 2 * x);
-                    read_one(f1, st_cur, 1, 2 * x + 1);
+                if (x >= 1 && x < 7) {
+                    read_one(f1, pa_cur, pb_cur, 1, 2 * x - 2);
+                    read_one(f1, pa_cur, pb_cur, 1, 2 * x - 1);
                 }
                 __builtin_amdgcn_sched_barrier(0);
             }
@@ -398,9 +453,9 @@ __global__ __launch_bounds__(NT, 1) void gemm_fp8_dma8_kernel(Problem pb)
 #pragma unroll
             for (int x = 0; x < 8; ++x) {
                 mma_one(f1, x);
-                if (x < 6) {
-                    read_one(f0, st_nxt, 0, 2 * x);
-                    read_one(f0, st_nxt, 0, 2 * x + 1);
+                if (x >= 1 && x < 7) {
+                    read_one(f0, pa_nxt, pb_nxt, 0, 2 * x - 2);
+                    read_one(f0, pa_nxt, pb_nxt, 0, 2 * x - 1);
                 }
                 dma_one(ld_a, ld_b, cur, x);
                 __builtin_amdgcn_sched_barrier(0);
@@ -460,14 +515,19 @@ __global__ __launch_bounds__(NT, 1) void gemm_fp8_dma8_kernel(Problem pb)
                 const int rw = it * 8 + (lane >> 3);
                 staged[it] = *reinterpret_cast<const uint4*>(stg + rw * 128 + (((lane & 7) ^ ((rw >> 1) & 7)) << 4));
             }
+            // rows [rt, rt + 32) of the tile; a pass that lies completely inside the stored range (the common
+            // case, decided per wave) needs no per-lane predicate
+            const bool all_rows = !Problem::kMaskRows || (rt >= td.row_lo && rt + 32 <= td.row_hi);
+            uint16_t* crow = td.c + (int64_t)(rt + (lane >> 3)) * pb.ldc + wn * WTN + (lane & 7) * 8;
+            if (all_rows) {
 #pragma unroll
-            for (int it = 0; it < 4; ++it) {
-                const int trow = rt + it * 8 + (lane >> 3);
-                uint4* dst = reinterpret_cast<uint4*>(td.c + (int64_t)trow * pb.ldc + wn * WTN + (lane & 7) * 8);
-                if constexpr (Problem::kMaskRows) {
-                    if (trow >= td.row_lo && trow < td.row_hi) *dst = staged[it];
-                } else {
-                    *dst = staged[it];
+                for (int it = 0; it < 4; ++it) *reinterpret_cast<uint4*>(crow + (int64_t)(it * 8) * pb.ldc) = staged[it];
+            } else {
+#pragma unroll
+                for (int it = 0; it < 4; ++it) {
+                    const int trow = rt + it * 8 + (lane >> 3);
+                    if (trow >= td.row_lo && trow < td.row_hi)
+                        *reinterpret_cast<uint4*>(crow + (int64_t)(it * 8) * pb.ldc) = staged[it];
                 }
             }
             __builtin_amdgcn_s_waitcnt(0xc07f);  // the reads are done before the next pass overwrites
