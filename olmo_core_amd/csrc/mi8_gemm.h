@@ -32,6 +32,15 @@ __device__ __forceinline__ uint16_t f32_to_bf16_bits(float f)
     return __builtin_bit_cast(uint16_t, h);
 }
 
+// Two floats -> two bf16 (round-to-nearest-even) in one dword, low half first: a single v_cvt_pk_bf16_f32.
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+typedef float f32x2_t __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi)
+{
+    const f32x2_t f = {lo, hi};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(f, bf16x2_t));
+}
+
 // Linear tile index -> tile coordinates: tiles are walked in groups of 8 tile-rows (all columns of the group
 // before the next group) so that tiles with neighbouring indices share A and B panels.
 __device__ __forceinline__ void tile_coords(const GemmArgs& g, int t, int& tm, int& tn)

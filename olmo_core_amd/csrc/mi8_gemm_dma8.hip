@@ -63,7 +63,7 @@ struct DenseProblem {
     GemmArgs g;
     int64_t lda, ldb, ldc;
     static constexpr bool kVecScales = VEC;  // both scales are vectors (per row / per column) or both single
-    static constexpr bool kMaskRows = false, kXcdRanges = true;
+    static constexpr bool kMaskRows = false, kXcdRanges = true, kPeelFirstStep = true;
     using Cache = NoCache;
     __device__ __forceinline__ Cache prepare() const { return Cache{}; }
     __device__ __forceinline__ int total_tiles(const Cache&) const { return g.tiles_m * g.tiles_n; }
@@ -213,7 +213,7 @@ struct GroupedProblem {
     int N, K, tiles_n;
     const float* sa;
     const float* sb;
-    static constexpr bool kVecScales = true, kMaskRows = true, kXcdRanges = true;
+    static constexpr bool kVecScales = true, kMaskRows = true, kXcdRanges = true, kPeelFirstStep = false;
     using Cache = GroupCache;
     __device__ __forceinline__ Cache prepare() const { return build_group_cache<BM>(sizes, E, T); }
     __device__ __forceinline__ int total_tiles(const Cache& c) const
@@ -258,7 +258,7 @@ struct GroupedWgradProblem {
     int N, Kl, tiles_n, tiles_k;
     const float* sa;  // [E, N]
     const float* sb;  // [E, Kl]
-    static constexpr bool kVecScales = true, kMaskRows = false, kXcdRanges = false;
+    static constexpr bool kVecScales = true, kMaskRows = false, kXcdRanges = false, kPeelFirstStep = true;
     using Cache = GroupCache;
     __device__ __forceinline__ Cache prepare() const { return build_group_cache<128>(sizes, E, T); }
     __device__ __forceinline__ int total_tiles(const Cache&) const { return E * tiles_n * tiles_k; }
@@ -404,11 +404,15 @@ __global__ __launch_bounds__(NT, 1) void gemm_fp8_dma8_kernel(Problem pb)
                 for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
     };
     // D' = B . A^T : first MFMA operand is the B fragment (its type code goes to cbsz)
-    auto mma_one = [&](const Frags& f, int x) __attribute__((always_inline)) {
+    // `fresh`: the tile's first touch of this accumulator; the MFMA then takes the constant 0 as its addend, so
+    // the 128 accumulator registers never have to be cleared between tiles
+    auto mma_one = [&](const Frags& f, int x, bool fresh) __attribute__((always_inline)) {
         const int i = x >> 1, j = x & 1;
         const v8i fa = __builtin_shufflevector(f.h[frag_a(i)], f.h[frag_a(i) + 1], 0, 1, 2, 3, 4, 5, 6, 7);
         const v8i fb = __builtin_shufflevector(f.h[frag_b(j)], f.h[frag_b(j) + 1], 0, 1, 2, 3, 4, 5, 6, 7);
-        acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fb, fa, acc[i][j], BLGP_B, CBSZ_A, 0, 0, 0, 0);
+        const v16f zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+        acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fb, fa, fresh ? zero : acc[i][j], BLGP_B, CBSZ_A, 0, 0,
+                                                                     0, 0);
     };
 
     // ---- prologue: stages of steps 0 and 1, fragments of step 0 ----------------------------------------
@@ -421,7 +425,6 @@ __global__ __launch_bounds__(NT, 1) void gemm_fp8_dma8_kernel(Problem pb)
             advance_load_cursor();
         }
     }
-    clear_acc();
     Frags f0, f1;
     __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wave's direct loads have landed
     __syncthreads();
@@ -431,14 +434,17 @@ __global__ __launch_bounds__(NT, 1) void gemm_fp8_dma8_kernel(Problem pb)
     int step = 0;
     for (int cp_tile = 0; cp_tile < my_tiles; ++cp_tile) {
         const TileDesc td = my_tile(cp_tile);
-        for (int kt = 0; kt < td.nk; ++kt, ++step) {
+        // One 128-byte K step.  `fresh`: the tile's first step, whose phase A starts the accumulators from 0.
+        // The first step is written out separately from the loop (not as a branch inside it) so that the two
+        // copies share no hoisted address registers.
+        auto k_step = [&](bool fresh) __attribute__((always_inline)) {
             const int cur = step & 1;
             const uint32_t pa_cur = xa00 + cur * STAGE, pb_cur = xb00 + cur * STAGE;
             const uint32_t pa_nxt = xa00 + (cur ^ 1) * STAGE, pb_nxt = xb00 + (cur ^ 1) * STAGE;
-            // phase A
+            // phase A: its 8 MFMAs touch each of the 8 accumulator tiles once
 #pragma unroll
             for (int x = 0; x < 8; ++x) {
-                mma_one(f0, x);
+                mma_one(f0, x, fresh);
                 if (x >= 1 && x < 7) {
                     read_one(f1, pa_cur, pb_cur, 1, 2 * x - 2);
                     read_one(f1, pa_cur, pb_cur, 1, 2 * x - 1);
@@ -452,7 +458,7 @@ __global__ __launch_bounds__(NT, 1) void gemm_fp8_dma8_kernel(Problem pb)
             // phase B
 #pragma unroll
             for (int x = 0; x < 8; ++x) {
-                mma_one(f1, x);
+                mma_one(f1, x, false);
                 if (x >= 1 && x < 7) {
                     read_one(f0, pa_nxt, pb_nxt, 0, 2 * x - 2);
                     read_one(f0, pa_nxt, pb_nxt, 0, 2 * x - 1);
@@ -461,12 +467,23 @@ __global__ __launch_bounds__(NT, 1) void gemm_fp8_dma8_kernel(Problem pb)
                 __builtin_amdgcn_sched_barrier(0);
             }
             advance_load_cursor();
+            ++step;
+        };
+        if constexpr (Problem::kPeelFirstStep) {
+            if (td.nk > 0) {
+                k_step(true);
+                for (int kt = 1; kt < td.nk; ++kt) k_step(false);
+            }
+        } else {
+            clear_acc();
+            for (int kt = 0; kt < td.nk; ++kt) k_step(false);
         }
 
         // ---- tile finished: epilogue -------------------------------------------------------------------
         // acc[i][j][e] of lane l is C[row = 32 i + l%32][col = 32 j + 8*(e/4) + 4*(l/32) + e%4] of the wave tile.
         // A single scale is inverted with an IEEE division, scale vectors with v_rcp_f32 (exact for the
         // power-of-two scales of the axiswise recipes, within 1 ulp otherwise).
+        if (Problem::kPeelFirstStep && td.nk == 0) clear_acc();  // nothing was accumulated (empty group)
         uint8_t* stg = lds + 2 * STAGE + wave * (32 * WTN * 2);  // wave-private 4 KB: 32 rows x 128 bytes
         const bool zero_tile = td.nk == 0;  // nothing accumulated; the scales may be unset
         float isb[TN][4][4];
@@ -483,10 +500,11 @@ __global__ __launch_bounds__(NT, 1) void gemm_fp8_dma8_kernel(Problem pb)
                 }
         }
         const float isb_scalar = Problem::kVecScales ? 1.0f : 1.0f / td.sb[0];
+        const float isa_scalar = Problem::kVecScales ? 1.0f : 1.0f / td.sa[0];
 #pragma unroll
         for (int i = 0; i < TM; ++i) {
             const int rt = wm * WTM + i * 32;  // first tile row of this pass
-            float mult = Problem::kVecScales ? __builtin_amdgcn_rcpf(td.sa[rt + l32]) : 1.0f / td.sa[0];
+            float mult = Problem::kVecScales ? __builtin_amdgcn_rcpf(td.sa[rt + l32]) : isa_scalar;
             mult = zero_tile ? 0.0f : mult * isb_scalar;
             // 32 rows x 64 bf16 through the wave's staging area: pitch 128 bytes, the 16-byte chunk index XORed
             // with (row >> 1) & 7 so that 16 consecutive rows cover all banks
@@ -502,8 +520,8 @@ __global__ __launch_bounds__(NT, 1) void gemm_fp8_dma8_kernel(Problem pb)
                         if constexpr (Problem::kVecScales) v[e] *= isb[j][q][e];
                     }
                     uint2 o;
-                    o.x = (uint32_t)f32_to_bf16_bits(v[0]) | ((uint32_t)f32_to_bf16_bits(v[1]) << 16);
-                    o.y = (uint32_t)f32_to_bf16_bits(v[2]) | ((uint32_t)f32_to_bf16_bits(v[3]) << 16);
+                    o.x = pack_bf16x2(v[0], v[1]);
+                    o.y = pack_bf16x2(v[2], v[3]);
                     const int chunk = (cw >> 3) ^ ((l32 >> 1) & 7);
                     *reinterpret_cast<uint2*>(stg + l32 * 128 + chunk * 16 + (cw & 4) * 2) = o;
                 }
@@ -533,7 +551,6 @@ __global__ __launch_bounds__(NT, 1) void gemm_fp8_dma8_kernel(Problem pb)
             __builtin_amdgcn_s_waitcnt(0xc07f);  // the reads are done before the next pass overwrites
             __builtin_amdgcn_wave_barrier();
         }
-        clear_acc();
     }
     // direct loads issued for steps past the end must have landed before the LDS allocation is released
     __builtin_amdgcn_s_waitcnt(0x0070);  // vmcnt(0) lgkmcnt(0)
