@@ -306,7 +306,7 @@ def main():
         },
         "pct_fp8_mfma_peak": round(100.0 * tflops / FP8_MFMA_PEAK_TFLOPS, 2),
         "roofline": {
-            "kernel": "gemm_fp8_kernel (9 launches per step, 2*16384*4096*11008 flop each)",
+            "kernel": "gemm_fp8_dma8_kernel (9 launches per step, 2*16384*4096*11008 flop each)",
             "bound": "mfma",
             "achieved": round(achieved, 2),
             "peak": FP8_MFMA_PEAK_TFLOPS,
