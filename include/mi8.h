@@ -74,29 +74,32 @@ int mi8_scale_from_partials(const uint32_t* slots, int32_t n_slots, int fp8_dtyp
  *   scale source: if slots != NULL the scale is reduced from slots[0..n_slots) exactly as
  *   mi8_scale_from_partials does (and written to scale_out[0] if scale_out != NULL);
  *   otherwise it is read from scale_in[0] (device float32).
- *   out   (may be NULL): fp8 [rows, cols], row-major.
+ *   out   (may be NULL): fp8 [rows, ld_out], row-major with row pitch ld_out >= cols, ld_out % 16 == 0;
+ *                        bytes cols..ld_out-1 of a row are not touched.
  *   out_t (may be NULL): fp8 [cols, ld_t], the transposed copy; ld_t >= rows, ld_t % 16 == 0; columns
- *                        rows..ld_t-1 of out_t are written as zero.
- * cols % 16 == 0 is required. */
+ *                        rows..round_up(rows,16)-1 of out_t are written as zero (so that a GEMM may contract
+ *                        over round_up(rows,16)), columns beyond are not touched.
+ * cols % 16 == 0 is required.  The GEMMs accept any operand pitch that is a multiple of 16. */
 int mi8_cast_tensorwise(const void* x, int hp_dtype, int64_t rows, int64_t cols, const uint32_t* slots,
                         int32_t n_slots, const float* scale_in, int fp8_dtype, uint32_t flags, void* out,
-                        void* out_t, int64_t ld_t, float* scale_out, void* stream);
+                        int64_t ld_out, void* out_t, int64_t ld_t, float* scale_out, void* stream);
+
 
 /* ---------------------------------------------------------------------------------------------
  * Axiswise ("rowwise" recipe) dynamic casts: AXISWISE cast configs of the rowwise recipes
  * (reference: AOFloat8LinearRecipe.rowwise / rowwise_with_gw_hp, src/olmo_core/float8/ao.py:100-109).
  * ------------------------------------------------------------------------------------------- */
 
-/* One scale per row (amax over the last axis): out fp8 [rows, cols], scale_out float32 [rows].
- * cols % 16 == 0, cols <= 65536. Single pass over x. */
+/* One scale per row (amax over the last axis): out fp8 [rows, ld_out] (ld_out >= cols, ld_out % 16 == 0),
+ * scale_out float32 [rows].  cols % 16 == 0, cols <= 65536. Single pass over x. */
 int mi8_cast_rowwise(const void* x, int hp_dtype, int64_t rows, int64_t cols, int fp8_dtype, uint32_t flags,
-                     void* out, float* scale_out, void* stream);
+                     void* out, int64_t ld_out, float* scale_out, void* stream);
 
 /* Number of uint32 a column-amax workspace needs for a [rows, cols] input. */
 int64_t mi8_colamax_workspace_slots(int64_t rows, int64_t cols);
 
 /* One scale per column (amax over axis 0), output written TRANSPOSED: out_t fp8 [cols, ld_t] (pad columns
- * rows..ld_t-1 zero), scale_out float32 [cols].  This is the operand layout the grad_weight GEMM and the
+ * rows..round_up(rows,16)-1 zero), scale_out float32 [cols].  This is the operand layout the grad_weight GEMM and the
  * axiswise grad_input GEMM consume.  workspace: mi8_colamax_workspace_slots(rows, cols) uint32.
  * Two kernels: column amax, then cast + transpose. */
 int mi8_cast_colwise_t(const void* x, int hp_dtype, int64_t rows, int64_t cols, int fp8_dtype, uint32_t flags,

@@ -34,10 +34,13 @@ _SIGNATURES = {
     "mi8_scale_from_partials": (c_int, [c_void_p, c_int32, c_int, c_uint32, c_void_p, c_void_p]),
     "mi8_cast_tensorwise": (
         c_int,
-        [c_void_p, c_int, c_int64, c_int64, c_void_p, c_int32, c_void_p, c_int, c_uint32, c_void_p, c_void_p,
-         c_int64, c_void_p, c_void_p],
+        [c_void_p, c_int, c_int64, c_int64, c_void_p, c_int32, c_void_p, c_int, c_uint32, c_void_p, c_int64,
+         c_void_p, c_int64, c_void_p, c_void_p],
     ),
-    "mi8_cast_rowwise": (c_int, [c_void_p, c_int, c_int64, c_int64, c_int, c_uint32, c_void_p, c_void_p, c_void_p]),
+    "mi8_cast_rowwise": (
+        c_int,
+        [c_void_p, c_int, c_int64, c_int64, c_int, c_uint32, c_void_p, c_int64, c_void_p, c_void_p],
+    ),
     "mi8_colamax_workspace_slots": (c_int64, [c_int64, c_int64]),
     "mi8_cast_colwise_t": (
         c_int,

@@ -121,7 +121,8 @@ struct TileCastArgs {
     int n_slots;
     const float* scale_in;
     bool pow2;
-    uint8_t* out;    // [rows, cols] or null
+    uint8_t* out;    // [rows, ld_out] or null
+    int64_t ld_out;
     uint8_t* out_t;  // [cols, ld_t] or null
     int64_t ld_t;
     float* scale_out;  // scalar modes: [1]; per-column mode: [cols]; may be null
@@ -144,7 +145,7 @@ __device__ __forceinline__ int tile_lds_chunk(int col, int part /* 0..7: which 1
 // chunks at or beyond dst_end are not written.
 template <int HP, int FP8, bool SW>
 __device__ __forceinline__ void tile_cast_body(const void* x, int64_t row_end, int64_t cols, int64_t row0, int64_t col0,
-                                               const float (&sc)[8], uint8_t* out, uint8_t* out_t, int64_t ld_t,
+                                               const float (&sc)[8], uint8_t* out, int64_t ld_out, uint8_t* out_t, int64_t ld_t,
                                                int64_t dst0, int64_t dst_end, uint32_t* lds_t)
 {
     const int tid = threadIdx.x;
@@ -175,7 +176,7 @@ __device__ __forceinline__ void tile_cast_body(const void* x, int64_t row_end, i
             lo[j] = quant4<FP8, SW>(v[0], v[1], v[2], v[3], sc[0], sc[1], sc[2], sc[3]);
             hi[j] = quant4<FP8, SW>(v[4], v[5], v[6], v[7], sc[4], sc[5], sc[6], sc[7]);
             if (!ok) lo[j] = hi[j] = 0;  // padding is zero bytes whatever the scale is (0 * NaN is NaN)
-            if (out && ok) *reinterpret_cast<uint2*>(out + r * cols + c8) = make_uint2(lo[j], hi[j]);
+            if (out && ok) *reinterpret_cast<uint2*>(out + r * ld_out + c8) = make_uint2(lo[j], hi[j]);
         }
         if (out_t) {
             uint32_t t[8];
@@ -250,7 +251,8 @@ __global__ __launch_bounds__(kThreads) void tile_cast_kernel(TileCastArgs a)
         for (int i = 0; i < 8; ++i) sc[i] = s;
     }
 
-    tile_cast_body<HP, FP8, SW>(a.x, a.rows, a.cols, row0, col0, sc, a.out, a.out_t, a.ld_t, row0, a.ld_t, lds_t);
+    tile_cast_body<HP, FP8, SW>(a.x, a.rows, a.cols, row0, col0, sc, a.out, a.ld_out, a.out_t, a.ld_t, row0,
+                                (a.rows + 15) / 16 * 16, lds_t);
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -331,7 +333,7 @@ __global__ __launch_bounds__(kThreads) void colamax_kernel(const void* __restric
 template <int HP, int FP8, bool SW, int TPR /* 64 or 256 */, int NV /* 8-element vectors per lane */>
 __global__ __launch_bounds__(kThreads) void rowwise_cast_kernel(const void* __restrict__ x, int64_t rows,
                                                                 int64_t cols, bool pow2,
-                                                                uint8_t* __restrict__ out,
+                                                                uint8_t* __restrict__ out, int64_t ld_out,
                                                                 float* __restrict__ scale_out)
 {
     __shared__ uint32_t smem[4];
@@ -357,7 +359,7 @@ __global__ __launch_bounds__(kThreads) void rowwise_cast_kernel(const void* __re
         m = block_umax(m, smem);
     const float s = scale_from_amax_bits<FP8>(m, pow2);
     if (row_ok && lane == 0) scale_out[row] = s;
-    uint8_t* orow = out + row * cols;
+    uint8_t* orow = out + row * ld_out;
 #pragma unroll
     for (int i = 0; i < NV; ++i) {
         const int v = lane + TPR * i;
@@ -487,7 +489,7 @@ __global__ __launch_bounds__(kThreads) void grouped_tile_cast_kernel(GroupedCast
 #pragma unroll
     for (int i = 0; i < 8; ++i) sc[i] = s_scale[8 * cl + i];
     const int64_t dst0 = (int64_t)kTile * blockIdx.y;
-    tile_cast_body<HP, FP8, SW>(a.x, row_end, a.cols, row0, col0, sc, nullptr, a.out_t, a.ld_t, dst0, a.ld_t, lds_t);
+    tile_cast_body<HP, FP8, SW>(a.x, row_end, a.cols, row0, col0, sc, nullptr, 0, a.out_t, a.ld_t, dst0, a.ld_t, lds_t);
 }
 
 // ---- dispatch helpers ------------------------------------------------------------------------------
@@ -526,13 +528,13 @@ void dispatch_tile_cast(int hp, int fp8, bool sw, int mode, const TileCastArgs& 
 }
 
 template <int HP, int FP8, bool SW>
-int launch_rowwise(const void* x, int64_t rows, int64_t cols, bool pow2, uint8_t* out, float* scale_out,
+int launch_rowwise(const void* x, int64_t rows, int64_t cols, bool pow2, uint8_t* out, int64_t ld_out, float* scale_out,
                    hipStream_t st)
 {
     const int64_t nvec = cols / 8;
 #define MI8_RW(TPR_, NV_)                                                                                    \
     hipLaunchKernelGGL((rowwise_cast_kernel<HP, FP8, SW, TPR_, NV_>), dim3((unsigned)ceil_div(rows, kThreads / TPR_)), \
-                       dim3(kThreads), 0, st, x, rows, cols, pow2, out, scale_out)
+                       dim3(kThreads), 0, st, x, rows, cols, pow2, out, ld_out, scale_out)
     if (nvec <= 64 * 2) { MI8_RW(64, 2); }
     else if (nvec <= 64 * 4) { MI8_RW(64, 4); }
     else if (nvec <= 64 * 8) { MI8_RW(64, 8); }
@@ -613,7 +615,7 @@ extern "C" int mi8_scale_from_partials(const uint32_t* slots, int32_t n_slots, i
 
 extern "C" int mi8_cast_tensorwise(const void* x, int hp_dtype, int64_t rows, int64_t cols, const uint32_t* slots,
                                    int32_t n_slots, const float* scale_in, int fp8_dtype, uint32_t flags, void* out,
-                                   void* out_t, int64_t ld_t, float* scale_out, void* stream)
+                                   int64_t ld_out, void* out_t, int64_t ld_t, float* scale_out, void* stream)
 {
     MI8_REQUIRE(x, MI8_ERR_ARG, "mi8_cast_tensorwise: x is null");
     MI8_REQUIRE(out || out_t, MI8_ERR_ARG, "mi8_cast_tensorwise: no output requested");
@@ -628,21 +630,25 @@ extern "C" int mi8_cast_tensorwise(const void* x, int hp_dtype, int64_t rows, in
                 (long long)cols);
     MI8_REQUIRE(aligned16(x) && aligned16(out) && aligned16(out_t), MI8_ERR_UNSUPPORTED,
                 "mi8_cast_tensorwise: pointers must be 16-byte aligned");
+    if (out)
+        MI8_REQUIRE(ld_out >= cols && ld_out % 16 == 0, MI8_ERR_UNSUPPORTED,
+                    "mi8_cast_tensorwise: ld_out (%lld) must be a multiple of 16 and at least cols", (long long)ld_out);
     if (out_t)
-        MI8_REQUIRE(ld_t >= rows && ld_t % 16 == 0 && ld_t <= round_up(rows, kTile), MI8_ERR_UNSUPPORTED,
-                    "mi8_cast_tensorwise: ld_t (%lld) must be a multiple of 16 in [rows, round_up(rows,128)]",
-                    (long long)ld_t);
+        MI8_REQUIRE(ld_t >= rows && ld_t % 16 == 0, MI8_ERR_UNSUPPORTED,
+                    "mi8_cast_tensorwise: ld_t (%lld) must be a multiple of 16 and at least rows", (long long)ld_t);
     TileCastArgs a{x, rows, cols, slots, n_slots, scale_in, (flags & MI8_FLAG_POW2_SCALE) != 0,
-                   (uint8_t*)out, (uint8_t*)out_t, ld_t, scale_out};
+                   (uint8_t*)out, ld_out, (uint8_t*)out_t, ld_t, scale_out};
     dispatch_tile_cast(hp_dtype, fp8_dtype, (flags & MI8_FLAG_SW_CVT) != 0, slots ? kScalarFromSlots : kScalarFromPtr,
                        a, (hipStream_t)stream);
     return launch_status("mi8_cast_tensorwise");
 }
 
 extern "C" int mi8_cast_rowwise(const void* x, int hp_dtype, int64_t rows, int64_t cols, int fp8_dtype,
-                                uint32_t flags, void* out, float* scale_out, void* stream)
+                                uint32_t flags, void* out, int64_t ld_out, float* scale_out, void* stream)
 {
     MI8_REQUIRE(x && out && scale_out, MI8_ERR_ARG, "mi8_cast_rowwise: null pointer");
+    MI8_REQUIRE(ld_out >= cols && ld_out % 16 == 0, MI8_ERR_UNSUPPORTED,
+                "mi8_cast_rowwise: ld_out (%lld) must be a multiple of 16 and at least cols", (long long)ld_out);
     MI8_REQUIRE(valid_hp(hp_dtype) && valid_fp8(fp8_dtype), MI8_ERR_ARG, "mi8_cast_rowwise: unknown dtype");
     MI8_REQUIRE(rows > 0 && cols > 0, MI8_ERR_ARG, "mi8_cast_rowwise: empty input");
     MI8_REQUIRE(cols % 16 == 0 && cols <= 65536, MI8_ERR_UNSUPPORTED,
@@ -652,8 +658,8 @@ extern "C" int mi8_cast_rowwise(const void* x, int hp_dtype, int64_t rows, int64
     hipStream_t st = (hipStream_t)stream;
     int rc;
 #define MI8_ROW(HP_, FP8_) \
-    rc = sw ? launch_rowwise<HP_, FP8_, true>(x, rows, cols, pow2, (uint8_t*)out, scale_out, st) \
-            : launch_rowwise<HP_, FP8_, false>(x, rows, cols, pow2, (uint8_t*)out, scale_out, st)
+    rc = sw ? launch_rowwise<HP_, FP8_, true>(x, rows, cols, pow2, (uint8_t*)out, ld_out, scale_out, st) \
+            : launch_rowwise<HP_, FP8_, false>(x, rows, cols, pow2, (uint8_t*)out, ld_out, scale_out, st)
     if (hp_dtype == MI8_BF16) {
         if (fp8_dtype == MI8_E4M3) { MI8_ROW(MI8_BF16, MI8_E4M3); } else { MI8_ROW(MI8_BF16, MI8_E5M2); }
     } else {
@@ -679,8 +685,8 @@ extern "C" int mi8_cast_colwise_t(const void* x, int hp_dtype, int64_t rows, int
     MI8_REQUIRE(rows > 0 && cols > 0, MI8_ERR_ARG, "mi8_cast_colwise_t: empty input");
     MI8_REQUIRE(cols % 16 == 0, MI8_ERR_UNSUPPORTED, "mi8_cast_colwise_t: cols (%lld) must be a multiple of 16",
                 (long long)cols);
-    MI8_REQUIRE(ld_t >= rows && ld_t % 16 == 0 && ld_t <= round_up(rows, kTile), MI8_ERR_UNSUPPORTED,
-                "mi8_cast_colwise_t: ld_t (%lld) must be a multiple of 16 in [rows, round_up(rows,128)]", (long long)ld_t);
+    MI8_REQUIRE(ld_t >= rows && ld_t % 16 == 0, MI8_ERR_UNSUPPORTED,
+                "mi8_cast_colwise_t: ld_t (%lld) must be a multiple of 16 and at least rows", (long long)ld_t);
     MI8_REQUIRE(aligned16(x) && aligned16(out_t), MI8_ERR_UNSUPPORTED,
                 "mi8_cast_colwise_t: pointers must be 16-byte aligned");
     hipStream_t st = (hipStream_t)stream;
@@ -694,7 +700,7 @@ extern "C" int mi8_cast_colwise_t(const void* x, int hp_dtype, int64_t rows, int
     int rc = launch_status("mi8_cast_colwise_t(amax)");
     if (rc != MI8_OK) return rc;
     TileCastArgs a{x, rows, cols, workspace, n_chunks, nullptr, (flags & MI8_FLAG_POW2_SCALE) != 0,
-                   nullptr, (uint8_t*)out_t, ld_t, scale_out};
+                   nullptr, 0, (uint8_t*)out_t, ld_t, scale_out};
     dispatch_tile_cast(hp_dtype, fp8_dtype, (flags & MI8_FLAG_SW_CVT) != 0, kPerColumnFromWorkspace, a, st);
     return launch_status("mi8_cast_colwise_t(cast)");
 }

@@ -42,7 +42,8 @@ __device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi)
 }
 
 // Linear tile index -> tile coordinates: tiles are walked in groups of 8 tile-rows (all columns of the group
-// before the next group) so that tiles with neighbouring indices share A and B panels.
+// before the next group, walked from a group-dependent start column) so that tiles with neighbouring indices
+// share A and B panels.
 __device__ __forceinline__ void tile_coords(const GemmArgs& g, int t, int& tm, int& tn)
 {
     constexpr int GROUP = 8;
@@ -51,7 +52,9 @@ __device__ __forceinline__ void tile_coords(const GemmArgs& g, int t, int& tm, i
     const int gsz = (g.tiles_m - first_m < GROUP) ? g.tiles_m - first_m : GROUP;
     const int in = t % span;
     tm = first_m + in % gsz;
-    tn = in / gsz;
+    // Every group starts its column sweep somewhere else: groups that run at the same time on different XCDs
+    // (one group per XCD when tiles_m = 64) would otherwise request the same B panels from memory in lockstep.
+    tn = (in / gsz + (t / span) * ((g.tiles_n + GROUP - 1) / GROUP)) % g.tiles_n;
 }
 
 // Workgroup id -> output tile.  Consecutive workgroup ids are spread round-robin over the 8 XCDs, each with

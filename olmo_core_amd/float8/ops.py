@@ -87,6 +87,17 @@ def tensor_to_scale(x: torch.Tensor, fp8_dtype: torch.dtype, pow2: bool = False)
     return scale_from_partials(slots, used, fp8_dtype, pow2)[0]
 
 
+def _operand(shape: Tuple[int, int], fp8_dtype: torch.dtype, device, pitch: Optional[int] = None) -> torch.Tensor:
+    """Uninitialised fp8 ``[rows, k]`` GEMM operand; with ``pitch > k`` a view of a wider buffer (the kernels take
+    any row pitch that is a multiple of 16)."""
+    rows, k = shape
+    if pitch is None or pitch == k:
+        return torch.empty((rows, k), dtype=fp8_dtype, device=device)
+    if pitch < k or pitch % 16:
+        raise ValueError(f"operand pitch {pitch} must be a multiple of 16 and at least {k}")
+    return torch.empty((rows, pitch), dtype=fp8_dtype, device=device)[:, :k]
+
+
 def cast_tensorwise(
     x: torch.Tensor,
     fp8_dtype: torch.dtype,
@@ -96,6 +107,8 @@ def cast_tensorwise(
     want_transposed: bool = False,
     slots: Optional[Tuple[torch.Tensor, int]] = None,
     scale: Optional[torch.Tensor] = None,
+    pitch: Optional[int] = None,
+    pitch_t: Optional[int] = None,
 ) -> Tuple[Optional[torch.Tensor], Optional[torch.Tensor], torch.Tensor]:
     """
     Quantise ``x [rows, cols]`` with one scale.  Returns ``(q, q_t, scale)``: ``q`` fp8 ``[rows, cols]``,
@@ -107,9 +120,8 @@ def cast_tensorwise(
     dev = x.device
     if scale is None and slots is None:
         slots = amax_partials(x)
-    q = torch.empty((rows, cols), dtype=fp8_dtype, device=dev) if want_rowmajor else None
-    ld_t = pad16(rows)
-    q_t = torch.empty((cols, ld_t), dtype=fp8_dtype, device=dev) if want_transposed else None
+    q = _operand((rows, cols), fp8_dtype, dev, pitch) if want_rowmajor else None
+    q_t = _operand((cols, pad16(rows)), fp8_dtype, dev, pitch_t) if want_transposed else None
     scale_out = torch.empty(1, dtype=torch.float32, device=dev)
     if scale is not None:
         scale = scale.reshape(1).to(torch.float32)
@@ -119,8 +131,8 @@ def cast_tensorwise(
             slots[0].data_ptr() if scale is None else None, slots[1] if scale is None else 0,
             scale.data_ptr() if scale is not None else None,
             _FP8_CODE[fp8_dtype], _flags(pow2),
-            q.data_ptr() if q is not None else None,
-            q_t.data_ptr() if q_t is not None else None, ld_t,
+            q.data_ptr() if q is not None else None, q.stride(0) if q is not None else 0,
+            q_t.data_ptr() if q_t is not None else None, q_t.stride(0) if q_t is not None else 0,
             scale_out.data_ptr(), _stream(x),
         ),
         "mi8_cast_tensorwise",
@@ -128,34 +140,37 @@ def cast_tensorwise(
     return q, q_t, scale_out
 
 
-def cast_rowwise(x: torch.Tensor, fp8_dtype: torch.dtype, *, pow2: bool = False) -> Tuple[torch.Tensor, torch.Tensor]:
+def cast_rowwise(
+    x: torch.Tensor, fp8_dtype: torch.dtype, *, pow2: bool = False, pitch: Optional[int] = None
+) -> Tuple[torch.Tensor, torch.Tensor]:
     """One scale per row: returns (q fp8 [rows, cols], scale float32 [rows])."""
     x = _hp2d(x, "cast_rowwise")
     rows, cols = x.shape
-    q = torch.empty((rows, cols), dtype=fp8_dtype, device=x.device)
+    q = _operand((rows, cols), fp8_dtype, x.device, pitch)
     s = torch.empty(rows, dtype=torch.float32, device=x.device)
     _C.check(
         _C.lib().mi8_cast_rowwise(
             x.data_ptr(), _HP_CODE[x.dtype], rows, cols, _FP8_CODE[fp8_dtype], _flags(pow2), q.data_ptr(),
-            s.data_ptr(), _stream(x),
+            q.stride(0), s.data_ptr(), _stream(x),
         ),
         "mi8_cast_rowwise",
     )
     return q, s
 
 
-def cast_colwise_t(x: torch.Tensor, fp8_dtype: torch.dtype, *, pow2: bool = False) -> Tuple[torch.Tensor, torch.Tensor]:
+def cast_colwise_t(
+    x: torch.Tensor, fp8_dtype: torch.dtype, *, pow2: bool = False, pitch_t: Optional[int] = None
+) -> Tuple[torch.Tensor, torch.Tensor]:
     """One scale per column, transposed output: returns (q_t fp8 [cols, pad16(rows)], scale float32 [cols])."""
     x = _hp2d(x, "cast_colwise_t")
     rows, cols = x.shape
-    ld_t = pad16(rows)
-    q_t = torch.empty((cols, ld_t), dtype=fp8_dtype, device=x.device)
+    q_t = _operand((cols, pad16(rows)), fp8_dtype, x.device, pitch_t)
     s = torch.empty(cols, dtype=torch.float32, device=x.device)
     ws = torch.empty(_C.lib().mi8_colamax_workspace_slots(rows, cols), dtype=torch.int32, device=x.device)
     _C.check(
         _C.lib().mi8_cast_colwise_t(
             x.data_ptr(), _HP_CODE[x.dtype], rows, cols, _FP8_CODE[fp8_dtype], _flags(pow2), ws.data_ptr(),
-            q_t.data_ptr(), ld_t, s.data_ptr(), _stream(x),
+            q_t.data_ptr(), q_t.stride(0), s.data_ptr(), _stream(x),
         ),
         "mi8_cast_colwise_t",
     )

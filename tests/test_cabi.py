@@ -41,7 +41,7 @@ def test_host_only_entry_points():
 
 def test_argument_validation_happens_before_any_gpu_call():
     L = _C.lib()
-    assert L.mi8_cast_rowwise(None, 0, 4, 16, 0, 0, None, None, None) == -1
+    assert L.mi8_cast_rowwise(None, 0, 4, 16, 0, 0, None, 16, None, None) == -1
     assert "null" in _C.last_error()
     assert L.mi8_gemm_fp8(None, 0, 16, None, 0, 16, 1, 1, 16, None, 0, None, 0, None, 0, 16, -1, None) == -1
     with pytest.raises(Exception):

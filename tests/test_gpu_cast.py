@@ -185,6 +185,36 @@ def test_colwise_transposed(dev, shape, pow2, cvt_mode):
             assert int(u8(q_t[:, rows:]).max()) == 0
 
 
+@pytest.mark.parametrize("shape", [(100, 272), (256, 4096), (1000, 144)], ids=lambda s: f"{s[0]}x{s[1]}")
+def test_operand_pitches(dev, shape):
+    """Outputs with a row pitch wider than the row: same bytes in the view, nothing written outside it, and a GEMM
+    on the padded operands equal to the GEMM on the packed ones."""
+    rows, cols = shape
+    x = seeded(shape, seed=rows + 11, std=0.3)
+    xd = x.to(dev)
+    ref_q, ref_s = O.cast(x, E4M3, O.TENSORWISE, None, False)
+    q, q_t, s = ops.cast_tensorwise(xd, E4M3, want_transposed=True, pitch=cols + 128, pitch_t=ops.pad16(rows) + 272)
+    assert q.stride(0) == cols + 128 and q_t.stride(0) == ops.pad16(rows) + 272
+    assert_scale_equal(s, ref_s)
+    assert_bytes_equal(q, ref_q, what="row-major view")
+    assert_bytes_equal(q_t[:, :rows], ref_q.t(), what="transposed view")
+    if q_t.shape[1] > rows:
+        assert int(u8(q_t[:, rows:]).max()) == 0
+    ref_q, ref_s = O.cast(x, E4M3, O.AXISWISE, -1, True)
+    qr, sr = ops.cast_rowwise(xd, E4M3, pow2=True, pitch=cols + 16)
+    assert_scale_equal(sr, ref_s)
+    assert_bytes_equal(qr, ref_q, what="rowwise view")
+    ref_q, ref_s = O.cast(x, E4M3, O.AXISWISE, 0, True)
+    qc, sc = ops.cast_colwise_t(xd, E4M3, pow2=True, pitch_t=ops.pad16(rows) + 128)
+    assert_scale_equal(sc, ref_s)
+    assert_bytes_equal(qc[:, :rows], ref_q.t(), what="colwise view")
+    # the GEMMs take the pitch from the view
+    packed, _, _ = ops.cast_tensorwise(xd, E4M3)
+    w = seeded((256, cols), seed=5, std=0.1).to(E4M3).to(dev)
+    one = torch.ones(1, device=dev)
+    assert torch.equal(ops.gemm_fp8(q, one, w, one), ops.gemm_fp8(packed, one, w, one))
+
+
 def test_colwise_float32_input(dev):
     g = torch.Generator().manual_seed(8)
     x = torch.randn(300, 160, generator=g)
