@@ -38,7 +38,12 @@ typedef enum mi8_status {
 typedef enum mi8_fp8 { MI8_E4M3 = 0 /* float8_e4m3fn, max 448 */, MI8_E5M2 = 1 /* float8_e5m2, max 57344 */ } mi8_fp8;
 
 /* high-precision element types accepted by the casts (src/olmo_core/config.py:370-372) */
-typedef enum mi8_hp { MI8_BF16 = 0, MI8_F32 = 1 } mi8_hp;
+typedef enum mi8_hp {
+    MI8_BF16 = 0,
+    MI8_F32 = 1,
+    MI8_F16 = 2,  /* token-permutation entry points only */
+    MI8_RAW8 = 3  /* opaque 1-byte elements (fp8 rows): unweighted permutation only */
+} mi8_hp;
 
 /* flags shared by the cast entry points */
 #define MI8_FLAG_POW2_SCALE 1u /* round every scale down to a power of two (ao.py:167 round_scales_to_power_of_2) */
@@ -171,6 +176,54 @@ int mi8_grouped_wgrad_fp8(const void* a_t, int a_dtype, const void* b_t, int b_d
 int mi8_swiglu_fwd(const void* x1, const void* x3, void* h, int64_t n, uint32_t* slots_h, void* stream);
 int mi8_swiglu_bwd(const void* x1, const void* x3, const void* gh, void* g1, void* g3, int64_t n,
                    uint32_t* slots_g1, uint32_t* slots_g3, void* stream);
+
+/* ---------------------------------------------------------------------------------------------
+ * Token permutation around the expert GEMMs of a mixture-of-experts layer.  These replace the copy kernels of
+ * src/olmo_core/kernels/moe.py (gather :101-139, padded_scatter / scatter :142-192, scatter_wgrad :251-298,
+ * binned_gather :377-406, binned_scatter :409-441, binned_scatter_wgrad :512-537), which the autograd functions
+ * of src/olmo_core/ops/moe.py:26-205 call.
+ *
+ *   tokens, hidden : x is [tokens, hidden]; every token has top_k slots, slot s belongs to token s / top_k.
+ *   indices        : int32 [tokens * top_k], the slot held by each row of the expert-sorted side
+ *                    (argsort of the flattened expert assignment, ops/moe.py / parallel_mlp.py:102-125).
+ *   weights        : [tokens * top_k] of w_dtype (MI8_BF16 / MI8_F16 / MI8_F32) indexed by slot, or NULL.
+ *   bins           : int32 [experts], inclusive prefix sums of the tokens per expert (binned forms).
+ * Products are formed in float32 and rounded once to the element type, as the reference kernels do.  Rows are
+ * moved with 16-byte accesses when hidden * element size is a multiple of 16 and the buffers are 16-byte
+ * aligned, element by element otherwise.  An index outside [0, tokens * top_k) is treated as a dropped token.
+ * ------------------------------------------------------------------------------------------- */
+
+/* out[i, :] = x[indices[i] / top_k, :] * weights[indices[i]]           out: [tokens * top_k, hidden] */
+int mi8_moe_gather(const void* x, int dtype, int64_t tokens, int64_t hidden, const int32_t* indices,
+                   const void* weights, int w_dtype, int32_t top_k, void* out, void* stream);
+
+/* out[e, j, :] = the j-th token row of expert e (scaled), zero rows beyond the expert's token count; tokens
+ * beyond `capacity` are dropped.                                          out: [experts, capacity, hidden] */
+int mi8_moe_binned_gather(const void* x, int dtype, int64_t tokens, int64_t hidden, const int32_t* indices,
+                          const void* weights, int w_dtype, const int32_t* bins, int32_t experts, int64_t capacity,
+                          int32_t top_k, void* out, void* stream);
+
+/* out[t, :] = sum over the top_k slots s of token t of round(x[row holding s, :] * weights[s]), summed in float32
+ * in slot order and rounded once (top_k == 1: a pure move).  x: [tokens * top_k, hidden], out: [tokens, hidden].
+ * inverse_workspace: int32 [tokens * top_k], overwritten. */
+int mi8_moe_scatter(const void* x, int dtype, int64_t tokens, int64_t hidden, const int32_t* indices,
+                    const void* weights, int w_dtype, int32_t top_k, int32_t* inverse_workspace, void* out,
+                    void* stream);
+
+/* The same from the binned layout x: [experts, capacity, hidden]; dropped tokens contribute zero. */
+int mi8_moe_binned_scatter(const void* x, int dtype, int64_t tokens, int64_t hidden, const int32_t* indices,
+                           const void* weights, int w_dtype, const int32_t* bins, int32_t experts, int64_t capacity,
+                           int32_t top_k, int32_t* inverse_workspace, void* out, void* stream);
+
+/* Gradient of the scatter weights: out[indices[i]] = dot(x[i, :], grad[indices[i] / top_k, :]) accumulated in
+ * float32.  x: [tokens * top_k, hidden], grad: [tokens, hidden], out: [tokens * top_k] of dtype. */
+int mi8_moe_scatter_wgrad(const void* x, const void* grad, int dtype, int64_t tokens, int64_t hidden,
+                          const int32_t* indices, int32_t top_k, void* out, void* stream);
+
+/* The same from the binned layout; slots of dropped tokens get zero. */
+int mi8_moe_binned_scatter_wgrad(const void* x, const void* grad, int dtype, int64_t tokens, int64_t hidden,
+                                 const int32_t* indices, const int32_t* bins, int32_t experts, int64_t capacity,
+                                 int32_t top_k, void* out, void* stream);
 
 #ifdef __cplusplus
 }

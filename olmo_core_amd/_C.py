@@ -20,7 +20,7 @@ import os
 LIB_PATH = Path(os.environ.get("MI8_LIBRARY") or (Path(__file__).resolve().parent / "lib" / "libmi8.so"))
 
 MI8_E4M3, MI8_E5M2 = 0, 1
-MI8_BF16, MI8_F32 = 0, 1
+MI8_BF16, MI8_F32, MI8_F16, MI8_RAW8 = 0, 1, 2, 3
 FLAG_POW2_SCALE = 1
 FLAG_SW_CVT = 2
 AMAX_SLOTS = 2048
@@ -57,6 +57,32 @@ _SIGNATURES = {
     "mi8_swiglu_bwd": (
         c_int,
         [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_void_p, c_void_p, c_void_p],
+    ),
+    "mi8_moe_gather": (
+        c_int,
+        [c_void_p, c_int, c_int64, c_int64, c_void_p, c_void_p, c_int, c_int32, c_void_p, c_void_p],
+    ),
+    "mi8_moe_binned_gather": (
+        c_int,
+        [c_void_p, c_int, c_int64, c_int64, c_void_p, c_void_p, c_int, c_void_p, c_int32, c_int64, c_int32, c_void_p,
+         c_void_p],
+    ),
+    "mi8_moe_scatter": (
+        c_int,
+        [c_void_p, c_int, c_int64, c_int64, c_void_p, c_void_p, c_int, c_int32, c_void_p, c_void_p, c_void_p],
+    ),
+    "mi8_moe_binned_scatter": (
+        c_int,
+        [c_void_p, c_int, c_int64, c_int64, c_void_p, c_void_p, c_int, c_void_p, c_int32, c_int64, c_int32, c_void_p,
+         c_void_p, c_void_p],
+    ),
+    "mi8_moe_scatter_wgrad": (
+        c_int,
+        [c_void_p, c_void_p, c_int, c_int64, c_int64, c_void_p, c_int32, c_void_p, c_void_p],
+    ),
+    "mi8_moe_binned_scatter_wgrad": (
+        c_int,
+        [c_void_p, c_void_p, c_int, c_int64, c_int64, c_void_p, c_void_p, c_int32, c_int64, c_int32, c_void_p, c_void_p],
     ),
     "mi8_grouped_padded_rows": (c_int64, [c_int64, c_int32]),
     "mi8_grouped_cast_colwise_t": (
