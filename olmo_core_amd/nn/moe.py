@@ -137,3 +137,66 @@ class DroplessMoEMLP(nn.Module):
             x2 = x2.to(torch.bfloat16)
         y = float8_dropless_mlp(x2, self.w1, self.w2, self.w3, batch_size_per_expert, self.num_experts)
         return y.reshape(*lead, self.d_model).to(x.dtype)
+
+
+class ParallelDroplessMLP(nn.Module):
+    """
+    Routing wrapper around :class:`DroplessMoEMLP`: sorts the token slots by expert, gathers the rows, runs the
+    experts and scatters the weighted results back (reference ``ParallelDroplessMLP`` /
+    ``ParallelMLPBase.forward``, ``src/olmo_core/nn/moe/parallel_mlp.py:102-183``, ``:634-666``, ``:851-871``).
+    Single-device path only: expert parallelism needs more than one GPU.
+    """
+
+    def __init__(self, *, mlp: DroplessMoEMLP, top_k: int):
+        super().__init__()
+        self.mlp = mlp
+        self.top_k = top_k
+
+    @property
+    def d_model(self) -> int:
+        return self.mlp.d_model
+
+    @property
+    def num_experts(self) -> int:
+        return self.mlp.num_experts
+
+    def apply_ep(self, *args, **kwargs):
+        raise NotImplementedError("expert parallelism is outside the single-GPU scope of this build")
+
+    def indices_and_bins(self, expert_indices: torch.Tensor, batch_size_per_expert: torch.Tensor):
+        """``(indices, bin_ids, bins)``: argsort of the flattened expert assignment, the sorted expert ids and
+        the inclusive prefix sums of the per-expert counts (all int32)."""
+        bin_ids, indices = torch.sort(expert_indices.int())
+        bins = torch.cumsum(batch_size_per_expert, 0).to(torch.int32)
+        return indices.int(), bin_ids, bins
+
+    def forward(self, x, expert_weights, expert_indices, batch_size_per_expert):
+        """
+        :param x: ``(N, d_model)`` (any leading shape).
+        :param expert_weights: ``(N, top_k)`` router weights.
+        :param expert_indices: ``(N, top_k)`` expert ids.
+        :param batch_size_per_expert: ``(num_experts,)`` token slots per expert.
+        :returns: the output with the shape of ``x``.
+        """
+        in_shape = x.size()
+        x = x.view(-1, x.shape[-1])
+        expert_weights = expert_weights.flatten()
+        expert_indices = expert_indices.flatten()
+        with torch.no_grad():
+            indices, bin_ids, bins = self.indices_and_bins(expert_indices, batch_size_per_expert)
+        out = self.forward_once(x, expert_weights=expert_weights, expert_indices=expert_indices, indices=indices,
+                                bin_ids=bin_ids, bins=bins, batch_size_per_expert=batch_size_per_expert)
+        return out.view(in_shape)
+
+    def forward_once(self, x, *, expert_weights, expert_indices, indices, bin_ids, bins, batch_size_per_expert):
+        del expert_indices
+        return self.permute_and_compute(x, batch_size_per_expert=batch_size_per_expert, indices=indices,
+                                        bin_ids=bin_ids, expert_weights=expert_weights, bins=bins, top_k=self.top_k)
+
+    def permute_and_compute(self, x, *, batch_size_per_expert, indices, bin_ids, expert_weights, bins, top_k: int):
+        from ..ops import moe as moe_ops
+
+        x = x.view(-1, x.shape[-1])
+        x = moe_ops.gather(x, indices, bin_ids, bins, top_k)
+        x = self.mlp(x, batch_size_per_expert)
+        return moe_ops.scatter(x, indices, bin_ids, expert_weights, bins, top_k)

@@ -5,11 +5,12 @@ import torch
 
 from helpers import E4M3, assert_bytes_equal, assert_gemm_close, assert_scale_equal, gemm_errors, seeded, u8
 from oracle import float8_oracle as O
+from oracle import moe_oracle as MO
 
 pytestmark = pytest.mark.gpu
 
 from olmo_core_amd.float8 import ops  # noqa: E402
-from olmo_core_amd.nn import DroplessMoEMLP  # noqa: E402
+from olmo_core_amd.nn import DroplessMoEMLP, ParallelDroplessMLP  # noqa: E402
 
 SIZE_CASES = [
     [3, 2],
@@ -221,3 +222,51 @@ def test_dropless_mlp_against_oracle(dev, sizes, dims):
         if m == 0:
             assert torch.count_nonzero(mlp.w1.grad.view(E, H, D)[e]) == 0
             assert torch.count_nonzero(mlp.w2.grad.view(E, H, D)[e]) == 0
+
+
+@pytest.mark.parametrize("tokens,top_k", [(96, 2), (700, 4)])
+def test_routed_layer_against_oracle(dev, tokens, top_k):
+    """Router output -> sort -> gather -> experts -> weighted scatter (reference ParallelDroplessMLP,
+    src/olmo_core/nn/moe/parallel_mlp.py:102-183, :851-871) against the oracle's composition: NumPy-loop
+    permutation around the per-expert float8 emulation."""
+    E, D, H = 8, 256, 384
+    g = torch.Generator().manual_seed(11)
+    x = seeded((tokens, D), 12)
+    logits = torch.randn(tokens, E, generator=g)
+    logits[:, 5] = -1e9  # an expert nobody picks
+    scores = logits.softmax(-1)
+    expert_weights, expert_indices = torch.topk(scores, top_k, dim=-1)
+    expert_weights = expert_weights.bfloat16()
+    sizes = O.batched_histc(expert_indices.reshape(1, -1), E)[0]
+    go = seeded((tokens, D), 13, std=1e-2)
+
+    mlp = DroplessMoEMLP(d_model=D, hidden_size=H, num_experts=E, dtype=torch.bfloat16)
+    with torch.no_grad():
+        for p_ in mlp.parameters():
+            p_.copy_((torch.randn(p_.shape, generator=g) * 0.02).bfloat16())
+    w1, w2, w3 = (p_.detach().clone().view(E, H, D) for p_ in (mlp.w1, mlp.w2, mlp.w3))
+
+    # oracle: permutation loops + per-expert emulated float8 MLP (forward and grad_x through the same ops)
+    indices, bin_ids, bins = MO.indices_and_bins(expert_indices, E)
+    xs = MO.gather(x, indices, None, top_k)
+    ref = O.dropless_mlp_fwd_bwd(xs, w1, w2, w3, sizes.tolist(), None, O.recipe("rowwise"))
+    want = MO.scatter(ref["y"], indices, expert_weights.reshape(-1), top_k)
+
+    layer = ParallelDroplessMLP(mlp=mlp.to(dev), top_k=top_k)
+    xd = x.to(dev).requires_grad_(True)
+    wd = expert_weights.to(dev).requires_grad_(True)
+    out = layer(xd, wd, expert_indices.to(dev), sizes.to(dev))
+    assert out.shape == x.shape
+    rel, cos = gemm_errors(out, want)
+    assert rel <= 2e-2 and cos >= 0.9999, (rel, cos)
+    out.backward(go.to(dev))
+    # gradients: the oracle's chain, scatter^T = weighted gather, then the experts' backward, then gather^T = scatter
+    gys = MO.gather(go, indices, expert_weights.reshape(-1), top_k)
+    refb = O.dropless_mlp_fwd_bwd(xs, w1, w2, w3, sizes.tolist(), gys, O.recipe("rowwise"))
+    want_gx = MO.scatter(refb["grad_x"], indices, None, top_k)
+    rel, cos = gemm_errors(xd.grad, want_gx)
+    assert rel <= 3e-2 and cos >= 0.9995, ("grad_x", rel, cos)
+    want_gw = MO.scatter_wgrad(ref["y"], go, indices, top_k).reshape(tokens, top_k)
+    rel, cos = gemm_errors(wd.grad, want_gw)
+    assert rel <= 3e-2 and cos >= 0.9995, ("grad_expert_weights", rel, cos)
+    assert torch.count_nonzero(mlp.w1.grad.view(E, H, D)[5]) == 0
