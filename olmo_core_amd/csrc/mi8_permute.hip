@@ -18,6 +18,7 @@ namespace {
 
 constexpr int kThreads = 256;
 constexpr int kWavesPerBlock = kThreads / 64;
+constexpr int64_t kMaxBlocks = 256 * 8;
 
 // ---- element types --------------------------------------------------------------------------------------
 template <int DT>
@@ -133,13 +134,14 @@ template <int DT, bool SCALE, bool BINNED>
 __global__ __launch_bounds__(kThreads) void gather_kernel(PermuteArgs a, int64_t rows)
 {
     const int lane = threadIdx.x & 63;
-    const int64_t r = (int64_t)blockIdx.x * kWavesPerBlock + (threadIdx.x >> 6);
-    if (r >= rows) return;
     using T = typename El<DT>::T;
-    const int64_t idx = slot_of_row<BINNED>(a, r);
-    const T* src = idx < 0 ? nullptr : reinterpret_cast<const T*>(a.x) + (idx / a.top_k) * a.hidden;
-    const float w = (SCALE && idx >= 0) ? load_weight(a.weights, a.w_dtype, idx) : 1.0f;
-    copy_row<DT, SCALE>(src, reinterpret_cast<T*>(a.out) + r * a.hidden, a.hidden, w, a.vec, lane);
+    for (int64_t r = (int64_t)blockIdx.x * kWavesPerBlock + (threadIdx.x >> 6); r < rows;
+         r += (int64_t)gridDim.x * kWavesPerBlock) {
+        const int64_t idx = slot_of_row<BINNED>(a, r);
+        const T* src = idx < 0 ? nullptr : reinterpret_cast<const T*>(a.x) + (idx / a.top_k) * a.hidden;
+        const float w = (SCALE && idx >= 0) ? load_weight(a.weights, a.w_dtype, idx) : 1.0f;
+        copy_row<DT, SCALE>(src, reinterpret_cast<T*>(a.out) + r * a.hidden, a.hidden, w, a.vec, lane);
+    }
 }
 
 template <typename T>
@@ -165,11 +167,11 @@ __global__ __launch_bounds__(kThreads) void scatter_reduce_kernel(PermuteArgs a,
     using T = typename El<DT>::T;
     constexpr int N = 16 / sizeof(T);
     const int lane = threadIdx.x & 63;
-    const int64_t t = (int64_t)blockIdx.x * kWavesPerBlock + (threadIdx.x >> 6);
-    if (t >= tokens) return;
     const T* x = reinterpret_cast<const T*>(a.x);
-    T* out = reinterpret_cast<T*>(a.out) + t * a.hidden;
     const int k = a.top_k;
+    for (int64_t t = (int64_t)blockIdx.x * kWavesPerBlock + (threadIdx.x >> 6); t < tokens;
+         t += (int64_t)gridDim.x * kWavesPerBlock) {
+    T* out = reinterpret_cast<T*>(a.out) + t * a.hidden;
     if (a.vec) {
         const int64_t chunks = a.hidden / N;
         for (int64_t c = lane; c < chunks; c += 64) {
@@ -214,6 +216,7 @@ __global__ __launch_bounds__(kThreads) void scatter_reduce_kernel(PermuteArgs a,
             out[c] = (k == 1) ? first : El<DT>::from_f32(acc);
         }
     }
+    }
 }
 
 __device__ __forceinline__ float wave_sum(float v)
@@ -230,10 +233,10 @@ __global__ __launch_bounds__(kThreads) void scatter_wgrad_kernel(PermuteArgs a, 
     using T = typename El<DT>::T;
     constexpr int N = 16 / sizeof(T);
     const int lane = threadIdx.x & 63;
-    const int64_t r = (int64_t)blockIdx.x * kWavesPerBlock + (threadIdx.x >> 6);
-    if (r >= rows) return;
+    for (int64_t r = (int64_t)blockIdx.x * kWavesPerBlock + (threadIdx.x >> 6); r < rows;
+         r += (int64_t)gridDim.x * kWavesPerBlock) {
     const int64_t idx = slot_of_row<BINNED>(a, r);
-    if (idx < 0) return;
+    if (idx < 0) continue;
     const T* x = reinterpret_cast<const T*>(a.x) + r * a.hidden;
     const T* g = reinterpret_cast<const T*>(a.grad) + (idx / a.top_k) * a.hidden;
     float acc = 0.0f;
@@ -251,13 +254,20 @@ __global__ __launch_bounds__(kThreads) void scatter_wgrad_kernel(PermuteArgs a, 
     }
     acc = wave_sum(acc);
     if (lane == 0) reinterpret_cast<T*>(a.out)[idx] = El<DT>::from_f32(acc);
+    }
 }
 
 // ---- host side --------------------------------------------------------------------------------------------
 int elem_size(int dt) { return dt == MI8_F32 ? 4 : (dt == MI8_RAW8 ? 1 : 2); }
 bool valid_dt(int dt, bool allow_raw) { return dt == MI8_BF16 || dt == MI8_F32 || dt == MI8_F16 || (allow_raw && dt == MI8_RAW8); }
 bool valid_w(int dt) { return dt == MI8_BF16 || dt == MI8_F32 || dt == MI8_F16; }
-unsigned wave_blocks(int64_t rows) { return (unsigned)ceil_div(rows, kWavesPerBlock); }
+// one wave per row; long inputs are walked by a fixed-size grid (8 blocks per CU's worth) so that waves stay
+// resident and keep several rows in flight
+unsigned wave_blocks(int64_t rows)
+{
+    const int64_t need = ceil_div(rows, kWavesPerBlock);
+    return (unsigned)(need < kMaxBlocks ? need : kMaxBlocks);
+}
 
 bool rows_vectorisable(int64_t hidden, int dt, const void* p0, const void* p1, const void* p2 = nullptr)
 {
