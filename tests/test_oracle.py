@@ -53,6 +53,30 @@ def test_cast_known_answers():
     assert torch.tensor([1e9]).to(E4M3).view(torch.uint8).item() == 0x7F
 
 
+def test_decoders_against_format_tables():
+    """Every fp8 code decodes to the value the format specification gives it (tests/golden/fp8_decode_tables.json,
+    built from the closed form with exact rationals): torch-CPU and the C restatement, independently."""
+    import json
+    import math
+    from pathlib import Path
+
+    tables = json.loads((Path(__file__).parent / "golden" / "fp8_decode_tables.json").read_text())
+    for fp8, name in ((E4M3, "float8_e4m3fn"), (E5M2, "float8_e5m2")):
+        codes = torch.arange(256, dtype=torch.int32).to(torch.uint8)
+        got_torch = codes.view(fp8).float()
+        for c, want in enumerate(tables[name]):
+            got_c = C.lib().orc_fp8_to_f32(c, CODE[fp8])
+            for got in (float(got_torch[c]), float(got_c)):
+                if want == "nan":
+                    assert math.isnan(got), (name, c)
+                elif want in ("inf", "-inf"):
+                    assert got == float(want), (name, c)
+                elif want == "-0.0":
+                    assert got == 0.0 and math.copysign(1.0, got) < 0, (name, c)
+                else:
+                    assert got == float.fromhex(want), (name, c, got, want)
+
+
 def test_cast_decode_roundtrip():
     """Every finite fp8 code decodes (C table) to a float that encodes back to the same code."""
     for fp8 in (E4M3, E5M2):
