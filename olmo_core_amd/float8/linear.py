@@ -164,8 +164,13 @@ class _Float8Matmul(torch.autograd.Function):
         return gx, gw, None
 
 
+@torch.compiler.disable
 def float8_linear_function(x: torch.Tensor, weight: torch.Tensor, config: Float8LinearConfig) -> torch.Tensor:
-    """``x [*, K] @ weight[N, K].T`` through the float8 path, differentiable in x and weight."""
+    """``x [*, K] @ weight[N, K].T`` through the float8 path, differentiable in x and weight.
+
+    Opaque to ``torch.compile`` (a graph break per call): the kernels are reached through ctypes, which Dynamo
+    cannot trace; the reference takes the same route for its grouped GEMM (``src/olmo_core/nn/moe/mlp.py:256``).
+    """
     K = x.shape[-1]
     if weight.dim() != 2 or weight.shape[1] != K:
         raise ValueError(f"float8 linear: input features {K} do not match weight {tuple(weight.shape)}")

@@ -36,6 +36,7 @@ class _SwiGLU(torch.autograd.Function):
         return g1, g3
 
 
+@torch.compiler.disable
 def swiglu(x1: torch.Tensor, x3: torch.Tensor) -> torch.Tensor:
     """``silu(x1) * x3`` for bfloat16 GPU tensors (one fused kernel forward, one backward)."""
     return _SwiGLU.apply(x1, x3)
@@ -127,6 +128,11 @@ def _fusable(ff: "FeedForward", x: torch.Tensor) -> bool:
     return same and x.is_cuda and x.dtype == torch.bfloat16 and not torch.is_autocast_enabled()
 
 
+@torch.compiler.disable
+def _fused_mlp(x2, w1, w2, w3, config):
+    return _Float8SwiGLUMLP.apply(x2, w1, w2, w3, config)
+
+
 class FeedForward(nn.Module):
     """Gated feed-forward with SiLU activation: ``w2(silu(w1 x) * w3 x)``."""
 
@@ -151,7 +157,7 @@ class FeedForward(nn.Module):
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         if self.fuse_float8 and _fusable(self, x):
             x2 = x.reshape(-1, x.shape[-1])
-            y = _Float8SwiGLUMLP.apply(x2, self.w1.weight, self.w2.weight, self.w3.weight, self.w1.config)
+            y = _fused_mlp(x2, self.w1.weight, self.w2.weight, self.w3.weight, self.w1.config)
             return y.reshape(*x.shape[:-1], self.w2.weight.shape[0])
         x1, x3 = self.w1(x), self.w3(x)
         if x1.is_cuda and x1.dtype == torch.bfloat16:

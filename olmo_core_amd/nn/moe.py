@@ -92,6 +92,7 @@ class _Float8DroplessMLP(torch.autograd.Function):
         return gx, as_param(gw1, w1), as_param(gw2, w2), as_param(gw3, w3), None, None, None
 
 
+@torch.compiler.disable
 def float8_dropless_mlp(x, w1, w2, w3, batch_size_per_expert, num_experts: int, pow2: bool = True):
     """``gmm(silu(gmm(x, w1^T)) * gmm(x, w3^T), w2)`` with float8 grouped GEMMs; ``x`` is ``[T, d_model]`` bf16."""
     return _Float8DroplessMLP.apply(x, w1, w2, w3, batch_size_per_expert, num_experts, pow2)

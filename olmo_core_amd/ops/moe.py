@@ -197,6 +197,7 @@ class GatherOp(torch.autograd.Function):
         return _scatter(grad.contiguous(), indices, None, ctx.top_k), None, None, None, None
 
 
+@torch.compiler.disable
 def gather(x, indices, bin_ids, bins, top_k: int) -> torch.Tensor:
     return GatherOp.apply(x, indices, bin_ids, bins, top_k)
 
@@ -222,6 +223,7 @@ class ScatterOp(torch.autograd.Function):
         return dgrad, None, None, wgrad, None, None
 
 
+@torch.compiler.disable
 def scatter(x, indices, bin_ids, weights, bins, top_k: int) -> torch.Tensor:
     return ScatterOp.apply(x, indices, bin_ids, weights, bins, top_k)
 
@@ -241,6 +243,7 @@ class BinnedGatherOp(torch.autograd.Function):
         return _binned_scatter(grad.contiguous(), indices, None, bins, ctx.top_k), None, None, None, None
 
 
+@torch.compiler.disable
 def binned_gather(x, indices, bins, bin_size: int, top_k: int) -> torch.Tensor:
     return BinnedGatherOp.apply(x, indices, bins, bin_size, top_k)
 
@@ -266,6 +269,7 @@ class BinnedScatterOp(torch.autograd.Function):
         return out, None, wgrad, None, None
 
 
+@torch.compiler.disable
 def binned_scatter(x, indices, weights, bins, top_k: int) -> torch.Tensor:
     return BinnedScatterOp.apply(x, indices, weights, bins, top_k)
 

@@ -174,3 +174,37 @@ def test_apply_float8_linear_on_gpu_model(dev):
     x = torch.randn(4, 32, 64, device=dev, dtype=torch.bfloat16)
     m(x).float().sum().backward()
     assert all(p.grad is not None for p in m.parameters())
+
+
+def test_torch_compile_composes(dev):
+    """A compiled block with converted linears inside runs (the float8 linear is a graph break, as the reference
+    accepts for its grouped GEMM, src/olmo_core/nn/moe/mlp.py:256) and gives the eager result bit for bit."""
+    import torch.nn as nn
+
+    from olmo_core_amd.float8 import Float8Config
+
+    class Block(nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.norm = nn.LayerNorm(256)
+            self.w1 = nn.Linear(256, 512, bias=False)
+            self.w2 = nn.Linear(512, 256, bias=True)
+
+        def forward(self, x):
+            return x + self.w2(torch.nn.functional.silu(self.w1(self.norm(x))))
+
+    torch.manual_seed(0)
+    m = Block().to(dev).bfloat16()
+    Float8Config(enabled=True).apply_float8_linear(m)
+    x = torch.randn(64, 256, device=dev, dtype=torch.bfloat16, requires_grad=True)
+    y0 = m(x)
+    y0.float().sum().backward()
+    g0, gw0 = x.grad.clone(), m.w1.weight.grad.clone()
+    x.grad = None
+    m.zero_grad()
+    mc = torch.compile(m, fullgraph=False)
+    y1 = mc(x)
+    y1.float().sum().backward()
+    assert torch.allclose(y1.float(), y0.float(), rtol=2e-2, atol=2e-2)  # inductor may fuse the bf16 pointwise parts differently
+    assert torch.allclose(x.grad.float(), g0.float(), rtol=5e-2, atol=5e-2)
+    assert torch.allclose(m.w1.weight.grad.float(), gw0.float(), rtol=5e-2, atol=5e-2)
