@@ -124,7 +124,7 @@ int mi8_gemm_fp8(const void* a, int a_dtype, int64_t lda, const void* b, int b_d
                  int64_t N, int64_t K, const float* sa, int sa_is_vector, const float* sb, int sb_is_vector,
                  void* out, int out_dtype, int64_t ldc, int variant, void* stream);
 
-/* Number of GEMM kernel variants compiled in (variant ids 0..n-1; 0 is the default). */
+/* Number of GEMM kernel variants compiled in (variant ids 0..n-1; -1 lets the library choose by shape). */
 int mi8_gemm_num_variants(void);
 const char* mi8_gemm_variant_name(int variant);
 

@@ -77,6 +77,8 @@ __device__ __forceinline__ bool tile_of_block(const GemmArgs& g, int& tm, int& t
 int launch_dma(GemmArgs& g, int a_dtype, int b_dtype, hipStream_t st);
 // same, 8 waves per workgroup and full 128-byte rows; additionally K % 128 == 0 (mi8_gemm_dma8.hip)
 int launch_dma8(GemmArgs& g, int a_dtype, int b_dtype, hipStream_t st);
+// the same kernel with four waves of 128 x 128 (one wave per SIMD)
+int launch_dma4(GemmArgs& g, int a_dtype, int b_dtype, hipStream_t st);
 // The same kernel over the ragged grouped problems (bf16 output, per-row / per-column scale vectors):
 // forward / grad_input (T, N >= 256, K % 128 == 0) and grad_weight (N, Kl >= 256).
 int launch_dma8_grouped(const uint8_t* a, int a_dtype, int64_t lda, const uint8_t* b, int b_dtype, int64_t ldb,

@@ -24,22 +24,36 @@ namespace gemm {
 namespace {
 
 constexpr int BM = 256, BN = 256;
-constexpr int WTM = 128, WTN = 64;
-constexpr int TM = 4, TN = 2;
-constexpr int NT = 512;
+constexpr int WTM = 128, TM = 4;               // two waves along M, each 4 MFMA tiles of 32 rows
 constexpr int STAGE = (BM + BN) * BK;          // 64 KB
-constexpr int OUT_STAGING = 8 * 32 * WTN * 2;  // 8 waves x (32 rows x 64 bf16) = 32 KB
+constexpr int OUT_STAGING = 8 * 4096;           // 4 KB of output staging per wave
 constexpr int LDS_BYTES = 2 * STAGE + OUT_STAGING;
-constexpr int NH = 2 * (TM + TN);              // 16-byte fragment halves per K sub-step: 12
+
+// The wave layout is 2 x WN.  WN = 4: eight waves of 128 x 64 (two per SIMD, 256 registers each).  WN = 2: four
+// waves of 128 x 128 (one per SIMD, 512 registers: twice the accumulators, a third less LDS read traffic, but no
+// second wave to fill the matrix pipe while one waits).
+template <int WN>
+struct Layout {
+    static constexpr int kWaves = 2 * WN;
+    static constexpr int kThreads = kWaves * 64;
+    static constexpr int WTN = BN / WN;            // wave tile columns: 64 or 128
+    static constexpr int TN = WTN / 32;            // MFMA tiles along N per wave: 2 or 4
+    static constexpr int NH = 2 * (TM + TN);       // 16-byte fragment halves per K sub-step: 12 or 16
+    static constexpr int kMmas = TM * TN;          // MFMAs per K sub-step: 8 or 16
+    static constexpr int kRowsPerWave = BM / kWaves;  // operand rows a wave fetches per step: 32 or 64
+    static constexpr int kLoads = kRowsPerWave / 8;   // direct loads per operand, step and wave: 4 or 8
+};
 
 typedef __attribute__((address_space(1))) const void* gptr_t;
 typedef __attribute__((address_space(3))) void* lptr_t;
 
-// fragment halves of one 64-byte K sub-step in consumption order: A0, B0, B1, A1, A2, A3 (two halves each)
+// fragment halves of one 64-byte K sub-step in consumption order: A0, B0 .. B(TN-1), A1, A2, A3 (two halves each)
+template <int NH>
 struct Frags {
     v4i h[NH];
 };
-__device__ __forceinline__ constexpr int frag_a(int i) { return i == 0 ? 0 : 4 + 2 * i; }
+template <int TN>
+__device__ __forceinline__ constexpr int frag_a(int i) { return i == 0 ? 0 : 2 * TN + 2 * i; }
 __device__ __forceinline__ constexpr int frag_b(int j) { return 2 + 2 * j; }
 
 
@@ -286,15 +300,18 @@ struct GroupedWgradProblem {
     }
 };
 
-template <typename Problem, int CBSZ_A, int BLGP_B>
-__global__ __launch_bounds__(NT, 1) void gemm_fp8_dma8_kernel(Problem pb)
+template <typename Problem, int WN, int CBSZ_A, int BLGP_B>
+__global__ __launch_bounds__(Layout<WN>::kThreads, 1) void gemm_fp8_dma8_kernel(Problem pb)
 {
+    using L = Layout<WN>;
+    constexpr int WTN = L::WTN, TN = L::TN, NH = L::NH;
+    using Frags = mi8::gemm::Frags<NH>;
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int wm = wave >> 2, wn = wave & 3;
+    const int wm = wave / WN, wn = wave % WN;
     const int l32 = lane & 31, half = lane >> 5;
 
     // ---- fragment read offsets.  MFMA tile `tile` of a wave reads rows r0 + 32 tile (r0 = wave origin + l32, the
@@ -306,32 +323,34 @@ __global__ __launch_bounds__(NT, 1) void gemm_fp8_dma8_kernel(Problem pb)
     // registers instead of eight precomputed addresses matters: the kernel runs at the 256-register limit.
     const uint32_t xa00 = (uint32_t)((wm * WTM + l32) * BK + (((2 * half) ^ swz(wm * WTM + l32)) << 4));
     const uint32_t xb00 = (uint32_t)(BM * BK + (wn * WTN + l32) * BK + (((2 * half) ^ swz(wn * WTN + l32)) << 4));
-    // slot x of Frags: 0,1 = A0; 2..5 = B0,B1; 6..11 = A1..A3.  pa / pb: xa00 / xb00 plus the stage's byte offset.
+    // slot x of Frags: 0,1 = A0; then two per B tile; then A1..A3.  pa / pb: xa00 / xb00 plus the stage's byte offset.
     auto read_one = [&](Frags& f, uint32_t pa, uint32_t pb_, int s, int x) __attribute__((always_inline)) {
-        const bool is_a = (x < 2) || (x >= 6);
-        const int tile = x < 2 ? 0 : (x < 6 ? (x - 2) >> 1 : (x - 4) >> 1);
+        const bool is_a = (x < 2) || (x >= 2 + 2 * TN);
+        const int tile = x < 2 ? 0 : (x < 2 + 2 * TN ? (x - 2) >> 1 : (x - 2 * TN) >> 1);
         const int q = x & 1;
         const uint32_t off = ((is_a ? pa : pb_) ^ (uint32_t)(((4 * (s ^ (tile & 1))) | q) << 4)) + tile * 32 * BK;
         f.h[x] = *reinterpret_cast<const v4i*>(lds + off);
     };
 
-    // ---- direct loads: wave w fills rows [32 w + 8 p, +8) of each operand, p = 0..3;
-    // lane -> row 32 w + 8 p + lr (lr = lane / 8), position lane % 8; swz(row) = (lr ^ (4 w + p)) & 7
+    // ---- direct loads: wave w fills rows [R w + 8 p, +8) of each operand, R = kRowsPerWave, p = 0..kLoads-1;
+    // lane -> row R w + 8 p + lr (lr = lane / 8), position lane % 8; swz(row) = (lr ^ (R/8 w + p)) & 7
+    constexpr int RPW = L::kRowsPerWave, NLD = L::kLoads;
     const int lr = lane >> 3;
     const uint32_t c0 = (uint32_t)((lane & 7) ^ lr);
-    const uint32_t rowoff_a = (uint32_t)((int64_t)(wave * 32 + lr) * pb.lda);
-    const uint32_t rowoff_b = (uint32_t)((int64_t)(wave * 32 + lr) * pb.ldb);
-    // x in 0..7: 0..3 -> A rows 8 x, 4..7 -> B rows 8 (x - 4)
+    const uint32_t rowoff_a = (uint32_t)((int64_t)(wave * RPW + lr) * pb.lda);
+    const uint32_t rowoff_b = (uint32_t)((int64_t)(wave * RPW + lr) * pb.ldb);
+    // x in 0..2 NLD-1: the first NLD -> A rows 8 x, the rest -> B rows 8 (x - NLD)
     auto dma_one = [&](const uint8_t* a_origin, const uint8_t* b_origin, int stage, int x) __attribute__((always_inline)) {
-        const int p = x & 3;
+        const int p = x % NLD;
+        const bool is_a = x < NLD;
         // uniform 64-bit base + 32-bit lane offset.  The empty asm makes the lane's chunk index opaque at every
         // use: the offset is then rebuilt with two cheap vector instructions next to the load (and folded into
         // its scalar-base addressing) instead of living in eight hoisted 64-bit lane addresses.
         uint32_t c = c0;
         asm volatile("" : "+v"(c));
-        const uint32_t voff = (x < 4 ? rowoff_a : rowoff_b) + ((c ^ (uint32_t)((4 * wave + p) & 7)) << 4);
-        const uint8_t* src = (x < 4 ? a_origin + (int64_t)(8 * p) * pb.lda : b_origin + (int64_t)(8 * p) * pb.ldb) + voff;
-        uint8_t* dst = lds + stage * STAGE + (x < 4 ? 0 : BM * BK) + (wave * 32 + 8 * p) * BK;
+        const uint32_t voff = (is_a ? rowoff_a : rowoff_b) + ((c ^ (uint32_t)((NLD * wave + p) & 7)) << 4);
+        const uint8_t* src = (is_a ? a_origin + (int64_t)(8 * p) * pb.lda : b_origin + (int64_t)(8 * p) * pb.ldb) + voff;
+        uint8_t* dst = lds + stage * STAGE + (is_a ? 0 : BM * BK) + (wave * RPW + 8 * p) * BK;
         __builtin_amdgcn_global_load_lds((gptr_t)src, (lptr_t)dst, 16, 0, 0);
     };
 
@@ -407,8 +426,8 @@ __global__ __launch_bounds__(NT, 1) void gemm_fp8_dma8_kernel(Problem pb)
     // `fresh`: the tile's first touch of this accumulator; the MFMA then takes the constant 0 as its addend, so
     // the 128 accumulator registers never have to be cleared between tiles
     auto mma_one = [&](const Frags& f, int x, bool fresh) __attribute__((always_inline)) {
-        const int i = x >> 1, j = x & 1;
-        const v8i fa = __builtin_shufflevector(f.h[frag_a(i)], f.h[frag_a(i) + 1], 0, 1, 2, 3, 4, 5, 6, 7);
+        const int i = x / TN, j = x % TN;
+        const v8i fa = __builtin_shufflevector(f.h[frag_a<TN>(i)], f.h[frag_a<TN>(i) + 1], 0, 1, 2, 3, 4, 5, 6, 7);
         const v8i fb = __builtin_shufflevector(f.h[frag_b(j)], f.h[frag_b(j) + 1], 0, 1, 2, 3, 4, 5, 6, 7);
         const v16f zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
         acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fb, fa, fresh ? zero : acc[i][j], BLGP_B, CBSZ_A, 0, 0,
@@ -421,7 +440,7 @@ __global__ __launch_bounds__(NT, 1) void gemm_fp8_dma8_kernel(Problem pb)
 #pragma unroll
         for (int s = 0; s < 2; ++s) {
 #pragma unroll
-            for (int x = 0; x < 8; ++x) dma_one(ld_a, ld_b, s, x);
+            for (int x = 0; x < 2 * NLD; ++x) dma_one(ld_a, ld_b, s, x);
             advance_load_cursor();
         }
     }
@@ -441,14 +460,26 @@ __global__ __launch_bounds__(NT, 1) void gemm_fp8_dma8_kernel(Problem pb)
             const int cur = step & 1;
             const uint32_t pa_cur = xa00 + cur * STAGE, pb_cur = xb00 + cur * STAGE;
             const uint32_t pa_nxt = xa00 + (cur ^ 1) * STAGE, pb_nxt = xb00 + (cur ^ 1) * STAGE;
-            // phase A: its 8 MFMAs touch each of the 8 accumulator tiles once
-#pragma unroll
-            for (int x = 0; x < 8; ++x) {
-                mma_one(f0, x, fresh);
-                if (x >= 1 && x < 7) {
-                    read_one(f1, pa_cur, pb_cur, 1, 2 * x - 2);
-                    read_one(f1, pa_cur, pb_cur, 1, 2 * x - 1);
+            // Fragment reads trail the MFMAs: with 8 MFMAs per phase two reads follow MFMAs 1..6 (any earlier and
+            // the 256-register budget overflows), with 16 MFMAs two reads follow each of the first eight.
+            auto reads_after = [&](Frags& f, uint32_t pa, uint32_t pb_, int s, int x) __attribute__((always_inline)) {
+                if constexpr (TN == 2) {
+                    if (x >= 1 && x < 7) {
+                        read_one(f, pa, pb_, s, 2 * x - 2);
+                        read_one(f, pa, pb_, s, 2 * x - 1);
+                    }
+                } else {
+                    if (x < 8) {
+                        read_one(f, pa, pb_, s, 2 * x);
+                        read_one(f, pa, pb_, s, 2 * x + 1);
+                    }
                 }
+            };
+            // phase A: its MFMAs touch each accumulator tile once
+#pragma unroll
+            for (int x = 0; x < L::kMmas; ++x) {
+                mma_one(f0, x, fresh);
+                reads_after(f1, pa_cur, pb_cur, 1, x);
                 __builtin_amdgcn_sched_barrier(0);
             }
             // the compiler does not track direct-to-LDS loads across a barrier: wait for this wave's
@@ -457,13 +488,10 @@ __global__ __launch_bounds__(NT, 1) void gemm_fp8_dma8_kernel(Problem pb)
             __syncthreads();
             // phase B
 #pragma unroll
-            for (int x = 0; x < 8; ++x) {
+            for (int x = 0; x < L::kMmas; ++x) {
                 mma_one(f1, x, false);
-                if (x >= 1 && x < 7) {
-                    read_one(f0, pa_nxt, pb_nxt, 0, 2 * x - 2);
-                    read_one(f0, pa_nxt, pb_nxt, 0, 2 * x - 1);
-                }
-                dma_one(ld_a, ld_b, cur, x);
+                reads_after(f0, pa_nxt, pb_nxt, 0, x);
+                dma_one(ld_a, ld_b, cur, x);  // kMmas == 2 * kLoads: one direct load per MFMA (bunching them up is slower)
                 __builtin_amdgcn_sched_barrier(0);
             }
             advance_load_cursor();
@@ -484,72 +512,80 @@ __global__ __launch_bounds__(NT, 1) void gemm_fp8_dma8_kernel(Problem pb)
         // A single scale is inverted with an IEEE division, scale vectors with v_rcp_f32 (exact for the
         // power-of-two scales of the axiswise recipes, within 1 ulp otherwise).
         if (Problem::kPeelFirstStep && td.nk == 0) clear_acc();  // nothing was accumulated (empty group)
-        uint8_t* stg = lds + 2 * STAGE + wave * (32 * WTN * 2);  // wave-private 4 KB: 32 rows x 128 bytes
+        // The wave's output goes through its private staging area 32 rows x 64 columns at a time (4 KB, pitch 128
+        // bytes), i.e. one row group of MFMA tiles and two tile columns per pass.
+        uint8_t* stg = lds + 2 * STAGE + wave * 4096;
         const bool zero_tile = td.nk == 0;  // nothing accumulated; the scales may be unset
-        float isb[TN][4][4];
-        if constexpr (Problem::kVecScales) {
-#pragma unroll
-            for (int j = 0; j < TN; ++j)
-#pragma unroll
-                for (int q = 0; q < 4; ++q) {
-                    const float4 s4 = *reinterpret_cast<const float4*>(td.sb + wn * WTN + j * 32 + 8 * q + 4 * half);
-                    isb[j][q][0] = zero_tile ? 0.0f : __builtin_amdgcn_rcpf(s4.x);
-                    isb[j][q][1] = zero_tile ? 0.0f : __builtin_amdgcn_rcpf(s4.y);
-                    isb[j][q][2] = zero_tile ? 0.0f : __builtin_amdgcn_rcpf(s4.z);
-                    isb[j][q][3] = zero_tile ? 0.0f : __builtin_amdgcn_rcpf(s4.w);
-                }
-        }
         const float isb_scalar = Problem::kVecScales ? 1.0f : 1.0f / td.sb[0];
-        const float isa_scalar = Problem::kVecScales ? 1.0f : 1.0f / td.sa[0];
 #pragma unroll
-        for (int i = 0; i < TM; ++i) {
-            const int rt = wm * WTM + i * 32;  // first tile row of this pass
-            float mult = Problem::kVecScales ? __builtin_amdgcn_rcpf(td.sa[rt + l32]) : isa_scalar;
-            mult = zero_tile ? 0.0f : mult * isb_scalar;
-            // 32 rows x 64 bf16 through the wave's staging area: pitch 128 bytes, the 16-byte chunk index XORed
-            // with (row >> 1) & 7 so that 16 consecutive rows cover all banks
+        for (int jh = 0; jh < TN / 2; ++jh) {
+            float isb[2][4][4];
+            if constexpr (Problem::kVecScales) {
 #pragma unroll
-            for (int j = 0; j < TN; ++j)
+                for (int j = 0; j < 2; ++j)
 #pragma unroll
-                for (int q = 0; q < 4; ++q) {
-                    const int cw = j * 32 + 8 * q + 4 * half;  // column inside the wave tile, multiple of 4
-                    float v[4];
-#pragma unroll
-                    for (int e = 0; e < 4; ++e) {
-                        v[e] = acc[i][j][4 * q + e] * mult;
-                        if constexpr (Problem::kVecScales) v[e] *= isb[j][q][e];
+                    for (int q = 0; q < 4; ++q) {
+                        const float4 s4 =
+                            *reinterpret_cast<const float4*>(td.sb + wn * WTN + (2 * jh + j) * 32 + 8 * q + 4 * half);
+                        isb[j][q][0] = zero_tile ? 0.0f : __builtin_amdgcn_rcpf(s4.x);
+                        isb[j][q][1] = zero_tile ? 0.0f : __builtin_amdgcn_rcpf(s4.y);
+                        isb[j][q][2] = zero_tile ? 0.0f : __builtin_amdgcn_rcpf(s4.z);
+                        isb[j][q][3] = zero_tile ? 0.0f : __builtin_amdgcn_rcpf(s4.w);
                     }
-                    uint2 o;
-                    o.x = pack_bf16x2(v[0], v[1]);
-                    o.y = pack_bf16x2(v[2], v[3]);
-                    const int chunk = (cw >> 3) ^ ((l32 >> 1) & 7);
-                    *reinterpret_cast<uint2*>(stg + l32 * 128 + chunk * 16 + (cw & 4) * 2) = o;
-                }
-            __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): the wave's own LDS writes have landed
-            __builtin_amdgcn_wave_barrier();
-            uint4 staged[4];
-#pragma unroll
-            for (int it = 0; it < 4; ++it) {
-                const int rw = it * 8 + (lane >> 3);
-                staged[it] = *reinterpret_cast<const uint4*>(stg + rw * 128 + (((lane & 7) ^ ((rw >> 1) & 7)) << 4));
             }
-            // rows [rt, rt + 32) of the tile; a pass that lies completely inside the stored range (the common
-            // case, decided per wave) needs no per-lane predicate
-            const bool all_rows = !Problem::kMaskRows || (rt >= td.row_lo && rt + 32 <= td.row_hi);
-            uint16_t* crow = td.c + (int64_t)(rt + (lane >> 3)) * pb.ldc + wn * WTN + (lane & 7) * 8;
-            if (all_rows) {
 #pragma unroll
-                for (int it = 0; it < 4; ++it) *reinterpret_cast<uint4*>(crow + (int64_t)(it * 8) * pb.ldc) = staged[it];
-            } else {
+            for (int i = 0; i < TM; ++i) {
+                const int rt = wm * WTM + i * 32;  // first tile row of this pass
+                // A single scale is re-read (volatile) in every pass: the pass then depends on a load, as it does
+                // with scale vectors; with a loop-invariant multiplier the compiler forms the products of the
+                // whole tile up front and spills accumulators.
+                float mult = Problem::kVecScales ? __builtin_amdgcn_rcpf(td.sa[rt + l32])
+                                                 : 1.0f / *reinterpret_cast<const volatile float*>(td.sa);
+                mult = zero_tile ? 0.0f : mult * isb_scalar;
+                // the 16-byte chunk index is XORed with (row >> 1) & 7 so that 16 consecutive rows cover all banks
+#pragma unroll
+                for (int j = 0; j < 2; ++j)
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) {
+                        const int cw = j * 32 + 8 * q + 4 * half;  // column inside the 64-column pass, multiple of 4
+                        float v[4];
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) {
+                            v[e] = acc[i][2 * jh + j][4 * q + e] * mult;
+                            if constexpr (Problem::kVecScales) v[e] *= isb[j][q][e];
+                        }
+                        uint2 o;
+                        o.x = pack_bf16x2(v[0], v[1]);
+                        o.y = pack_bf16x2(v[2], v[3]);
+                        const int chunk = (cw >> 3) ^ ((l32 >> 1) & 7);
+                        *reinterpret_cast<uint2*>(stg + l32 * 128 + chunk * 16 + (cw & 4) * 2) = o;
+                    }
+                __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): the wave's own LDS writes have landed
+                __builtin_amdgcn_wave_barrier();
+                v4i staged[4];  // (an ext-vector type: arrays of HIP's uint4 struct end up in scratch)
 #pragma unroll
                 for (int it = 0; it < 4; ++it) {
-                    const int trow = rt + it * 8 + (lane >> 3);
-                    if (trow >= td.row_lo && trow < td.row_hi)
-                        *reinterpret_cast<uint4*>(crow + (int64_t)(it * 8) * pb.ldc) = staged[it];
+                    const int rw = it * 8 + (lane >> 3);
+                    staged[it] = *reinterpret_cast<const v4i*>(stg + rw * 128 + (((lane & 7) ^ ((rw >> 1) & 7)) << 4));
                 }
+                // rows [rt, rt + 32) of the tile; a pass that lies completely inside the stored range (the common
+                // case, decided per wave) needs no per-lane predicate
+                const bool all_rows = !Problem::kMaskRows || (rt >= td.row_lo && rt + 32 <= td.row_hi);
+                uint16_t* crow = td.c + (int64_t)(rt + (lane >> 3)) * pb.ldc + wn * WTN + jh * 64 + (lane & 7) * 8;
+                if (all_rows) {
+#pragma unroll
+                    for (int it = 0; it < 4; ++it) *reinterpret_cast<v4i*>(crow + (int64_t)(it * 8) * pb.ldc) = staged[it];
+                } else {
+#pragma unroll
+                    for (int it = 0; it < 4; ++it) {
+                        const int trow = rt + it * 8 + (lane >> 3);
+                        if (trow >= td.row_lo && trow < td.row_hi)
+                            *reinterpret_cast<v4i*>(crow + (int64_t)(it * 8) * pb.ldc) = staged[it];
+                    }
+                }
+                __builtin_amdgcn_s_waitcnt(0xc07f);  // the reads are done before the next pass overwrites
+                __builtin_amdgcn_wave_barrier();
             }
-            __builtin_amdgcn_s_waitcnt(0xc07f);  // the reads are done before the next pass overwrites
-            __builtin_amdgcn_wave_barrier();
         }
     }
     // direct loads issued for steps past the end must have landed before the LDS allocation is released
@@ -572,10 +608,10 @@ int num_cus()
 
 // persistent: one workgroup per CU walks a static share of the tiles (right when all tiles cost the same);
 // otherwise one workgroup per tile, handed to free CUs by the hardware dispatcher (tiles of unequal cost).
-template <typename Problem, int CBSZ_A, int BLGP_B>
+template <typename Problem, int WN, int CBSZ_A, int BLGP_B>
 int launch(const Problem& pb, int max_tiles, bool persistent, hipStream_t st)
 {
-    auto kern = gemm_fp8_dma8_kernel<Problem, CBSZ_A, BLGP_B>;
+    auto kern = gemm_fp8_dma8_kernel<Problem, WN, CBSZ_A, BLGP_B>;
     static bool configured = false;
     if (!configured) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
@@ -588,18 +624,18 @@ int launch(const Problem& pb, int max_tiles, bool persistent, hipStream_t st)
     }
     int blocks = persistent ? num_cus() : max_tiles;
     if (blocks > max_tiles) blocks = max_tiles;
-    hipLaunchKernelGGL(kern, dim3(blocks), dim3(NT), LDS_BYTES, st, pb);
+    hipLaunchKernelGGL(kern, dim3(blocks), dim3(Layout<WN>::kThreads), LDS_BYTES, st, pb);
     return launch_status("mi8 direct-to-LDS GEMM (8 waves)");
 }
 
-template <typename Problem>
+template <typename Problem, int WN = 4>
 int launch_typed(const Problem& pb, int max_tiles, bool persistent, int a_dtype, int b_dtype, hipStream_t st)
 {
     if (a_dtype == MI8_E4M3)
-        return b_dtype == MI8_E4M3 ? launch<Problem, 0, 0>(pb, max_tiles, persistent, st)
-                                   : launch<Problem, 0, 1>(pb, max_tiles, persistent, st);
-    return b_dtype == MI8_E4M3 ? launch<Problem, 1, 0>(pb, max_tiles, persistent, st)
-                               : launch<Problem, 1, 1>(pb, max_tiles, persistent, st);
+        return b_dtype == MI8_E4M3 ? launch<Problem, WN, 0, 0>(pb, max_tiles, persistent, st)
+                                   : launch<Problem, WN, 0, 1>(pb, max_tiles, persistent, st);
+    return b_dtype == MI8_E4M3 ? launch<Problem, WN, 1, 0>(pb, max_tiles, persistent, st)
+                               : launch<Problem, WN, 1, 1>(pb, max_tiles, persistent, st);
 }
 
 }  // namespace
@@ -614,6 +650,18 @@ int launch_dma8(GemmArgs& g, int a_dtype, int b_dtype, hipStream_t st)
     }
     DenseProblem<false> pb{g, g.lda, g.ldb, g.ldc};
     return launch_typed(pb, g.tiles_m * g.tiles_n, true, a_dtype, b_dtype, st);
+}
+
+int launch_dma4(GemmArgs& g, int a_dtype, int b_dtype, hipStream_t st)
+{
+    g.tiles_m = (g.M + BM - 1) / BM;
+    g.tiles_n = (g.N + BN - 1) / BN;
+    if (g.sa_vec) {
+        DenseProblem<true> pb{g, g.lda, g.ldb, g.ldc};
+        return launch_typed<DenseProblem<true>, 2>(pb, g.tiles_m * g.tiles_n, true, a_dtype, b_dtype, st);
+    }
+    DenseProblem<false> pb{g, g.lda, g.ldb, g.ldc};
+    return launch_typed<DenseProblem<false>, 2>(pb, g.tiles_m * g.tiles_n, true, a_dtype, b_dtype, st);
 }
 
 int launch_dma8_grouped(const uint8_t* a, int a_dtype, int64_t lda, const uint8_t* b, int b_dtype, int64_t ldb,
