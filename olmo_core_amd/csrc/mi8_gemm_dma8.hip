@@ -28,6 +28,7 @@ constexpr int WTM = 128, TM = 4;               // two waves along M, each 4 MFMA
 constexpr int STAGE = (BM + BN) * BK;          // 64 KB
 constexpr int OUT_STAGING = 8 * 4096;           // 4 KB of output staging per wave
 constexpr int LDS_BYTES = 2 * STAGE + OUT_STAGING;
+constexpr int kGroupedWN = 2;  // wave layout of the ragged problems (2 x 2 measured faster than 2 x 4)
 
 // The wave layout is 2 x WN.  WN = 4: eight waves of 128 x 64 (two per SIMD, 256 registers each).  WN = 2: four
 // waves of 128 x 128 (one per SIMD, 512 registers: twice the accumulators, a third less LDS read traffic, but no
@@ -497,7 +498,9 @@ __global__ __launch_bounds__(Layout<WN>::kThreads, 1) void gemm_fp8_dma8_kernel(
             advance_load_cursor();
             ++step;
         };
-        if constexpr (Problem::kPeelFirstStep) {
+        // (with eight waves the ragged-M instantiation compiles to slower code when the first step is peeled)
+        constexpr bool kPeel = Problem::kPeelFirstStep || WN == 2;
+        if constexpr (kPeel) {
             if (td.nk > 0) {
                 k_step(true);
                 for (int kt = 1; kt < td.nk; ++kt) k_step(false);
@@ -511,12 +514,17 @@ __global__ __launch_bounds__(Layout<WN>::kThreads, 1) void gemm_fp8_dma8_kernel(
         // acc[i][j][e] of lane l is C[row = 32 i + l%32][col = 32 j + 8*(e/4) + 4*(l/32) + e%4] of the wave tile.
         // A single scale is inverted with an IEEE division, scale vectors with v_rcp_f32 (exact for the
         // power-of-two scales of the axiswise recipes, within 1 ulp otherwise).
-        if (Problem::kPeelFirstStep && td.nk == 0) clear_acc();  // nothing was accumulated (empty group)
+        if (kPeel && td.nk == 0) clear_acc();  // nothing was accumulated (empty group)
         // The wave's output goes through its private staging area 32 rows x 64 columns at a time (4 KB, pitch 128
         // bytes), i.e. one row group of MFMA tiles and two tile columns per pass.
         uint8_t* stg = lds + 2 * STAGE + wave * 4096;
         const bool zero_tile = td.nk == 0;  // nothing accumulated; the scales may be unset
         const float isb_scalar = Problem::kVecScales ? 1.0f : 1.0f / td.sb[0];
+        const int ldc_bytes = (int)pb.ldc * 2;
+        __amdgpu_buffer_rsrc_t c_rows;
+        if constexpr (Problem::kMaskRows)
+            c_rows = __builtin_amdgcn_make_buffer_rsrc(td.c + (int64_t)td.row_lo * pb.ldc, 0,
+                                                       (td.row_hi - td.row_lo) * ldc_bytes, 0x00020000);
 #pragma unroll
         for (int jh = 0; jh < TN / 2; ++jh) {
             float isb[2][4][4];
@@ -568,20 +576,19 @@ __global__ __launch_bounds__(Layout<WN>::kThreads, 1) void gemm_fp8_dma8_kernel(
                     const int rw = it * 8 + (lane >> 3);
                     staged[it] = *reinterpret_cast<const v4i*>(stg + rw * 128 + (((lane & 7) ^ ((rw >> 1) & 7)) << 4));
                 }
-                // rows [rt, rt + 32) of the tile; a pass that lies completely inside the stored range (the common
-                // case, decided per wave) needs no per-lane predicate
-                const bool all_rows = !Problem::kMaskRows || (rt >= td.row_lo && rt + 32 <= td.row_hi);
-                uint16_t* crow = td.c + (int64_t)(rt + (lane >> 3)) * pb.ldc + wn * WTN + jh * 64 + (lane & 7) * 8;
-                if (all_rows) {
+                if constexpr (Problem::kMaskRows) {
+                    // Only rows [row_lo, row_hi) of the tile belong to this tile's group.  The stores go through a
+                    // buffer descriptor that spans exactly those rows: a lane whose row lies outside gets an
+                    // offset below zero (huge when read as unsigned) or past the end, and the hardware drops its
+                    // store - no divergent branches around the stores.
+                    const int voff = (rt + (lane >> 3) - td.row_lo) * ldc_bytes + (wn * WTN + jh * 64 + (lane & 7) * 8) * 2;
+#pragma unroll
+                    for (int it = 0; it < 4; ++it)
+                        __builtin_amdgcn_raw_buffer_store_b128(staged[it], c_rows, voff + it * 8 * ldc_bytes, 0, 0);
+                } else {
+                    uint16_t* crow = td.c + (int64_t)(rt + (lane >> 3)) * pb.ldc + wn * WTN + jh * 64 + (lane & 7) * 8;
 #pragma unroll
                     for (int it = 0; it < 4; ++it) *reinterpret_cast<v4i*>(crow + (int64_t)(it * 8) * pb.ldc) = staged[it];
-                } else {
-#pragma unroll
-                    for (int it = 0; it < 4; ++it) {
-                        const int trow = rt + it * 8 + (lane >> 3);
-                        if (trow >= td.row_lo && trow < td.row_hi)
-                            *reinterpret_cast<v4i*>(crow + (int64_t)(it * 8) * pb.ldc) = staged[it];
-                    }
                 }
                 __builtin_amdgcn_s_waitcnt(0xc07f);  // the reads are done before the next pass overwrites
                 __builtin_amdgcn_wave_barrier();
@@ -671,7 +678,8 @@ int launch_dma8_grouped(const uint8_t* a, int a_dtype, int64_t lda, const uint8_
     const int tiles_n = (N + BN - 1) / BN;
     GroupedProblem pb{a, b, out, lda, ldb, ldc, b_group_stride, sb_group_stride, sizes, E, T, N, K, tiles_n, sa, sb};
     const int64_t max_tiles = ((T + BM - 1) / BM + E) * tiles_n;
-    return launch_typed(pb, max_tiles > (1 << 30) ? (1 << 30) : (int)max_tiles, true, a_dtype, b_dtype, st);
+    return launch_typed<GroupedProblem, kGroupedWN>(pb, max_tiles > (1 << 30) ? (1 << 30) : (int)max_tiles, true, a_dtype,
+                                                        b_dtype, st);
 }
 
 int launch_dma8_grouped_wgrad(const uint8_t* a_t, int a_dtype, const uint8_t* b_t, int b_dtype, int64_t ld_t,
@@ -680,7 +688,7 @@ int launch_dma8_grouped_wgrad(const uint8_t* a_t, int a_dtype, const uint8_t* b_
 {
     const int tiles_n = (N + BM - 1) / BM, tiles_k = (Kl + BN - 1) / BN;
     GroupedWgradProblem pb{a_t, b_t, out, ld_t, ld_t, Kl, sizes, E, T, N, Kl, tiles_n, tiles_k, sa, sb};
-    return launch_typed(pb, E * tiles_n * tiles_k, false, a_dtype, b_dtype, st);
+    return launch_typed<GroupedWgradProblem, kGroupedWN>(pb, E * tiles_n * tiles_k, false, a_dtype, b_dtype, st);
 }
 
 }  // namespace gemm
