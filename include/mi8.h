@@ -75,6 +75,16 @@ int32_t mi8_amax_slots_for(int64_t n);
 int mi8_scale_from_partials(const uint32_t* slots, int32_t n_slots, int fp8_dtype, uint32_t flags, float* out,
                             void* stream);
 
+/* Tensorwise dynamic scales of many tensors in three launches: the once-per-optimizer-step refresh of all
+ * float8 weight scales (reference: torchao precompute_float8_dynamic_scale_for_fsdp, called from
+ * src/olmo_core/nn/transformer/model.py:1001-1008 when Float8Config.should_precompute_float8_dynamic_scale_for_fsdp,
+ * src/olmo_core/float8/__init__.py:54-62).
+ *   ptrs / numels: DEVICE arrays [n_tensors] of tensor base pointers (16-byte aligned) and element counts
+ *   (multiples of 8 for bf16, 4 for float32); amax_workspace: uint32 [n_tensors] (overwritten);
+ *   scales_out: float32 [n_tensors], the same values mi8_scale_from_partials gives tensor by tensor. */
+int mi8_multi_tensor_scales(const void* const* ptrs, const int64_t* numels, int32_t n_tensors, int hp_dtype,
+                            int fp8_dtype, uint32_t flags, uint32_t* amax_workspace, float* scales_out, void* stream);
+
 /* Saturating cast of x[rows, cols] with one scale for the whole tensor.
  *   scale source: if slots != NULL the scale is reduced from slots[0..n_slots) exactly as
  *   mi8_scale_from_partials does (and written to scale_out[0] if scale_out != NULL);

@@ -32,6 +32,10 @@ _SIGNATURES = {
     "mi8_amax_partials": (c_int, [c_void_p, c_int, c_int64, c_void_p, POINTER(c_int32), c_void_p]),
     "mi8_amax_slots_for": (c_int32, [c_int64]),
     "mi8_scale_from_partials": (c_int, [c_void_p, c_int32, c_int, c_uint32, c_void_p, c_void_p]),
+    "mi8_multi_tensor_scales": (
+        c_int,
+        [c_void_p, c_void_p, c_int32, c_int, c_int, c_uint32, c_void_p, c_void_p, c_void_p],
+    ),
     "mi8_cast_tensorwise": (
         c_int,
         [c_void_p, c_int, c_int64, c_int64, c_void_p, c_int32, c_void_p, c_int, c_uint32, c_void_p, c_int64,

@@ -595,6 +595,79 @@ extern "C" int mi8_amax_partials(const void* x, int hp_dtype, int64_t n, uint32_
     return launch_status("mi8_amax_partials");
 }
 
+namespace mi8 {
+namespace {
+
+// amax of many tensors in one launch (the per-optimizer-step scale refresh of all float8 weights): block
+// (chunk, tensor) folds its share of tensor `blockIdx.y` and merges it with an integer atomic maximum, which is
+// order-independent, so the result is deterministic.  Tensors must be 16-byte aligned with numel % 8 == 0 (bf16)
+// or % 4 == 0 (float32).
+template <int HP>
+__global__ __launch_bounds__(kThreads) void multi_amax_kernel(const void* const* __restrict__ ptrs,
+                                                              const int64_t* __restrict__ numels,
+                                                              uint32_t* __restrict__ amax_bits)
+{
+    __shared__ uint32_t smem[4];
+    const int t = blockIdx.y;
+    const uint4* x = reinterpret_cast<const uint4*>(ptrs[t]);
+    const int64_t nvec = numels[t] / (HP == MI8_BF16 ? 8 : 4);
+    uint32_t acc[4] = {0, 0, 0, 0};
+    const int64_t stride = (int64_t)gridDim.x * kThreads;
+    int64_t i = (int64_t)blockIdx.x * kThreads + threadIdx.x;
+    for (; i + 3 * stride < nvec; i += 4 * stride) {
+        uint4 v0 = x[i], v1 = x[i + stride], v2 = x[i + 2 * stride], v3 = x[i + 3 * stride];
+        absmax_accumulate<HP>(v0, acc);
+        absmax_accumulate<HP>(v1, acc);
+        absmax_accumulate<HP>(v2, acc);
+        absmax_accumulate<HP>(v3, acc);
+    }
+    for (; i < nvec; i += stride) absmax_accumulate<HP>(x[i], acc);
+    uint32_t m = block_umax(absmax_fold<HP>(acc), smem);
+    if (threadIdx.x == 0 && m) atomicMax(&amax_bits[t], m);
+}
+
+template <int FP8>
+__global__ void multi_scale_kernel(const uint32_t* __restrict__ amax_bits, int n, bool pow2, float* __restrict__ scales)
+{
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) scales[i] = scale_from_amax_bits<FP8>(amax_bits[i], pow2);
+}
+
+__global__ void zero_u32_kernel(uint32_t* p, int n)
+{
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) p[i] = 0;
+}
+
+}  // namespace
+}  // namespace mi8
+
+extern "C" int mi8_multi_tensor_scales(const void* const* ptrs, const int64_t* numels, int32_t n_tensors, int hp_dtype,
+                                       int fp8_dtype, uint32_t flags, uint32_t* amax_workspace, float* scales_out,
+                                       void* stream)
+{
+    MI8_REQUIRE(ptrs && numels && amax_workspace && scales_out, MI8_ERR_ARG, "mi8_multi_tensor_scales: null pointer");
+    MI8_REQUIRE(valid_hp(hp_dtype) && valid_fp8(fp8_dtype), MI8_ERR_ARG, "mi8_multi_tensor_scales: unknown dtype");
+    MI8_REQUIRE(n_tensors > 0 && n_tensors <= 65535, MI8_ERR_ARG, "mi8_multi_tensor_scales: %d tensors (1..65535)",
+                n_tensors);
+    hipStream_t st = (hipStream_t)stream;
+    const unsigned nb = (unsigned)ceil_div(n_tensors, 256);
+    hipLaunchKernelGGL(zero_u32_kernel, dim3(nb), dim3(256), 0, st, amax_workspace, n_tensors);
+    const dim3 grid(64, (unsigned)n_tensors);
+    if (hp_dtype == MI8_BF16)
+        hipLaunchKernelGGL((multi_amax_kernel<MI8_BF16>), grid, dim3(kThreads), 0, st, ptrs, numels, amax_workspace);
+    else
+        hipLaunchKernelGGL((multi_amax_kernel<MI8_F32>), grid, dim3(kThreads), 0, st, ptrs, numels, amax_workspace);
+    const bool pow2 = flags & MI8_FLAG_POW2_SCALE;
+    if (fp8_dtype == MI8_E4M3)
+        hipLaunchKernelGGL((multi_scale_kernel<MI8_E4M3>), dim3(nb), dim3(256), 0, st, amax_workspace, n_tensors, pow2,
+                           scales_out);
+    else
+        hipLaunchKernelGGL((multi_scale_kernel<MI8_E5M2>), dim3(nb), dim3(256), 0, st, amax_workspace, n_tensors, pow2,
+                           scales_out);
+    return launch_status("mi8_multi_tensor_scales");
+}
+
 extern "C" int mi8_scale_from_partials(const uint32_t* slots, int32_t n_slots, int fp8_dtype, uint32_t flags,
                                        float* out, void* stream)
 {

@@ -19,7 +19,20 @@ from ..config import Config
 from ..exceptions import OLMoConfigurationError
 from .ao import AOFloat8LinearConfig, AOFloat8LinearRecipe, AOMXLinearConfig
 
-__all__ = ["Float8Config", "AOFloat8LinearConfig", "AOFloat8LinearRecipe", "AOMXLinearConfig"]
+__all__ = [
+    "Float8Config",
+    "AOFloat8LinearConfig",
+    "AOFloat8LinearRecipe",
+    "AOMXLinearConfig",
+    "precompute_float8_dynamic_scale_for_fsdp",
+]
+
+
+def precompute_float8_dynamic_scale_for_fsdp(module: nn.Module) -> None:
+    """See :func:`olmo_core_amd.float8.linear.precompute_float8_dynamic_scale_for_fsdp`."""
+    from .linear import precompute_float8_dynamic_scale_for_fsdp as impl
+
+    impl(module)
 
 log = logging.getLogger(__name__)
 

@@ -69,7 +69,7 @@ class _Float8Matmul(torch.autograd.Function):
     """y = x @ W^T with float8 operands; x [M, K] and W [N, K] in high precision."""
 
     @staticmethod
-    def forward(ctx, x2: torch.Tensor, weight: torch.Tensor, config: Float8LinearConfig):
+    def forward(ctx, x2: torch.Tensor, weight: torch.Tensor, config: Float8LinearConfig, weight_scale=None):
         c = config
         pow2 = c.round_scales_to_power_of_2
         need_gx = ctx.needs_input_grad[0]
@@ -97,7 +97,8 @@ class _Float8Matmul(torch.autograd.Function):
                 xq, sx = ops.cast_rowwise(x2, c.cast_config_input.target_dtype, pow2=pow2)
             if _is_tensorwise(c.cast_config_weight):
                 wq, wq_t, sw = ops.cast_tensorwise(
-                    weight, c.cast_config_weight.target_dtype, pow2=pow2, want_rowmajor=True, want_transposed=share_w
+                    weight, c.cast_config_weight.target_dtype, pow2=pow2, want_rowmajor=True, want_transposed=share_w,
+                    scale=weight_scale,
                 )
                 if share_w:
                     w_saved, w_is_q = (wq_t, sw), True
@@ -161,12 +162,17 @@ class _Float8Matmul(torch.autograd.Function):
                 gw = ops.gemm_fp8(go_cols[0], go_cols[1], x_op[0], x_op[1], out_dtype=ctx.x_dtype)
             if gw.dtype != ctx.w_dtype:
                 gw = gw.to(ctx.w_dtype)
-        return gx, gw, None
+        return gx, gw, None, None
 
 
 @torch.compiler.disable
-def float8_linear_function(x: torch.Tensor, weight: torch.Tensor, config: Float8LinearConfig) -> torch.Tensor:
+def float8_linear_function(
+    x: torch.Tensor, weight: torch.Tensor, config: Float8LinearConfig, weight_scale: Optional[torch.Tensor] = None
+) -> torch.Tensor:
     """``x [*, K] @ weight[N, K].T`` through the float8 path, differentiable in x and weight.
+
+    ``weight_scale``: a precomputed tensorwise scale of ``weight`` (float32 ``[1]``), used instead of reducing the
+    weight's amax again; ignored unless the weight cast is tensorwise.
 
     Opaque to ``torch.compile`` (a graph break per call): the kernels are reached through ctypes, which Dynamo
     cannot trace; the reference takes the same route for its grouped GEMM (``src/olmo_core/nn/moe/mlp.py:256``).
@@ -175,7 +181,7 @@ def float8_linear_function(x: torch.Tensor, weight: torch.Tensor, config: Float8
     if weight.dim() != 2 or weight.shape[1] != K:
         raise ValueError(f"float8 linear: input features {K} do not match weight {tuple(weight.shape)}")
     x2 = x.reshape(-1, K)
-    y = _Float8Matmul.apply(x2, weight, config)
+    y = _Float8Matmul.apply(x2, weight, config, weight_scale)
     return y.reshape(*x.shape[:-1], weight.shape[0])
 
 
@@ -199,10 +205,22 @@ class Float8Linear(nn.Linear):
     def forward(self, input: torch.Tensor) -> torch.Tensor:
         if torch.is_autocast_enabled():
             input = input.to(torch.get_autocast_dtype(input.device.type))
-        out = float8_linear_function(input, self.weight, self.config)
+        out = float8_linear_function(input, self.weight, self.config, self.precomputed_weight_scale())
         if self.bias is not None:
             out = out + self.bias.to(out.dtype)
         return out
+
+    def precomputed_weight_scale(self) -> Optional[torch.Tensor]:
+        """The scale stored by :func:`precompute_float8_dynamic_scale_for_fsdp` if the weight has not been
+        modified (or replaced) since; ``None`` otherwise, and the forward then reduces the amax itself."""
+        entry = getattr(self, "_precomputed_weight_scale", None)
+        if entry is None:
+            return None
+        scale, ptr, version = entry
+        w = self.weight
+        if w.data_ptr() != ptr or w._version != version or not _is_tensorwise(self.config.cast_config_weight):
+            return None
+        return scale
 
     def extra_repr(self) -> str:
         c = self.config
@@ -274,3 +292,32 @@ def convert_to_float8_training(
     """
     config = config if config is not None else Float8LinearConfig()
     return _swap(module, lambda m: Float8Linear.from_float(m, config), module_filter_fn)
+
+
+def precompute_float8_dynamic_scale_for_fsdp(module: nn.Module) -> None:
+    """
+    Refresh the tensorwise weight scales of every :class:`Float8Linear` under ``module`` in one batch of kernel
+    launches; call it right after the optimizer step (reference: torchao's function of the same name, called
+    from ``src/olmo_core/nn/transformer/model.py:1001-1008``).  Forwards then skip the weight's amax pass until
+    the weight changes again; the scales are the ones the forward would compute itself, bit for bit.
+    """
+    groups: dict = {}
+    for m in module.modules():
+        if not isinstance(m, Float8Linear):
+            continue
+        m._precomputed_weight_scale = None
+        c = m.config
+        w = m.weight
+        if not _is_tensorwise(c.cast_config_weight) or not w.is_cuda or not w.is_contiguous():
+            continue
+        if w.dtype not in (torch.bfloat16, torch.float32) or w.data_ptr() % 16:
+            continue
+        key = (w.device, w.dtype, c.cast_config_weight.target_dtype, c.round_scales_to_power_of_2)
+        groups.setdefault(key, []).append(m)
+    for (_, _, fp8_dtype, pow2), mods in groups.items():
+        for start in range(0, len(mods), 65535):
+            chunk = mods[start:start + 65535]
+            with torch.no_grad():
+                scales = ops.multi_tensor_scales([m.weight.detach() for m in chunk], fp8_dtype, pow2=pow2)
+            for i, m in enumerate(chunk):
+                m._precomputed_weight_scale = (scales[i:i + 1], m.weight.data_ptr(), m.weight._version)

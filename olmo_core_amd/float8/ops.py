@@ -87,6 +87,32 @@ def tensor_to_scale(x: torch.Tensor, fp8_dtype: torch.dtype, pow2: bool = False)
     return scale_from_partials(slots, used, fp8_dtype, pow2)[0]
 
 
+def multi_tensor_scales(tensors, fp8_dtype: torch.dtype, pow2: bool = False) -> torch.Tensor:
+    """Tensorwise dynamic scales of a list of same-dtype GPU tensors in one batch of launches: float32 ``[n]``."""
+    if not tensors:
+        raise ValueError("multi_tensor_scales: no tensors")
+    t0 = tensors[0]
+    _require_gpu(t0, "multi_tensor_scales")
+    step = 8 if t0.dtype == torch.bfloat16 else 4
+    for t in tensors:
+        if t.dtype != t0.dtype or t.dtype not in _HP_CODE or t.device != t0.device or not t.is_contiguous():
+            raise ValueError("multi_tensor_scales: tensors must be contiguous, on one GPU and of one dtype (bf16 or fp32)")
+        if t.numel() % step or t.data_ptr() % 16:
+            raise ValueError("multi_tensor_scales: every tensor needs 16-byte alignment and a multiple of 16 bytes")
+    n = len(tensors)
+    table = torch.tensor([[t.data_ptr() for t in tensors], [t.numel() for t in tensors]], dtype=torch.int64).to(t0.device)
+    ws = torch.empty(n, dtype=torch.int32, device=t0.device)
+    out = torch.empty(n, dtype=torch.float32, device=t0.device)
+    _C.check(
+        _C.lib().mi8_multi_tensor_scales(
+            table[0].data_ptr(), table[1].data_ptr(), n, _HP_CODE[t0.dtype], _FP8_CODE[fp8_dtype], _flags(pow2),
+            ws.data_ptr(), out.data_ptr(), _stream(t0),
+        ),
+        "mi8_multi_tensor_scales",
+    )
+    return out
+
+
 def _operand(shape: Tuple[int, int], fp8_dtype: torch.dtype, device, pitch: Optional[int] = None) -> torch.Tensor:
     """Uninitialised fp8 ``[rows, k]`` GEMM operand; with ``pitch > k`` a view of a wider buffer (the kernels take
     any row pitch that is a multiple of 16)."""

@@ -208,3 +208,50 @@ def test_torch_compile_composes(dev):
     assert torch.allclose(y1.float(), y0.float(), rtol=2e-2, atol=2e-2)  # inductor may fuse the bf16 pointwise parts differently
     assert torch.allclose(x.grad.float(), g0.float(), rtol=5e-2, atol=5e-2)
     assert torch.allclose(m.w1.weight.grad.float(), gw0.float(), rtol=5e-2, atol=5e-2)
+
+
+def test_precomputed_weight_scales(dev):
+    """precompute_float8_dynamic_scale_for_fsdp (reference: model.post_optim_step,
+    src/olmo_core/nn/transformer/model.py:1001-1008): one batch of launches gives every weight the scale its
+    forward would compute, forwards with it are bit-identical, and a scale goes stale with the weight."""
+    import torch.nn as nn
+
+    from olmo_core_amd.float8 import Float8Config, precompute_float8_dynamic_scale_for_fsdp
+    from olmo_core_amd.float8.linear import Float8Linear
+    from olmo_core_amd.nn import FeedForward
+
+    torch.manual_seed(1)
+    model = nn.ModuleDict(
+        {
+            "ff": FeedForward(d_model=256, hidden_size=512, bias=False, dtype=torch.bfloat16),
+            "proj": nn.Linear(256, 128, bias=True, dtype=torch.float32),
+            "odd": nn.Linear(256, 24, bias=False, dtype=torch.bfloat16),  # 24 % 16 != 0: left unconverted
+        }
+    ).to(dev)
+    with torch.no_grad():
+        model["proj"].weight.mul_(37.0)
+    Float8Config(enabled=True).apply_float8_linear(model)
+    lins = [m for m in model.modules() if isinstance(m, Float8Linear)]
+    assert len(lins) == 4
+    x = torch.randn(192, 256, device=dev, dtype=torch.bfloat16)
+    before = (model["ff"](x), model["proj"](x.float()))
+    precompute_float8_dynamic_scale_for_fsdp(model)
+    for m in lins:
+        s = m.precomputed_weight_scale()
+        assert s is not None and s.shape == (1,)
+        ref = ops.tensor_to_scale(m.weight.detach(), torch.float8_e4m3fn)
+        assert_scale_equal(s, ref.reshape(1), "precomputed weight scale")
+    after = (model["ff"](x), model["proj"](x.float()))
+    assert torch.equal(before[0], after[0]) and torch.equal(before[1], after[1])
+    # gradients flow as before
+    xg = x.clone().requires_grad_(True)
+    model["ff"](xg).float().sum().backward()
+    assert xg.grad is not None and model["ff"].w1.weight.grad is not None
+    # an optimizer step (any in-place update) invalidates the stored scale of that weight
+    with torch.no_grad():
+        model["proj"].weight.mul_(0.5)
+    assert model["proj"].precomputed_weight_scale() is None
+    assert model["ff"].w1.precomputed_weight_scale() is not None
+    out = model["proj"](x.float())
+    precompute_float8_dynamic_scale_for_fsdp(model)
+    assert torch.equal(out, model["proj"](x.float()))
