@@ -46,7 +46,7 @@ def build_mlp(dev):
     return mlp, x, go
 
 
-# ---- the other BASELINE configurations (parity-test shapes; measured with --config N for the design notes) ----
+# ---- the other benchmark configurations (parity-test shapes; measured with --config N) ----
 
 
 def build_config(n, dev):
@@ -238,7 +238,7 @@ def main():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--config", type=int, default=2, help="BASELINE configuration 1..5 (2 is the benchmark line)")
+    ap.add_argument("--config", type=int, default=2, help="benchmark configuration 1..5 (2 is the headline line)")
     ap.add_argument("--traffic-probe", action="store_true", help="workload for the FETCH_SIZE/WRITE_SIZE counter runs")
     ns = ap.parse_args()
     if ns.gpus != 1:
