@@ -207,7 +207,7 @@ extern "C" int mi8_grouped_gemm_fp8(const void* a, int a_dtype, int64_t lda, con
     hipStream_t st = (hipStream_t)stream;
     // full-tile shapes with bf16 output run on the persistent direct-to-LDS kernel
     if (out_dtype == MI8_BF16 && T >= 256 && N >= 256 && K % 128 == 0 && N % 8 == 0 && ldc % 8 == 0 && aligned16(out) &&
-        sb_group_stride % 4 == 0 && aligned16(sb) && lda < (1 << 23) && ldb < (1 << 23))
+        sb_group_stride % 4 == 0 && aligned16(sb) && lda < (1 << 23) && ldb < (1 << 23) && ldc < (1 << 22))
         return launch_dma8_grouped((const uint8_t*)a, a_dtype, lda, (const uint8_t*)b, b_dtype, ldb, b_group_stride,
                                    group_sizes, num_groups, T, (int)N, (int)K, sa, sb, sb_group_stride, (uint16_t*)out,
                                    ldc, st);

@@ -1,0 +1,101 @@
+"""
+The float8 linear as registered custom operators, for ``torch.compile``.
+
+A ctypes call is opaque to Dynamo; wrapped in ``torch.library.custom_op`` with a shape function it becomes one
+node of the traced graph, so that compiled blocks (the reference compiles every transformer block,
+``src/olmo_core/nn/transformer/block.py:78-79``) keep a single graph around their float8 linears.  The operators
+call the same forward / backward routines as the eager ``autograd.Function``.
+"""
+
+from __future__ import annotations
+
+from typing import Optional, Tuple
+
+import torch
+
+from . import ops
+from .linear import _COMPILED_CONFIGS, _backward_impl, _forward_impl, _saves_quantised
+
+_CONFIGS = _COMPILED_CONFIGS  # configs travel through the operators as indices into this list
+
+
+@torch.library.custom_op("olmo_core_amd::float8_linear_fwd", mutates_args=())
+def _linear_fwd(
+    x2: torch.Tensor, weight: torch.Tensor, weight_scale: Optional[torch.Tensor], cfg: int, need_gx: bool, need_gw: bool
+) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]:
+    y, x_saved, w_saved = _forward_impl(x2, weight, _CONFIGS[cfg], weight_scale, need_gx, need_gw)
+    xa, xb = x_saved if x_saved is not None else (x2.new_empty(0), x2.new_empty(0))
+    wa, wb = w_saved if w_saved is not None else (x2.new_empty(0), x2.new_empty(0))
+    return y, xa, xb, wa, wb
+
+
+@_linear_fwd.register_fake
+def _(x2, weight, weight_scale, cfg, need_gx, need_gw):
+    c = _CONFIGS[cfg]
+    M, K = x2.shape
+    N = weight.shape[0]
+    x_is_q, w_is_q = _saves_quantised(c, need_gx, need_gw)
+
+    def saved(is_q, rows, cols, dtype):
+        if not is_q:
+            return x2.new_empty(0), x2.new_empty(0)
+        return x2.new_empty((cols, (rows + 15) // 16 * 16), dtype=dtype), x2.new_empty(1, dtype=torch.float32)
+
+    xa, xb = saved(x_is_q, M, K, c.cast_config_input.target_dtype)
+    wa, wb = saved(w_is_q, N, K, c.cast_config_weight.target_dtype)
+    return x2.new_empty((M, N)), xa, xb, wa, wb
+
+
+@torch.library.custom_op("olmo_core_amd::float8_linear_bwd", mutates_args=())
+def _linear_bwd(
+    go: torch.Tensor, xa: torch.Tensor, xb: torch.Tensor, wa: torch.Tensor, wb: torch.Tensor, cfg: int, n: int,
+    x_is_q: bool, w_is_q: bool, need_gx: bool, need_gw: bool, x_dtype: torch.dtype, w_dtype: torch.dtype,
+) -> Tuple[torch.Tensor, torch.Tensor]:
+    gx, gw = _backward_impl(go, _CONFIGS[cfg], n, x_dtype, w_dtype, (xa, xb), (wa, wb), x_is_q, w_is_q, need_gx, need_gw)
+    return (gx if gx is not None else go.new_empty(0)), (gw if gw is not None else go.new_empty(0))
+
+
+@_linear_bwd.register_fake
+def _(go, xa, xb, wa, wb, cfg, n, x_is_q, w_is_q, need_gx, need_gw, x_dtype, w_dtype):
+    M = go.shape[0]
+    if x_is_q:
+        K = xa.shape[0]
+    elif need_gw:
+        K = xa.shape[1]
+    elif w_is_q:
+        K = wa.shape[0]
+    else:
+        K = wa.shape[1]
+    gx = go.new_empty((M, K), dtype=x_dtype) if need_gx else go.new_empty(0)
+    gw = go.new_empty((n, K), dtype=w_dtype) if need_gw else go.new_empty(0)
+    return gx, gw
+
+
+def _setup_context(ctx, inputs, output):
+    x2, weight, _, cfg, need_gx, need_gw = inputs
+    _, xa, xb, wa, wb = output
+    x_is_q, w_is_q = _saves_quantised(_CONFIGS[cfg], need_gx, need_gw)
+    ctx.meta = (cfg, weight.shape[0], x_is_q, w_is_q, need_gx, need_gw, x2.dtype, weight.dtype)
+    empty = xb  # a tensor to fill unused slots with
+    x_part = (xa, xb) if x_is_q else ((x2, empty) if need_gw else (empty, empty))
+    w_part = (wa, wb) if w_is_q else ((weight, empty) if need_gx else (empty, empty))
+    ctx.save_for_backward(*x_part, *w_part)
+
+
+def _backward(ctx, gy, *unused):
+    cfg, n, x_is_q, w_is_q, need_gx, need_gw, x_dtype, w_dtype = ctx.meta
+    xa, xb, wa, wb = ctx.saved_tensors
+    gx, gw = _linear_bwd(gy.contiguous(), xa, xb, wa, wb, cfg, n, x_is_q, w_is_q, need_gx, need_gw, x_dtype, w_dtype)
+    return (gx if need_gx else None), (gw if need_gw else None), None, None, None, None
+
+
+_linear_fwd.register_autograd(_backward, setup_context=_setup_context)
+
+
+def linear(x2: torch.Tensor, weight: torch.Tensor, cfg_id: int, weight_scale: Optional[torch.Tensor]):
+    """``x2 [M, K] @ weight[N, K].T`` as a traceable operator call; ``cfg_id`` indexes the registered configs."""
+    out = _linear_fwd(x2, weight, weight_scale, cfg_id, x2.requires_grad, weight.requires_grad)
+    return out[0]
+
+
+__all__ = ["linear", "ops"]

@@ -65,107 +65,130 @@ def _cols_operand(x: torch.Tensor, c: CastConfig, pow2: bool) -> Tuple[torch.Ten
     return ops.cast_colwise_t(x, c.target_dtype, pow2=pow2)
 
 
+def _saves_quantised(c: Float8LinearConfig, need_gx: bool, need_gw: bool) -> Tuple[bool, bool]:
+    """Whether the forward keeps the transposed fp8 copy (+ scale) of x / of the weight for the backward instead
+    of the high-precision tensor: possible when forward and backward quantise that tensor identically."""
+    if _is_disabled(c.cast_config_input):
+        return False, False
+    x_is_q = need_gw and _shared_tensorwise(c.cast_config_input, c.cast_config_input_for_grad_weight)
+    w_is_q = need_gx and _shared_tensorwise(c.cast_config_weight, c.cast_config_weight_for_grad_input)
+    return x_is_q, w_is_q
+
+
+def _forward_impl(x2, weight, c: Float8LinearConfig, weight_scale, need_gx: bool, need_gw: bool):
+    """y = x2 @ weight^T in float8.  Returns ``(y, x_saved, w_saved)``: the tensors the backward needs for x and
+    for the weight, each either ``(q_t, scale)`` (see :func:`_saves_quantised`) or ``None`` (keep the input)."""
+    pow2 = c.round_scales_to_power_of_2
+    share_x, share_w = _saves_quantised(c, need_gx, need_gw)
+    x_saved = w_saved = None
+    if _is_disabled(c.cast_config_input):
+        return torch.mm(x2, weight.t().to(x2.dtype)), None, None
+    if _is_tensorwise(c.cast_config_input):
+        xq, xq_t, sx = ops.cast_tensorwise(
+            x2, c.cast_config_input.target_dtype, pow2=pow2, want_rowmajor=True, want_transposed=share_x
+        )
+        if share_x:
+            x_saved = (xq_t, sx)
+    else:
+        xq, sx = ops.cast_rowwise(x2, c.cast_config_input.target_dtype, pow2=pow2)
+    if _is_tensorwise(c.cast_config_weight):
+        wq, wq_t, sw = ops.cast_tensorwise(
+            weight, c.cast_config_weight.target_dtype, pow2=pow2, want_rowmajor=True, want_transposed=share_w,
+            scale=weight_scale,
+        )
+        if share_w:
+            w_saved = (wq_t, sw)
+    else:
+        wq, sw = ops.cast_rowwise(weight, c.cast_config_weight.target_dtype, pow2=pow2)
+    return ops.gemm_fp8(xq, sx, wq, sw, out_dtype=x2.dtype), x_saved, w_saved
+
+
+def _backward_impl(go2, c: Float8LinearConfig, N: int, x_dtype, w_dtype, x_part, w_part, x_is_q: bool, w_is_q: bool,
+                   need_gx: bool, need_gw: bool):
+    """grad_input and grad_weight from grad_output ``go2 [M, N]``; ``x_part`` / ``w_part`` are what the forward
+    kept: ``(q_t, scale)`` if the flag says so, else ``(tensor,)``."""
+    pow2 = c.round_scales_to_power_of_2
+    if go2.dtype != x_dtype:
+        go2 = go2.to(x_dtype)
+    # quantise grad_output once if both backward GEMMs want the same tensorwise cast
+    go_rows = go_cols = None
+    cg, cgw = c.cast_config_grad_output, c.cast_config_grad_output_for_grad_weight
+    if need_gx and need_gw and _shared_tensorwise(cg, cgw):
+        q, q_t, s = ops.cast_tensorwise(go2, cg.target_dtype, pow2=pow2, want_rowmajor=True, want_transposed=True)
+        go_rows, go_cols = (q, s), (q_t, s)
+
+    gx = gw = None
+    if need_gx:
+        if _is_disabled(cg):
+            gx = torch.mm(go2, w_part[0].to(go2.dtype))
+        else:
+            if go_rows is None:
+                go_rows = _rows_operand(go2, cg, pow2)
+            w_op = (w_part[0], w_part[1]) if w_is_q else _cols_operand(w_part[0], c.cast_config_weight_for_grad_input, pow2)
+            gx = ops.gemm_fp8(go_rows[0], go_rows[1], w_op[0], w_op[1], k=N, out_dtype=x_dtype)
+    if need_gw:
+        if _is_disabled(cgw):
+            gw = torch.mm(go2.t(), x_part[0].to(go2.dtype))
+        else:
+            if go_cols is None:
+                go_cols = _cols_operand(go2, cgw, pow2)
+            x_op = (x_part[0], x_part[1]) if x_is_q else _cols_operand(x_part[0], c.cast_config_input_for_grad_weight, pow2)
+            gw = ops.gemm_fp8(go_cols[0], go_cols[1], x_op[0], x_op[1], out_dtype=x_dtype)
+        if gw.dtype != w_dtype:
+            gw = gw.to(w_dtype)
+    return gx, gw
+
+
 class _Float8Matmul(torch.autograd.Function):
     """y = x @ W^T with float8 operands; x [M, K] and W [N, K] in high precision."""
 
     @staticmethod
     def forward(ctx, x2: torch.Tensor, weight: torch.Tensor, config: Float8LinearConfig, weight_scale=None):
-        c = config
-        pow2 = c.round_scales_to_power_of_2
-        need_gx = ctx.needs_input_grad[0]
-        need_gw = ctx.needs_input_grad[1]
-        ctx.config = c
-        ctx.x_dtype = x2.dtype
-        ctx.w_dtype = weight.dtype
+        need_gx, need_gw = ctx.needs_input_grad[0], ctx.needs_input_grad[1]
+        y, x_saved, w_saved = _forward_impl(x2, weight, config, weight_scale, need_gx, need_gw)
+        ctx.config = config
+        ctx.x_dtype, ctx.w_dtype = x2.dtype, weight.dtype
         ctx.shapes = (x2.shape[0], x2.shape[1], weight.shape[0])
-        out_dtype = x2.dtype
-
-        x_saved = w_saved = None
-        x_is_q = w_is_q = False
-        if _is_disabled(c.cast_config_input):
-            y = torch.mm(x2, weight.t().to(x2.dtype))
-        else:
-            share_x = need_gw and _shared_tensorwise(c.cast_config_input, c.cast_config_input_for_grad_weight)
-            share_w = need_gx and _shared_tensorwise(c.cast_config_weight, c.cast_config_weight_for_grad_input)
-            if _is_tensorwise(c.cast_config_input):
-                xq, xq_t, sx = ops.cast_tensorwise(
-                    x2, c.cast_config_input.target_dtype, pow2=pow2, want_rowmajor=True, want_transposed=share_x
-                )
-                if share_x:
-                    x_saved, x_is_q = (xq_t, sx), True
-            else:
-                xq, sx = ops.cast_rowwise(x2, c.cast_config_input.target_dtype, pow2=pow2)
-            if _is_tensorwise(c.cast_config_weight):
-                wq, wq_t, sw = ops.cast_tensorwise(
-                    weight, c.cast_config_weight.target_dtype, pow2=pow2, want_rowmajor=True, want_transposed=share_w,
-                    scale=weight_scale,
-                )
-                if share_w:
-                    w_saved, w_is_q = (wq_t, sw), True
-            else:
-                wq, sw = ops.cast_rowwise(weight, c.cast_config_weight.target_dtype, pow2=pow2)
-            y = ops.gemm_fp8(xq, sx, wq, sw, out_dtype=out_dtype)
-
-        ctx.x_is_q, ctx.w_is_q = x_is_q, w_is_q
+        ctx.x_is_q, ctx.w_is_q = x_saved is not None, w_saved is not None
         to_save = []
         if need_gw:
-            to_save += list(x_saved) if x_is_q else [x2]
+            to_save += list(x_saved) if ctx.x_is_q else [x2]
         if need_gx:
-            to_save += list(w_saved) if w_is_q else [weight]
-        ctx.n_x = (2 if x_is_q else 1) if need_gw else 0
+            to_save += list(w_saved) if ctx.w_is_q else [weight]
+        ctx.n_x = (2 if ctx.x_is_q else 1) if need_gw else 0
         ctx.save_for_backward(*to_save)
         return y
 
     @staticmethod
     def backward(ctx, go: torch.Tensor):
-        c: Float8LinearConfig = ctx.config
-        pow2 = c.round_scales_to_power_of_2
         M, K, N = ctx.shapes
-        need_gx, need_gw = ctx.needs_input_grad[0], ctx.needs_input_grad[1]
         saved = ctx.saved_tensors
-        x_part, w_part = saved[: ctx.n_x], saved[ctx.n_x :]
-        go2 = go.reshape(M, N)
-        if go2.dtype != ctx.x_dtype:
-            go2 = go2.to(ctx.x_dtype)
-
-        # quantise grad_output once if both backward GEMMs want the same tensorwise cast
-        go_rows = go_cols = None
-        cg, cgw = c.cast_config_grad_output, c.cast_config_grad_output_for_grad_weight
-        if need_gx and need_gw and _shared_tensorwise(cg, cgw):
-            q, q_t, s = ops.cast_tensorwise(go2, cg.target_dtype, pow2=pow2, want_rowmajor=True, want_transposed=True)
-            go_rows, go_cols = (q, s), (q_t, s)
-
-        gx = gw = None
-        if need_gx:
-            if _is_disabled(cg):
-                w = w_part[0]
-                gx = torch.mm(go2, w.to(go2.dtype))
-            else:
-                if go_rows is None:
-                    go_rows = _rows_operand(go2, cg, pow2)
-                if ctx.w_is_q:
-                    w_op = (w_part[0], w_part[1])
-                else:
-                    w_op = _cols_operand(w_part[0], c.cast_config_weight_for_grad_input, pow2)
-                gx = ops.gemm_fp8(go_rows[0], go_rows[1], w_op[0], w_op[1], k=N, out_dtype=ctx.x_dtype)
-        if need_gw:
-            if _is_disabled(cgw):
-                x2 = x_part[0]
-                gw = torch.mm(go2.t(), x2.to(go2.dtype))
-            else:
-                if go_cols is None:
-                    go_cols = _cols_operand(go2, cgw, pow2)
-                if ctx.x_is_q:
-                    x_op = (x_part[0], x_part[1])
-                else:
-                    x_op = _cols_operand(x_part[0], c.cast_config_input_for_grad_weight, pow2)
-                gw = ops.gemm_fp8(go_cols[0], go_cols[1], x_op[0], x_op[1], out_dtype=ctx.x_dtype)
-            if gw.dtype != ctx.w_dtype:
-                gw = gw.to(ctx.w_dtype)
+        gx, gw = _backward_impl(
+            go.reshape(M, N), ctx.config, N, ctx.x_dtype, ctx.w_dtype, saved[: ctx.n_x], saved[ctx.n_x :],
+            ctx.x_is_q, ctx.w_is_q, ctx.needs_input_grad[0], ctx.needs_input_grad[1],
+        )
         return gx, gw, None, None
 
 
+# Operator arguments must be plain values: under torch.compile a config travels as its index in this list.  Configs
+# are registered when a module is built (tracing must not mutate the list).
+_COMPILED_CONFIGS: list = []
+
+
+def _register_config(c: Float8LinearConfig) -> int:
+    idx = getattr(c, "_compiled_id", None)
+    if idx is None:
+        _COMPILED_CONFIGS.append(c)
+        idx = len(_COMPILED_CONFIGS) - 1
+        c._compiled_id = idx
+    return idx
+
+
 @torch.compiler.disable
+def _eager_matmul(x2, weight, config, weight_scale):
+    return _Float8Matmul.apply(x2, weight, config, weight_scale)
+
+
 def float8_linear_function(
     x: torch.Tensor, weight: torch.Tensor, config: Float8LinearConfig, weight_scale: Optional[torch.Tensor] = None
 ) -> torch.Tensor:
@@ -174,14 +197,20 @@ def float8_linear_function(
     ``weight_scale``: a precomputed tensorwise scale of ``weight`` (float32 ``[1]``), used instead of reducing the
     weight's amax again; ignored unless the weight cast is tensorwise.
 
-    Opaque to ``torch.compile`` (a graph break per call): the kernels are reached through ctypes, which Dynamo
-    cannot trace; the reference takes the same route for its grouped GEMM (``src/olmo_core/nn/moe/mlp.py:256``).
+    Under ``torch.compile`` the call becomes a pair of registered custom operators (forward, backward) with shape
+    functions, so a compiled block keeps one graph; eagerly it is an ordinary ``autograd.Function``.
     """
     K = x.shape[-1]
     if weight.dim() != 2 or weight.shape[1] != K:
         raise ValueError(f"float8 linear: input features {K} do not match weight {tuple(weight.shape)}")
     x2 = x.reshape(-1, K)
-    y = _Float8Matmul.apply(x2, weight, config, weight_scale)
+    cfg_id = getattr(config, "_compiled_id", -1)
+    if torch.compiler.is_compiling() and cfg_id >= 0:
+        from . import compiled
+
+        y = compiled.linear(x2, weight, cfg_id, weight_scale)
+    else:  # eager, or a config no module registered: a graph break
+        y = _eager_matmul(x2, weight, config, weight_scale)
     return y.reshape(*x.shape[:-1], weight.shape[0])
 
 
@@ -198,6 +227,7 @@ class Float8Linear(nn.Linear):
 
     def _bind_config(self) -> None:
         c = self.config
+        _register_config(c)
         self.scaling_type_input = c.cast_config_input.scaling_type
         self.scaling_type_weight = c.cast_config_weight.scaling_type
         self.scaling_type_grad_output = c.cast_config_grad_output.scaling_type
@@ -205,7 +235,9 @@ class Float8Linear(nn.Linear):
     def forward(self, input: torch.Tensor) -> torch.Tensor:
         if torch.is_autocast_enabled():
             input = input.to(torch.get_autocast_dtype(input.device.type))
-        out = float8_linear_function(input, self.weight, self.config, self.precomputed_weight_scale())
+        # (the stored scale is checked against the weight's address and version counter: not traceable)
+        scale = None if torch.compiler.is_compiling() else self.precomputed_weight_scale()
+        out = float8_linear_function(input, self.weight, self.config, scale)
         if self.bias is not None:
             out = out + self.bias.to(out.dtype)
         return out

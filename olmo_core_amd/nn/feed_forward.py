@@ -156,14 +156,15 @@ class FeedForward(nn.Module):
         self.w3 = nn.Linear(d_model, hidden_size, bias=bias, dtype=dtype, device=init_device)
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
-        if self.fuse_float8 and _fusable(self, x):
+        compiling = torch.compiler.is_compiling()  # traced graphs take the per-linear operators
+        if self.fuse_float8 and not compiling and _fusable(self, x):
             x2 = x.reshape(-1, x.shape[-1])
             y = _fused_mlp(x2, self.w1.weight, self.w2.weight, self.w3.weight, self.w1.config,
                            self.w1.precomputed_weight_scale(), self.w2.precomputed_weight_scale(),
                            self.w3.precomputed_weight_scale())
             return y.reshape(*x.shape[:-1], self.w2.weight.shape[0])
         x1, x3 = self.w1(x), self.w3(x)
-        if x1.is_cuda and x1.dtype == torch.bfloat16:
+        if x1.is_cuda and x1.dtype == torch.bfloat16 and not compiling:
             h = swiglu(x1, x3)
         else:
             h = torch.nn.functional.silu(x1) * x3
