@@ -160,6 +160,17 @@ int mi8_grouped_cast_colwise_t(const void* x, int hp_dtype, int64_t T, int64_t c
                                int32_t num_groups, int fp8_dtype, uint32_t flags, uint32_t* amax_ws, void* out_t,
                                int64_t ld_t, float* scale_out, void* stream);
 
+/* The same two passes (amax, cast) also produce the per-row cast of x that the forward / grad_input GEMMs take:
+ * out_rows fp8 [T, ld_rows] row-major with one scale per row (row_scale_out float32 [T], the values
+ * mi8_cast_rowwise gives), saving the separate pass over x.  row_amax_ws: uint32 [T], ZERO on entry.  Both
+ * products use fp8_dtype and flags.  Rows beyond the last group (if the sizes sum to less than T) are not
+ * written. */
+int mi8_grouped_cast_rows_and_colwise_t(const void* x, int hp_dtype, int64_t T, int64_t cols,
+                                        const int64_t* group_sizes, int32_t num_groups, int fp8_dtype, uint32_t flags,
+                                        uint32_t* amax_ws, void* out_t, int64_t ld_t, float* scale_out,
+                                        uint32_t* row_amax_ws, void* out_rows, int64_t ld_rows, float* row_scale_out,
+                                        void* stream);
+
 /* out[R_e, :N] = (A[R_e, :K] . B_e[:N, :K]^T) / sa[r] / sb_e[n]   for every group e.
  *   A fp8 [T, lda]; B_e = b + e * b_group_stride (bytes), N rows of pitch ldb; sa float32 [T];
  *   sb_e = sb + e * sb_group_stride (floats), N values; out [T, ldc] of out_dtype. */

@@ -146,7 +146,8 @@ __device__ __forceinline__ int tile_lds_chunk(int col, int part /* 0..7: which 1
 template <int HP, int FP8, bool SW>
 __device__ __forceinline__ void tile_cast_body(const void* x, int64_t row_end, int64_t cols, int64_t row0, int64_t col0,
                                                const float (&sc)[8], uint8_t* out, int64_t ld_out, uint8_t* out_t, int64_t ld_t,
-                                               int64_t dst0, int64_t dst_end, uint32_t* lds_t)
+                                               int64_t dst0, int64_t dst_end, uint32_t* lds_t,
+                                               uint8_t* out_r = nullptr, int64_t ld_r = 0, const float* row_scale = nullptr)
 {
     const int tid = threadIdx.x;
     const int wave = tid >> 6, lane = tid & 63;
@@ -177,6 +178,12 @@ __device__ __forceinline__ void tile_cast_body(const void* x, int64_t row_end, i
             hi[j] = quant4<FP8, SW>(v[4], v[5], v[6], v[7], sc[4], sc[5], sc[6], sc[7]);
             if (!ok) lo[j] = hi[j] = 0;  // padding is zero bytes whatever the scale is (0 * NaN is NaN)
             if (out && ok) *reinterpret_cast<uint2*>(out + r * ld_out + c8) = make_uint2(lo[j], hi[j]);
+            if (out_r && ok) {  // the same values quantised with the row's own scale
+                const float sr = row_scale[r];
+                const uint32_t rl = quant4<FP8, SW>(v[0], v[1], v[2], v[3], sr, sr, sr, sr);
+                const uint32_t rh = quant4<FP8, SW>(v[4], v[5], v[6], v[7], sr, sr, sr, sr);
+                *reinterpret_cast<uint2*>(out_r + r * ld_r + c8) = make_uint2(rl, rh);
+            }
         }
         if (out_t) {
             uint32_t t[8];
@@ -386,6 +393,12 @@ struct GroupedCastArgs {
     uint8_t* out_t;  // [cols, ld_t]
     int64_t ld_t;
     float* scale_out;  // [E, cols]
+    // optional second product of the same two passes: the per-row cast of x (row-major), see
+    // mi8_grouped_cast_rows_and_colwise_t
+    uint32_t* row_amax;  // [T], zero on entry, or null
+    uint8_t* out_r;      // [T, ld_r] or null
+    int64_t ld_r;
+    float* row_scale;    // [T]
 };
 
 // Tile p of the padded row space (128 rows each; group e owns ceil(m_e / 128) consecutive tiles) -> its group,
@@ -430,16 +443,23 @@ __global__ __launch_bounds__(kThreads) void grouped_colamax_kernel(GroupedCastAr
     for (int v = 0; v < NV; ++v)
 #pragma unroll
         for (int k = 0; k < 4; ++k) acc[v][k] = 0;
-    if (c8 < a.cols) {
 #pragma unroll
-        for (int i = 0; i < kTile / 16; ++i) {
-            const int64_t r = row0 + rg + 16 * i;
-            if (r < row_end) {
+    for (int i = 0; i < kTile / 16; ++i) {
+        const int64_t r = row0 + rg + 16 * i;
+        uint32_t rowacc[4] = {0, 0, 0, 0};
+        if (c8 < a.cols && r < row_end) {
 #pragma unroll
-                for (int k = 0; k < NV; ++k)
-                    absmax_accumulate<HP>(
-                        reinterpret_cast<const uint4*>(xb + (r * a.cols + c8) * HpVec<HP>::kBytes)[k], acc[k]);
+            for (int k = 0; k < NV; ++k) {
+                const uint4 v = reinterpret_cast<const uint4*>(xb + (r * a.cols + c8) * HpVec<HP>::kBytes)[k];
+                absmax_accumulate<HP>(v, acc[k]);
+                if (a.row_amax) absmax_accumulate<HP>(v, rowacc);
             }
+        }
+        if (a.row_amax) {  // uniform; the 16 lanes that share this row fold their eight columns each
+            uint32_t m = absmax_fold<HP>(rowacc);
+#pragma unroll
+            for (int off = 8; off > 0; off >>= 1) m = umax32(m, (uint32_t)__shfl_xor((int)m, off, 16));
+            if (cl == 0 && r < row_end && m) atomicMax(&a.row_amax[r], m);
         }
     }
     if constexpr (HP == MI8_BF16) {
@@ -462,6 +482,13 @@ __global__ __launch_bounds__(kThreads) void grouped_colamax_kernel(GroupedCastAr
         for (int k = 0; k < 16; ++k) m = umax32(m, red[k][tid]);
         atomicMax(&a.amax[(int64_t)e * a.cols + col0 + tid], m);  // integer max: order-independent, deterministic
     }
+}
+
+template <int FP8>
+__global__ void row_scales_kernel(const uint32_t* __restrict__ row_amax, int64_t T, bool pow2, float* __restrict__ row_scale)
+{
+    const int64_t r = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (r < T) row_scale[r] = scale_from_amax_bits<FP8>(row_amax[r], pow2);
 }
 
 template <int HP, int FP8, bool SW>
@@ -489,7 +516,8 @@ __global__ __launch_bounds__(kThreads) void grouped_tile_cast_kernel(GroupedCast
 #pragma unroll
     for (int i = 0; i < 8; ++i) sc[i] = s_scale[8 * cl + i];
     const int64_t dst0 = (int64_t)kTile * blockIdx.y;
-    tile_cast_body<HP, FP8, SW>(a.x, row_end, a.cols, row0, col0, sc, nullptr, 0, a.out_t, a.ld_t, dst0, a.ld_t, lds_t);
+    tile_cast_body<HP, FP8, SW>(a.x, row_end, a.cols, row0, col0, sc, nullptr, 0, a.out_t, a.ld_t, dst0, a.ld_t, lds_t,
+                                a.out_r, a.ld_r, a.row_scale);
 }
 
 // ---- dispatch helpers ------------------------------------------------------------------------------
@@ -784,34 +812,46 @@ extern "C" int64_t mi8_grouped_padded_rows(int64_t T, int32_t num_groups)
     return round_up(T, kTile) + (int64_t)kTile * num_groups;
 }
 
-extern "C" int mi8_grouped_cast_colwise_t(const void* x, int hp_dtype, int64_t T, int64_t cols,
-                                          const int64_t* group_sizes, int32_t num_groups, int fp8_dtype,
-                                          uint32_t flags, uint32_t* amax_ws, void* out_t, int64_t ld_t,
-                                          float* scale_out, void* stream)
+namespace mi8 {
+namespace {
+
+int grouped_cast_launch(const char* what, const void* x, int hp_dtype, int64_t T, int64_t cols, const int64_t* group_sizes,
+                        int32_t num_groups, int fp8_dtype, uint32_t flags, uint32_t* amax_ws, void* out_t, int64_t ld_t,
+                        float* scale_out, uint32_t* row_amax_ws, void* out_rows, int64_t ld_rows, float* row_scale_out,
+                        void* stream)
 {
-    MI8_REQUIRE(x && group_sizes && amax_ws && out_t && scale_out, MI8_ERR_ARG, "mi8_grouped_cast_colwise_t: null pointer");
-    MI8_REQUIRE(valid_hp(hp_dtype) && valid_fp8(fp8_dtype), MI8_ERR_ARG, "mi8_grouped_cast_colwise_t: unknown dtype");
-    MI8_REQUIRE(T > 0 && cols > 0 && num_groups > 0, MI8_ERR_ARG, "mi8_grouped_cast_colwise_t: empty input");
-    MI8_REQUIRE(cols % 16 == 0, MI8_ERR_UNSUPPORTED, "mi8_grouped_cast_colwise_t: cols (%lld) must be a multiple of 16",
-                (long long)cols);
+    MI8_REQUIRE(x && group_sizes && amax_ws && out_t && scale_out, MI8_ERR_ARG, "%s: null pointer", what);
+    MI8_REQUIRE(valid_hp(hp_dtype) && valid_fp8(fp8_dtype), MI8_ERR_ARG, "%s: unknown dtype", what);
+    MI8_REQUIRE(T > 0 && cols > 0 && num_groups > 0, MI8_ERR_ARG, "%s: empty input", what);
+    MI8_REQUIRE(cols % 16 == 0, MI8_ERR_UNSUPPORTED, "%s: cols (%lld) must be a multiple of 16", what, (long long)cols);
     MI8_REQUIRE(ld_t % 16 == 0 && ld_t >= mi8_grouped_padded_rows(T, num_groups), MI8_ERR_UNSUPPORTED,
-                "mi8_grouped_cast_colwise_t: ld_t (%lld) must be a multiple of 16 and at least mi8_grouped_padded_rows() = %lld",
+                "%s: ld_t (%lld) must be a multiple of 16 and at least mi8_grouped_padded_rows() = %lld", what,
                 (long long)ld_t, (long long)mi8_grouped_padded_rows(T, num_groups));
-    MI8_REQUIRE(aligned16(x) && aligned16(out_t), MI8_ERR_UNSUPPORTED,
-                "mi8_grouped_cast_colwise_t: pointers must be 16-byte aligned");
+    MI8_REQUIRE(aligned16(x) && aligned16(out_t) && aligned16(out_rows), MI8_ERR_UNSUPPORTED,
+                "%s: pointers must be 16-byte aligned", what);
+    if (out_rows)
+        MI8_REQUIRE(row_amax_ws && row_scale_out && ld_rows >= cols && ld_rows % 16 == 0, MI8_ERR_ARG,
+                    "%s: the row output needs its workspace, its scale output and a pitch >= cols (multiple of 16)", what);
     const int64_t ptiles = ceil_div(T, kTile) + num_groups;
-    MI8_REQUIRE(ptiles <= 65535, MI8_ERR_UNSUPPORTED, "mi8_grouped_cast_colwise_t: too many row tiles (%lld)",
-                (long long)ptiles);
-    GroupedCastArgs a{x, T, cols, group_sizes, num_groups, (flags & MI8_FLAG_POW2_SCALE) != 0,
-                      amax_ws, (uint8_t*)out_t, ld_t, scale_out};
+    MI8_REQUIRE(ptiles <= 65535, MI8_ERR_UNSUPPORTED, "%s: too many row tiles (%lld)", what, (long long)ptiles);
+    const bool pow2 = (flags & MI8_FLAG_POW2_SCALE) != 0;
+    GroupedCastArgs a{x, T, cols, group_sizes, num_groups, pow2, amax_ws, (uint8_t*)out_t, ld_t, scale_out,
+                      out_rows ? row_amax_ws : nullptr, (uint8_t*)out_rows, ld_rows, row_scale_out};
     hipStream_t st = (hipStream_t)stream;
     dim3 grid((unsigned)ceil_div(cols, kTile), (unsigned)ptiles);
     if (hp_dtype == MI8_BF16)
         hipLaunchKernelGGL((grouped_colamax_kernel<MI8_BF16>), grid, dim3(kThreads), 0, st, a);
     else
         hipLaunchKernelGGL((grouped_colamax_kernel<MI8_F32>), grid, dim3(kThreads), 0, st, a);
-    int rc = launch_status("mi8_grouped_cast_colwise_t(amax)");
+    int rc = launch_status(what);
     if (rc != MI8_OK) return rc;
+    if (out_rows) {
+        const dim3 rg((unsigned)ceil_div(T, 256));
+        if (fp8_dtype == MI8_E4M3)
+            hipLaunchKernelGGL((row_scales_kernel<MI8_E4M3>), rg, dim3(256), 0, st, row_amax_ws, T, pow2, row_scale_out);
+        else
+            hipLaunchKernelGGL((row_scales_kernel<MI8_E5M2>), rg, dim3(256), 0, st, row_amax_ws, T, pow2, row_scale_out);
+    }
     const bool sw = flags & MI8_FLAG_SW_CVT;
 #define MI8_GC(HP_, FP8_)                                                                                   \
     if (sw)                                                                                                 \
@@ -824,5 +864,29 @@ extern "C" int mi8_grouped_cast_colwise_t(const void* x, int hp_dtype, int64_t T
         if (fp8_dtype == MI8_E4M3) { MI8_GC(MI8_F32, MI8_E4M3); } else { MI8_GC(MI8_F32, MI8_E5M2); }
     }
 #undef MI8_GC
-    return launch_status("mi8_grouped_cast_colwise_t(cast)");
+    return launch_status(what);
+}
+
+}  // namespace
+}  // namespace mi8
+
+extern "C" int mi8_grouped_cast_colwise_t(const void* x, int hp_dtype, int64_t T, int64_t cols,
+                                          const int64_t* group_sizes, int32_t num_groups, int fp8_dtype,
+                                          uint32_t flags, uint32_t* amax_ws, void* out_t, int64_t ld_t,
+                                          float* scale_out, void* stream)
+{
+    return grouped_cast_launch("mi8_grouped_cast_colwise_t", x, hp_dtype, T, cols, group_sizes, num_groups, fp8_dtype,
+                               flags, amax_ws, out_t, ld_t, scale_out, nullptr, nullptr, 0, nullptr, stream);
+}
+
+extern "C" int mi8_grouped_cast_rows_and_colwise_t(const void* x, int hp_dtype, int64_t T, int64_t cols,
+                                                   const int64_t* group_sizes, int32_t num_groups, int fp8_dtype,
+                                                   uint32_t flags, uint32_t* amax_ws, void* out_t, int64_t ld_t,
+                                                   float* scale_out, uint32_t* row_amax_ws, void* out_rows,
+                                                   int64_t ld_rows, float* row_scale_out, void* stream)
+{
+    MI8_REQUIRE(out_rows, MI8_ERR_ARG, "mi8_grouped_cast_rows_and_colwise_t: out_rows is null");
+    return grouped_cast_launch("mi8_grouped_cast_rows_and_colwise_t", x, hp_dtype, T, cols, group_sizes, num_groups,
+                               fp8_dtype, flags, amax_ws, out_t, ld_t, scale_out, row_amax_ws, out_rows, ld_rows,
+                               row_scale_out, stream);
 }

@@ -331,6 +331,35 @@ def grouped_cast_colwise_t(
     return q_t, scale
 
 
+def grouped_cast_rows_and_colwise_t(
+    x: torch.Tensor, group_sizes: torch.Tensor, fp8_dtype: torch.dtype, *, pow2: bool = False
+) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]:
+    """
+    :func:`cast_rowwise` and :func:`grouped_cast_colwise_t` of the same tensor in one pair of passes:
+    ``(q [T, cols], row_scale [T], q_t [cols, ld_t], col_scale [E, cols])``.  The group sizes must sum to ``T``
+    (rows after the last group are left unwritten).
+    """
+    x = _hp2d(x, "grouped_cast_rows_and_colwise_t")
+    T, cols = x.shape
+    sizes = _sizes_i64(group_sizes, x.device)
+    E = sizes.numel()
+    ld_t = grouped_padded_rows(T, E)
+    q_t = torch.empty((cols, ld_t), dtype=fp8_dtype, device=x.device)
+    scale = torch.empty((E, cols), dtype=torch.float32, device=x.device)
+    q = torch.empty((T, cols), dtype=fp8_dtype, device=x.device)
+    row_scale = torch.empty(T, dtype=torch.float32, device=x.device)
+    ws = torch.zeros(E * cols + T, dtype=torch.int32, device=x.device)
+    _C.check(
+        _C.lib().mi8_grouped_cast_rows_and_colwise_t(
+            x.data_ptr(), _HP_CODE[x.dtype], T, cols, sizes.data_ptr(), E, _FP8_CODE[fp8_dtype], _flags(pow2),
+            ws.data_ptr(), q_t.data_ptr(), ld_t, scale.data_ptr(), ws.data_ptr() + 4 * E * cols, q.data_ptr(), cols,
+            row_scale.data_ptr(), _stream(x),
+        ),
+        "mi8_grouped_cast_rows_and_colwise_t",
+    )
+    return q, row_scale, q_t, scale
+
+
 def grouped_gemm_fp8(
     a: torch.Tensor,
     sa: torch.Tensor,

@@ -34,62 +34,95 @@ class _Float8DroplessMLP(torch.autograd.Function):
         dev = x.device
         equal = torch.full((E,), H, dtype=torch.int64, device=dev)  # the experts' weights as equal-size groups
 
-        xq, sx = ops.cast_rowwise(x, _E4M3, pow2=pow2)
-        w1q, s1 = ops.cast_rowwise(w1, _E4M3, pow2=pow2)  # per output channel (row of w[e])
-        w3q, s3 = ops.cast_rowwise(w3, _E4M3, pow2=pow2)
+        need = ctx.needs_input_grad
+        need_w13 = need[1] or need[3]
+        any_grad = any(need[:4])
+        # operands that are needed in both layouts (by rows for the forward / grad-input GEMMs, by the group's
+        # columns for the weight-gradient GEMMs) come out of one pair of passes
+        xt = sxc = ht = shc = w1t = s1c = w3t = s3c = w2q = s2r = None
+        if need_w13:
+            xq, sx, xt, sxc = ops.grouped_cast_rows_and_colwise_t(x, sizes, _E4M3, pow2=pow2)
+        else:
+            xq, sx = ops.cast_rowwise(x, _E4M3, pow2=pow2)
+        # w1/w3: one scale per output channel (row of w[e]) forward, per input channel of w[e] for grad_input
+        if need[0]:
+            w1q, s1, w1t, s1c = ops.grouped_cast_rows_and_colwise_t(w1, equal, _E4M3, pow2=pow2)
+            w3q, s3, w3t, s3c = ops.grouped_cast_rows_and_colwise_t(w3, equal, _E4M3, pow2=pow2)
+        else:
+            w1q, s1 = ops.cast_rowwise(w1, _E4M3, pow2=pow2)
+            w3q, s3 = ops.cast_rowwise(w3, _E4M3, pow2=pow2)
         x1 = ops.grouped_gemm_fp8(xq, sx, w1q, s1, sizes, n=H, k=D, b_group_stride=H * w1q.stride(0), sb_group_stride=H)
         x2 = ops.grouped_gemm_fp8(xq, sx, w3q, s3, sizes, n=H, k=D, b_group_stride=H * w3q.stride(0), sb_group_stride=H)
         h, _ = ops.swiglu_fwd(x1, x2, want_amax=False)
-        hq, sh = ops.cast_rowwise(h, _E4M3, pow2=pow2)
+        if need[2]:
+            hq, sh, ht, shc = ops.grouped_cast_rows_and_colwise_t(h, sizes, _E4M3, pow2=pow2)
+        else:
+            hq, sh = ops.cast_rowwise(h, _E4M3, pow2=pow2)
+        del h
         # w2[e] is [H, D] and is used as-is (h_e @ w2[e]): its output channel is the column -> transposed copy
-        # [D, E*H] with one scale per (expert, column)
-        w2t, s2 = ops.grouped_cast_colwise_t(w2, equal, _E4M3, pow2=pow2)
+        # [D, E*H] with one scale per (expert, column); the by-rows copy is the grad_h GEMM's right operand
+        if any_grad:
+            w2q, s2r, w2t, s2 = ops.grouped_cast_rows_and_colwise_t(w2, equal, _E4M3, pow2=pow2)
+        else:
+            w2t, s2 = ops.grouped_cast_colwise_t(w2, equal, _E4M3, pow2=pow2)
         y = ops.grouped_gemm_fp8(hq, sh, w2t, s2, sizes, n=D, k=H, b_group_stride=H, sb_group_stride=D)
-        ctx.save_for_backward(x, w1, w2, w3, x1, x2, h, sizes, equal)
-        ctx.meta = (E, T, D, H, pow2)
+        none = x.new_empty(0)
+        opt = lambda t: none if t is None else t  # noqa: E731
+        ctx.save_for_backward(opt(xt), opt(sxc), x1, x2, opt(ht), opt(shc), opt(w1t), opt(s1c), opt(w3t), opt(s3c),
+                              opt(w2q), opt(s2r), sizes)
+        ctx.meta = (E, T, D, H, pow2, (x.dtype, w1.dtype, w2.dtype, w3.dtype))
         return y
 
     @staticmethod
     def backward(ctx, gy):
-        x, w1, w2, w3, x1, x2, h, sizes, equal = ctx.saved_tensors
-        E, T, D, H, pow2 = ctx.meta
+        xt, sxc, x1, x2, ht, shc, w1t, s1c, w3t, s3c, w2q, s2r, sizes = ctx.saved_tensors
+        E, T, D, H, pow2, (x_dt, w1_dt, w2_dt, w3_dt) = ctx.meta
         gy = gy.reshape(T, D).contiguous()
+        if gy.dtype != x_dt:
+            gy = gy.to(x_dt)
         need_x, need_w1, need_w2, need_w3 = ctx.needs_input_grad[:4]
 
-        gyq, sgy = ops.cast_rowwise(gy, _E4M3, pow2=pow2)
-        # gh_e = gy_e @ w2[e]^T : contraction over D, the right operand is w2[e] itself with one scale per row
-        w2q, s2r = ops.cast_rowwise(w2, _E4M3, pow2=pow2)
-        gh = ops.grouped_gemm_fp8(gyq, sgy, w2q, s2r, sizes, n=H, k=D, b_group_stride=H * w2q.stride(0), sb_group_stride=H)
         gw2 = None
         if need_w2:
+            gyq, sgy, gyt, sgyc = ops.grouped_cast_rows_and_colwise_t(gy, sizes, _E4M3, pow2=pow2)
             # gw2[e] [H, D] = h_e^T @ gy_e : contraction over the group's tokens
-            ht, shc = ops.grouped_cast_colwise_t(h, sizes, _E4M3, pow2=pow2)
-            gyt, sgyc = ops.grouped_cast_colwise_t(gy, sizes, _E4M3, pow2=pow2)
-            gw2 = ops.grouped_wgrad_fp8(ht, shc, gyt, sgyc, sizes, tokens=T, out_dtype=gy.dtype).reshape(E * H, D)
-        g1, g2, _, _ = ops.swiglu_bwd(x1, x2, gh, want_amax=False)
-        del gh
+            gw2 = ops.grouped_wgrad_fp8(ht, shc, gyt, sgyc, sizes, tokens=T, out_dtype=x_dt).reshape(E * H, D)
+            del gyt
+        else:
+            gyq, sgy = ops.cast_rowwise(gy, _E4M3, pow2=pow2)
         gx = gw1 = gw3 = None
-        if need_x:
-            # gx_e = g_e @ w[e] : contraction over H, the right operand is w[e]^T [D, H] with one scale per input channel
-            g1q, sg1 = ops.cast_rowwise(g1, _E4M3, pow2=pow2)
-            g2q, sg2 = ops.cast_rowwise(g2, _E4M3, pow2=pow2)
-            w1t, s1c = ops.grouped_cast_colwise_t(w1, equal, _E4M3, pow2=pow2)
-            w3t, s3c = ops.grouped_cast_colwise_t(w3, equal, _E4M3, pow2=pow2)
-            gx = ops.grouped_gemm_fp8(g1q, sg1, w1t, s1c, sizes, n=D, k=H, b_group_stride=H, sb_group_stride=D)
-            gx = gx + ops.grouped_gemm_fp8(g2q, sg2, w3t, s3c, sizes, n=D, k=H, b_group_stride=H, sb_group_stride=D)
-        if need_w1 or need_w3:
-            xt, sxc = ops.grouped_cast_colwise_t(x, sizes, _E4M3, pow2=pow2)
+        if need_x or need_w1 or need_w3:
+            # gh_e = gy_e @ w2[e]^T : contraction over D, the right operand is w2[e] itself, one scale per row
+            gh = ops.grouped_gemm_fp8(gyq, sgy, w2q, s2r, sizes, n=H, k=D, b_group_stride=H * w2q.stride(0),
+                                      sb_group_stride=H)
+            g1, g2, _, _ = ops.swiglu_bwd(x1, x2, gh, want_amax=False)
+            del gh
+
+            def both(g, want_rows, want_cols):
+                if want_rows and want_cols:
+                    return ops.grouped_cast_rows_and_colwise_t(g, sizes, _E4M3, pow2=pow2)
+                if want_rows:
+                    return (*ops.cast_rowwise(g, _E4M3, pow2=pow2), None, None)
+                if want_cols:
+                    return (None, None, *ops.grouped_cast_colwise_t(g, sizes, _E4M3, pow2=pow2))
+                return None, None, None, None
+
+            g1q, sg1, g1t, sg1c = both(g1, need_x, need_w1)
+            g2q, sg2, g2t, sg2c = both(g2, need_x, need_w3)
+            del g1, g2
+            if need_x:
+                # gx_e = g_e @ w[e] : contraction over H, the right operand is w[e]^T [D, H], one scale per input channel
+                gx = ops.grouped_gemm_fp8(g1q, sg1, w1t, s1c, sizes, n=D, k=H, b_group_stride=H, sb_group_stride=D)
+                gx = gx + ops.grouped_gemm_fp8(g2q, sg2, w3t, s3c, sizes, n=D, k=H, b_group_stride=H, sb_group_stride=D)
             if need_w1:
-                g1t, sg1c = ops.grouped_cast_colwise_t(g1, sizes, _E4M3, pow2=pow2)
-                gw1 = ops.grouped_wgrad_fp8(g1t, sg1c, xt, sxc, sizes, tokens=T, out_dtype=gy.dtype).reshape(E * H, D)
+                gw1 = ops.grouped_wgrad_fp8(g1t, sg1c, xt, sxc, sizes, tokens=T, out_dtype=x_dt).reshape(E * H, D)
             if need_w3:
-                g2t, sg2c = ops.grouped_cast_colwise_t(g2, sizes, _E4M3, pow2=pow2)
-                gw3 = ops.grouped_wgrad_fp8(g2t, sg2c, xt, sxc, sizes, tokens=T, out_dtype=gy.dtype).reshape(E * H, D)
+                gw3 = ops.grouped_wgrad_fp8(g2t, sg2c, xt, sxc, sizes, tokens=T, out_dtype=x_dt).reshape(E * H, D)
 
-        def as_param(g, ref):
-            return g if g is None or g.dtype == ref.dtype else g.to(ref.dtype)
+        def as_param(g, dt):
+            return g if g is None or g.dtype == dt else g.to(dt)
 
-        return gx, as_param(gw1, w1), as_param(gw2, w2), as_param(gw3, w3), None, None, None
+        return gx, as_param(gw1, w1_dt), as_param(gw2, w2_dt), as_param(gw3, w3_dt), None, None, None
 
 
 @torch.compiler.disable

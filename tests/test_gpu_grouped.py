@@ -49,6 +49,33 @@ def test_grouped_colwise_cast_bit_exact(dev, sizes):
         start += m
 
 
+@pytest.mark.parametrize("pow2", [True, False], ids=["pow2", "exact"])
+@pytest.mark.parametrize("sizes", SIZE_CASES, ids=lambda s: "-".join(map(str, s)))
+def test_rows_and_grouped_colwise_cast_bit_exact(dev, sizes, pow2):
+    """The two-product cast gives the oracle's per-row cast of the whole tensor and its per-expert per-column cast,
+    and is byte-identical to the two single-product entry points."""
+    T, C = sum(sizes), 272
+    x = seeded((T, C), 11, std=0.3)
+    x[:, 1] = 0
+    x[T // 2] = 0
+    xd = x.to(dev)
+    q, rs, q_t, cs = ops.grouped_cast_rows_and_colwise_t(xd, torch.tensor(sizes), E4M3, pow2=pow2)
+    ref_q, ref_s = O.cast(x, E4M3, O.AXISWISE, -1, pow2)
+    assert_scale_equal(rs, ref_s.reshape(-1), "row scales")
+    assert_bytes_equal(q, ref_q, what="row-major bytes")
+    q_t1, cs1 = ops.grouped_cast_colwise_t(xd, torch.tensor(sizes), E4M3, pow2=pow2)
+    start = 0
+    for e, (m, p0) in enumerate(zip(sizes, _padded_starts(sizes))):
+        if m == 0:
+            continue
+        ref_qc, ref_sc = O.cast(x[start:start + m], E4M3, O.AXISWISE, 0, pow2)
+        assert_scale_equal(cs[e], ref_sc, f"group {e} column scales")
+        assert_bytes_equal(q_t[:, p0:p0 + m], ref_qc.t(), what=f"group {e} transposed bytes")
+        assert torch.equal(u8(q_t[:, p0:p0 + 128 * ((m + 127) // 128)]), u8(q_t1[:, p0:p0 + 128 * ((m + 127) // 128)]))
+        assert torch.equal(cs[e], cs1[e])
+        start += m
+
+
 @pytest.mark.parametrize("sizes", SIZE_CASES, ids=lambda s: "-".join(map(str, s)))
 def test_grouped_gemm_exact_integers(dev, sizes):
     """Integer operands: the grouped forward GEMM must reproduce the per-expert integer matmul exactly, for both
