@@ -26,8 +26,8 @@ D_MODEL, HIDDEN, TOKENS = 4096, 11008, 16384
 FP8_MFMA_PEAK_TFLOPS = 5000.0  # MI355X dense fp8 matrix peak
 GEMMS_PER_STEP = 9
 # HBM-side bytes per GEMM launch (L2 fill reads + writes), mean over the 9 launches of a step, from the
-# FETCH_SIZE / WRITE_SIZE counter runs summarised in profiles/gemm_fp8_dma8_kernel__mlp7b_traffic_pmc.txt
-GEMM_TRAFFIC_BYTES_PER_LAUNCH = 1.424e9
+# FETCH_SIZE / WRITE_SIZE counter runs summarised in profiles/gemm_fp8_m16_kernel__mlp7b_traffic_pmc.txt
+GEMM_TRAFFIC_BYTES_PER_LAUNCH = 1.400e9
 
 
 def build_mlp(dev):
@@ -306,7 +306,7 @@ def main():
         },
         "pct_fp8_mfma_peak": round(100.0 * tflops / FP8_MFMA_PEAK_TFLOPS, 2),
         "roofline": {
-            "kernel": "gemm_fp8_dma8_kernel (9 launches per step, 2*16384*4096*11008 flop each)",
+            "kernel": "gemm_fp8_m16_kernel (9 launches per step, 2*16384*4096*11008 flop each)",
             "bound": "mfma",
             "achieved": round(achieved, 2),
             "peak": FP8_MFMA_PEAK_TFLOPS,

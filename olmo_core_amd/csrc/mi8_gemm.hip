@@ -38,8 +38,9 @@ constexpr Variant kVariants[] = {
     {"256x256_dma_w4_k64x4", 256, 256, 256},
     {"256x256_dma_w8_k128x2", 256, 256, 512},
     {"256x256_dma_w4x128_k128x2", 256, 256, 256},
+    {"256x256_dma_w4x128_m16x128", 256, 256, 256},
 };
-constexpr int kDma = 5, kDma8 = 6, kDma4 = 7;
+constexpr int kDma = 5, kDma8 = 6, kDma4 = 7, kM16 = 8;
 constexpr int kNumVariants = sizeof(kVariants) / sizeof(kVariants[0]);
 
 template <int BM, int BN, int WM, int WN, int CBSZ, int BLGP>
@@ -118,12 +119,13 @@ extern "C" int mi8_gemm_fp8(const void* a, int a_dtype, int64_t lda, const void*
     const bool dma_ok = (K % 64 == 0) && M >= 256 && N >= 256 && N % 8 == 0 && ldc % 8 == 0 && aligned16(out) &&
                         out_dtype == MI8_BF16 && (!sb_is_vector || aligned16(sb)) &&
                         (sa_is_vector != 0) == (sb_is_vector != 0);
-    // measured on MI355X: the four-wave layout is the faster of the two persistent kernels on every shape of the
-    // benchmark configurations (by 0-14 %)
-    if (variant < 0) variant = dma_ok ? (K % 128 == 0 ? kDma4 : kDma) : 1;
+    // measured on MI355X on the benchmark configurations' shapes: the four-wave layout beats the eight-wave one
+    // by 0-14 %, and its 16x16x128 form beats its 32x32x64 form by 1-6 % (random operands, power-limited clocks)
+    if (variant < 0) variant = dma_ok ? (K % 128 == 0 ? kM16 : kDma) : 1;
     if (variant == kDma8 && dma_ok && K % 128 == 0) return launch_dma8(g, a_dtype, b_dtype, st);
     if (variant == kDma4 && dma_ok && K % 128 == 0) return launch_dma4(g, a_dtype, b_dtype, st);
-    if (variant == kDma || variant == kDma8 || variant == kDma4) {
+    if (variant == kM16 && dma_ok && K % 128 == 0) return launch_m16(g, a_dtype, b_dtype, st);
+    if (variant == kDma || variant == kDma8 || variant == kDma4 || variant == kM16) {
         MI8_REQUIRE(dma_ok && variant == kDma, MI8_ERR_UNSUPPORTED,
                     "mi8_gemm_fp8: the direct-to-LDS variant needs M, N >= 256, K %% 64 == 0 (8 waves: 128), N %% 8 == 0, ldc %% 8 == 0, "
                     "scales that are both single values or both vectors, and a 16-byte aligned bf16 output (M=%lld N=%lld K=%lld ldc=%lld)",

@@ -17,13 +17,12 @@
 //
 // Swizzle: chunk position q (16 bytes) of row r holds global chunk q ^ ((r ^ r>>3) & 7).  A load instruction
 // fills 8 consecutive rows (lane l -> row l/8, position l%8), so lane l fetches chunk (l%8) ^ swz(row).
-#include "mi8_gemm.h"
+#include "mi8_gemm_tiles.h"
 
 namespace mi8 {
 namespace gemm {
 namespace {
 
-constexpr int BM = 256, BN = 256;
 constexpr int WTM = 128, TM = 4;               // two waves along M, each 4 MFMA tiles of 32 rows
 constexpr int STAGE = (BM + BN) * BK;          // 64 KB
 constexpr int OUT_STAGING = 8 * 4096;           // 4 KB of output staging per wave
@@ -58,249 +57,6 @@ __device__ __forceinline__ constexpr int frag_a(int i) { return i == 0 ? 0 : 2 *
 __device__ __forceinline__ constexpr int frag_b(int j) { return 2 + 2 * j; }
 
 
-// ---- what a workgroup needs to know about one output tile ---------------------------------------------
-struct TileDesc {
-    const uint8_t* a;  // first A row of the tile (K offset 0 of the tile's contraction range)
-    const uint8_t* b;  // first B row of the tile
-    int nk;            // 128-byte K steps (0: the tile is all zeros)
-    const float* sa;   // scale of the tile's first row (or the single scale)
-    const float* sb;   // scale of the tile's first column (or the single scale)
-    uint16_t* c;       // C element (first row, first column) of the tile
-    int row_lo, row_hi;  // rows [row_lo, row_hi) of the 256 are stored
-};
-
-struct NoCache {};
-
-// Dense problem: C[M, N] = A[M, K] . B[N, K]^T.  The last tile row / column is shifted back so that every tile
-// is full (M, N >= 256): the overlap is recomputed with the same K order and rewritten with identical values.
-template <bool VEC>
-struct DenseProblem {
-    GemmArgs g;
-    int64_t lda, ldb, ldc;
-    static constexpr bool kVecScales = VEC;  // both scales are vectors (per row / per column) or both single
-    static constexpr bool kMaskRows = false, kXcdRanges = true, kPeelFirstStep = true;
-    using Cache = NoCache;
-    __device__ __forceinline__ Cache prepare() const { return Cache{}; }
-    __device__ __forceinline__ int total_tiles(const Cache&) const { return g.tiles_m * g.tiles_n; }
-    __device__ __forceinline__ TileDesc tile(int t, const Cache&) const
-    {
-        int tm, tn;
-        tile_coords(g, t, tm, tn);
-        const int m0 = (tm * BM + BM <= g.M) ? tm * BM : g.M - BM;
-        const int n0 = (tn * BN + BN <= g.N) ? tn * BN : g.N - BN;
-        TileDesc d;
-        d.a = g.A + (int64_t)m0 * g.lda;
-        d.b = g.B + (int64_t)n0 * g.ldb;
-        d.nk = g.K / BK;
-        d.sa = g.sa + (VEC ? m0 : 0);
-        d.sb = g.sb + (VEC ? n0 : 0);
-        d.c = reinterpret_cast<uint16_t*>(g.C) + (int64_t)m0 * g.ldc + n0;
-        d.row_lo = 0;
-        d.row_hi = BM;
-        return d;
-    }
-};
-
-// ---- locating a group in the device-resident size list ---------------------------------------------------
-// Groups are consecutive row ranges; sizes are clamped so that their running sum never passes T.  A group of
-// m rows owns ceil(m / U) "units" (row tiles).  The 64 lanes of a wave each take one group of a 64-group chunk
-// and prefix-sum rows and units with shuffles, so a lookup costs one load latency instead of E dependent
-// ones.  Must be called by all lanes of the wave together; the result is wave-uniform.
-struct GroupSpan {
-    int e;                 // group index (E if the key is past the end)
-    int64_t rows_before;   // rows of the groups before it
-    int64_t m;             // its clamped size
-    int64_t units_before;  // units of the groups before it (all units if the key is past the end)
-};
-
-__device__ __forceinline__ int64_t uniform64(int64_t v)
-{
-    const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v);
-    const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)((uint64_t)v >> 32));
-    return (int64_t)(((uint64_t)hi << 32) | lo);
-}
-
-__device__ __forceinline__ int64_t wave_inclusive_sum(int64_t v, int lane)
-{
-#pragma unroll
-    for (int d = 1; d < 64; d <<= 1) {
-        const int64_t o = __shfl_up(v, d, 64);
-        if (lane >= d) v += o;
-    }
-    return v;
-}
-
-// BY_UNIT: key is a unit index, find the group that owns it; otherwise key is the group index itself.
-template <int U, bool BY_UNIT>
-__device__ __forceinline__ GroupSpan locate_group(const int64_t* sizes, int E, int64_t T, int64_t key)
-{
-    const int lane = (int)threadIdx.x & 63;
-    int64_t rows_c = 0, units_c = 0;
-    for (int base = 0; base < E; base += 64) {
-        const int e = base + lane;
-        int64_t m = (e < E) ? sizes[e] : 0;
-        m = m < 0 ? 0 : (m > T ? T : m);
-        int64_t end = rows_c + wave_inclusive_sum(m, lane);
-        int64_t start = end - m;
-        end = end < T ? end : T;
-        start = start < T ? start : T;
-        const int64_t me = end - start;
-        const int64_t un = (me + U - 1) / U;
-        const int64_t uend = units_c + wave_inclusive_sum(un, lane);
-        const bool hit = (e < E) && (BY_UNIT ? key < uend : key == e);
-        const uint64_t mask = __ballot(hit);
-        if (mask) {
-            const int src = __ffsll((unsigned long long)mask) - 1;
-            GroupSpan r;
-            r.e = base + src;
-            r.rows_before = uniform64(__shfl(start, src, 64));
-            r.m = uniform64(__shfl(me, src, 64));
-            r.units_before = uniform64(__shfl(uend - un, src, 64));
-            return r;
-        }
-        rows_c = uniform64(__shfl(end, 63, 64));
-        units_c = uniform64(__shfl(uend, 63, 64));
-    }
-    return GroupSpan{E, rows_c, 0, units_c};
-}
-
-// Up to 64 groups: the prefix sums live in four registers of every wave for the whole kernel (lane e holds
-// group e), and a lookup is a ballot and three lane reads, with no memory access inside the K loop.
-struct GroupCache {
-    int start, m, ubefore, uend;  // per lane: first row, clamped size, units before, units up to and including
-    bool valid;                   // wave-uniform: E <= 64 (otherwise lookups go to memory)
-};
-
-template <int U>
-__device__ __forceinline__ GroupCache build_group_cache(const int64_t* sizes, int E, int64_t T)
-{
-    GroupCache c{0, 0, 0, 0, E <= 64};
-    if (!c.valid) return c;
-    const int lane = (int)threadIdx.x & 63;
-    int64_t m = (lane < E) ? sizes[lane] : 0;
-    m = m < 0 ? 0 : (m > T ? T : m);
-    int64_t end = wave_inclusive_sum(m, lane);
-    int64_t start = end - m;
-    end = end < T ? end : T;
-    start = start < T ? start : T;
-    const int64_t me = end - start;
-    const int64_t un = (me + U - 1) / U;
-    const int64_t uend = wave_inclusive_sum(un, lane);
-    c.start = (int)start;  // T < 2^30 is checked on the host
-    c.m = (int)me;
-    c.ubefore = (int)(uend - un);
-    c.uend = (int)uend;
-    return c;
-}
-
-template <int U, bool BY_UNIT>
-__device__ __forceinline__ GroupSpan locate_group_cached(const GroupCache& c, const int64_t* sizes, int E, int64_t T,
-                                                         int64_t key)
-{
-    if (!c.valid) return locate_group<U, BY_UNIT>(sizes, E, T, key);
-    int src;
-    if constexpr (BY_UNIT) {
-        const uint64_t mask = __ballot((int64_t)c.uend > key);
-        if (mask == 0) return GroupSpan{E, T, 0, __builtin_amdgcn_readlane(c.uend, 63)};
-        src = __ffsll((unsigned long long)mask) - 1;
-    } else {
-        src = (int)key;
-    }
-    GroupSpan r;
-    r.e = src;
-    r.rows_before = __builtin_amdgcn_readlane(c.start, src);
-    r.m = __builtin_amdgcn_readlane(c.m, src);
-    r.units_before = __builtin_amdgcn_readlane(c.ubefore, src);
-    return r;
-}
-
-// Ragged-M grouped problem (dropless-MoE forward / grad_input): rows of A form consecutive groups, group e
-// multiplies B_e = B + e * b_group_stride.  A tile covers up to 256 rows of ONE group; it always loads a full
-// 256-row window (shifted back at the end of the matrix, T >= 256) and stores only its group's rows.
-struct GroupedProblem {
-    const uint8_t* A;
-    const uint8_t* B;
-    uint16_t* C;
-    int64_t lda, ldb, ldc, b_group_stride, sb_group_stride;
-    const int64_t* sizes;
-    int E;
-    int64_t T;
-    int N, K, tiles_n;
-    const float* sa;
-    const float* sb;
-    static constexpr bool kVecScales = true, kMaskRows = true, kXcdRanges = true, kPeelFirstStep = false;
-    using Cache = GroupCache;
-    __device__ __forceinline__ Cache prepare() const { return build_group_cache<BM>(sizes, E, T); }
-    __device__ __forceinline__ int total_tiles(const Cache& c) const
-    {
-        const GroupSpan s = locate_group_cached<BM, true>(c, sizes, E, T, (int64_t)1 << 60);
-        return (int)s.units_before * tiles_n;
-    }
-    __device__ __forceinline__ TileDesc tile(int t, const Cache& c) const
-    {
-        const int mt = t / tiles_n, nt = t % tiles_n;
-        const GroupSpan s = locate_group_cached<BM, true>(c, sizes, E, T, mt);
-        const int64_t want0 = s.rows_before + (mt - s.units_before) * BM;  // first row this tile is responsible for
-        int64_t want1 = want0 + BM;
-        const int64_t group_end = s.rows_before + s.m;
-        want1 = want1 < group_end ? want1 : group_end;                     // ... up to the group's end
-        const int64_t m0 = (want0 + BM <= T) ? want0 : T - BM;             // loaded window
-        const int n0 = (nt * BN + BN <= N) ? nt * BN : N - BN;
-        TileDesc d;
-        d.a = A + m0 * lda;
-        d.b = B + (int64_t)s.e * b_group_stride + (int64_t)n0 * ldb;
-        d.nk = K / BK;
-        d.sa = sa + m0;
-        d.sb = sb + (int64_t)s.e * sb_group_stride + n0;
-        d.c = C + m0 * ldc + n0;
-        d.row_lo = (int)(want0 - m0);
-        d.row_hi = (int)(want1 - m0);
-        return d;
-    }
-};
-
-// Ragged-K grouped problem (dropless-MoE grad_weight): out[e] = A_t[:, S_e] . B_t[:, S_e]^T over group e's
-// 128-aligned segment S_e of the padded token axis; N, Kl >= 256.  An empty group gives nk = 0: its tiles are
-// written as zeros and its scales (never produced) are ignored.
-struct GroupedWgradProblem {
-    const uint8_t* At;
-    const uint8_t* Bt;
-    uint16_t* C;
-    int64_t lda, ldb, ldc;  // lda = ldb = padded token pitch, ldc = Kl
-    const int64_t* sizes;
-    int E;
-    int64_t T;
-    int N, Kl, tiles_n, tiles_k;
-    const float* sa;  // [E, N]
-    const float* sb;  // [E, Kl]
-    static constexpr bool kVecScales = true, kMaskRows = false, kXcdRanges = false, kPeelFirstStep = true;
-    using Cache = GroupCache;
-    __device__ __forceinline__ Cache prepare() const { return build_group_cache<128>(sizes, E, T); }
-    __device__ __forceinline__ int total_tiles(const Cache&) const { return E * tiles_n * tiles_k; }
-    __device__ __forceinline__ TileDesc tile(int t, const Cache& c) const
-    {
-        const int per_group = tiles_n * tiles_k;
-        const int e = t / per_group, rem = t % per_group;
-        const int tn = rem / tiles_k, tk = rem % tiles_k;
-        const GroupSpan s = locate_group_cached<128, false>(c, sizes, E, T, e);
-        const int64_t seg0 = 128 * s.units_before;
-        int64_t seg = 128 * ((s.m + 127) / 128);
-        if (seg0 + seg > lda) seg = 0;
-        const int n0 = (tn * BM + BM <= N) ? tn * BM : N - BM;
-        const int k0 = (tk * BN + BN <= Kl) ? tk * BN : Kl - BN;
-        TileDesc d;
-        d.a = At + (int64_t)n0 * lda + seg0;
-        d.b = Bt + (int64_t)k0 * ldb + seg0;
-        d.nk = (int)(seg / BK);
-        d.sa = sa + (int64_t)e * N + n0;
-        d.sb = sb + (int64_t)e * Kl + k0;
-        d.c = C + ((int64_t)e * N + n0) * ldc + k0;
-        d.row_lo = 0;
-        d.row_hi = BM;
-        return d;
-    }
-};
-
 template <typename Problem, int WN, int CBSZ_A, int BLGP_B>
 __global__ __launch_bounds__(Layout<WN>::kThreads, 1) void gemm_fp8_dma8_kernel(Problem pb)
 {
@@ -325,12 +81,40 @@ __global__ __launch_bounds__(Layout<WN>::kThreads, 1) void gemm_fp8_dma8_kernel(
     const uint32_t xa00 = (uint32_t)((wm * WTM + l32) * BK + (((2 * half) ^ swz(wm * WTM + l32)) << 4));
     const uint32_t xb00 = (uint32_t)(BM * BK + (wn * WTN + l32) * BK + (((2 * half) ^ swz(wn * WTN + l32)) << 4));
     // slot x of Frags: 0,1 = A0; then two per B tile; then A1..A3.  pa / pb: xa00 / xb00 plus the stage's byte offset.
+    // The four-wave layout has registers to spare (its accumulators live in the other half of the register file)
+    // and one wave per SIMD, so every address instruction between two MFMAs is exposed: it keeps the four XOR
+    // variants per operand resident as LDS addresses of the stage being read (kResident) and moves them to the
+    // other stage with one add each per K step.
+    constexpr bool kResident = (WN == 2);
+    uint32_t ra[4], rb[4];
+    if constexpr (kResident) {
+        const uint32_t lds0 = (uint32_t)(uintptr_t)(lptr_t)lds;
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+            ra[v] = lds0 + (xa00 ^ (uint32_t)(((4 * (v >> 1)) | (v & 1)) << 4));
+            rb[v] = lds0 + (xb00 ^ (uint32_t)(((4 * (v >> 1)) | (v & 1)) << 4));
+        }
+    }
+    auto flip_read_stage = [&](int to_stage) __attribute__((always_inline)) {
+        const uint32_t delta = to_stage ? (uint32_t)STAGE : (uint32_t)(-STAGE);
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+            ra[v] += delta;
+            rb[v] += delta;
+        }
+    };
     auto read_one = [&](Frags& f, uint32_t pa, uint32_t pb_, int s, int x) __attribute__((always_inline)) {
         const bool is_a = (x < 2) || (x >= 2 + 2 * TN);
         const int tile = x < 2 ? 0 : (x < 2 + 2 * TN ? (x - 2) >> 1 : (x - 2 * TN) >> 1);
         const int q = x & 1;
-        const uint32_t off = ((is_a ? pa : pb_) ^ (uint32_t)(((4 * (s ^ (tile & 1))) | q) << 4)) + tile * 32 * BK;
-        f.h[x] = *reinterpret_cast<const v4i*>(lds + off);
+        if constexpr (kResident) {
+            const int v = 2 * (s ^ (tile & 1)) + q;
+            const uint32_t addr = (is_a ? ra[v] : rb[v]) + tile * 32 * BK;
+            f.h[x] = *reinterpret_cast<const __attribute__((address_space(3))) v4i*>((uintptr_t)addr);
+        } else {
+            const uint32_t off = ((is_a ? pa : pb_) ^ (uint32_t)(((4 * (s ^ (tile & 1))) | q) << 4)) + tile * 32 * BK;
+            f.h[x] = *reinterpret_cast<const v4i*>(lds + off);
+        }
     };
 
     // ---- direct loads: wave w fills rows [R w + 8 p, +8) of each operand, R = kRowsPerWave, p = 0..kLoads-1;
@@ -341,9 +125,28 @@ __global__ __launch_bounds__(Layout<WN>::kThreads, 1) void gemm_fp8_dma8_kernel(
     const uint32_t rowoff_a = (uint32_t)((int64_t)(wave * RPW + lr) * pb.lda);
     const uint32_t rowoff_b = (uint32_t)((int64_t)(wave * RPW + lr) * pb.ldb);
     // x in 0..2 NLD-1: the first NLD -> A rows 8 x, the rest -> B rows 8 (x - NLD)
+    // resident lane offsets of the 2 NLD loads (kResident): row offset and swizzled chunk in one register each, so a
+    // load is one M0 update and the load itself
+    uint32_t dvo[kResident ? 2 * NLD : 1];
+    if constexpr (kResident) {
+#pragma unroll
+        for (int x = 0; x < 2 * NLD; ++x) {
+            const int p = x % NLD;
+            const int64_t ld = x < NLD ? pb.lda : pb.ldb;
+            dvo[x] = (uint32_t)((int64_t)(wave * RPW + 8 * p + lr) * ld) + ((c0 ^ (uint32_t)((NLD * wave + p) & 7)) << 4);
+        }
+    }
     auto dma_one = [&](const uint8_t* a_origin, const uint8_t* b_origin, int stage, int x) __attribute__((always_inline)) {
         const int p = x % NLD;
         const bool is_a = x < NLD;
+        if constexpr (kResident) {
+            uint32_t o = dvo[x];
+            asm volatile("" : "+v"(o));  // keeps the offset 32 bits wide up to the load (uniform base + lane offset form)
+            const uint8_t* src = (is_a ? a_origin : b_origin) + o;
+            uint8_t* dst = lds + stage * STAGE + (is_a ? 0 : BM * BK) + (wave * RPW + 8 * p) * BK;
+            __builtin_amdgcn_global_load_lds((gptr_t)src, (lptr_t)dst, 16, 0, 0);
+            return;
+        }
         // uniform 64-bit base + 32-bit lane offset.  The empty asm makes the lane's chunk index opaque at every
         // use: the offset is then rebuilt with two cheap vector instructions next to the load (and folded into
         // its scalar-base addressing) instead of living in eight hoisted 64-bit lane addresses.
@@ -487,6 +290,7 @@ __global__ __launch_bounds__(Layout<WN>::kThreads, 1) void gemm_fp8_dma8_kernel(
             // outstanding ones (the next step's stage) before telling the others they have landed
             __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
             __syncthreads();
+            if constexpr (kResident) flip_read_stage(cur ^ 1);
             // phase B
 #pragma unroll
             for (int x = 0; x < L::kMmas; ++x) {

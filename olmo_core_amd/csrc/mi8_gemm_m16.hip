@@ -1,0 +1,458 @@
+// Persistent fp8 GEMM on 16x16x128 MFMAs: four waves of 128 x 128 per 256 x 256 workgroup tile, direct
+// global->LDS loads of full 128-byte rows.  Same problems, tile order and LDS budget as the 32x32x64 kernel
+// (mi8_gemm_dma8.hip); for full 256 x 256 tiles, K % 128 == 0, bf16 output.
+//
+// Why this MFMA shape: an MI355X running fp8 MFMAs on random operands is power limited (it clocks down to about
+// 1.7 GHz), so throughput follows energy per flop, and v_mfma_f32_16x16x128_f8f6f4 needs less of it than
+// v_mfma_f32_32x32x64_f8f6f4: back-to-back MFMAs on random bytes, nothing else running, measured 4.35 PFLOP/s
+// against 4.0 PFLOP/s (both 4.97 PFLOP/s on all-zero operands, where the clock stays up).
+//
+// A 128-byte K step of a wave is 8 x 8 MFMAs (A tile i: 16 rows, B tile j: 16 columns, 4 accumulator registers
+// each: 256 in all).  The step is split along M so that only half of the A fragments are double buffered:
+//
+//     phase A   32 x { MFMA (A tiles 0-3) x (B tiles 0-7) }; LDS reads of A tiles 4-7 of this step
+//     wait for this wave's loads of step s+1, barrier
+//     phase B   32 x { MFMA (A tiles 4-7) x (B tiles 0-7), B tile by B tile }; LDS reads of step s+1: A tiles 0-3
+//               and each B tile as soon as its four MFMAs are issued; 16 direct loads of step s+2 into the
+//               stage step s has vacated
+//
+// Fragment registers: 32 (A 0-3) + 32 (A 4-7) + 64 (B) = 128.
+//
+// LDS: two 64 KB operand stages [row][128 B]; 16-byte chunk position c of row r holds global chunk
+// c ^ ((r >> 1) & 7): the 16 rows one quarter-wave reads (same logical chunk) then cover all banks, and the
+// swizzle of a fragment row does not depend on the tile it belongs to, so two address registers per operand
+// serve all eight tiles through the instruction's offset field.
+#include "mi8_gemm_tiles.h"
+
+namespace mi8 {
+namespace gemm {
+namespace {
+
+typedef float v4f __attribute__((ext_vector_type(4)));
+typedef __attribute__((address_space(1))) const void* gptr_t;
+typedef __attribute__((address_space(3))) void* lptr_t;
+typedef const __attribute__((address_space(3))) v4i* lfrag_t;
+
+constexpr int STAGE = (BM + BN) * BK;        // 64 KB
+constexpr int OUT_STAGING = 4 * 4096;        // 4 KB of output staging per wave
+constexpr int SCALE_SLOT = 2 * 256 * 4;      // one tile's 256 row scales and 256 column scales
+constexpr int SCALE_SLOTS = 4;
+constexpr int LDS_BYTES = 2 * STAGE + OUT_STAGING + SCALE_SLOTS * SCALE_SLOT;
+constexpr int kThreads = 256;
+constexpr int WT = 128;                      // wave tile edge
+constexpr int NT = WT / 16;                  // MFMA tiles per wave tile edge
+constexpr int kLoads = 8;                    // direct loads per operand, step and wave (8 rows each)
+
+__device__ __forceinline__ int swz16(int r) { return (r >> 1) & 7; }
+
+template <typename Problem, int CBSZ_A, int BLGP_B>
+__global__ __launch_bounds__(kThreads, 1) void gemm_fp8_m16_kernel(Problem pb)
+{
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = wave >> 1, wn = wave & 1;
+    const int r16 = lane & 15, kb = lane >> 4;  // fragment row inside a tile; 32-byte K block of the lane
+
+    // ---- fragment read addresses of the stage being read (half q of the lane's 32 K bytes); tile t adds 2048 t
+    uint32_t ra[2], rb[2];
+    {
+        const uint32_t lds0 = (uint32_t)(uintptr_t)(lptr_t)lds;
+#pragma unroll
+        for (int q = 0; q < 2; ++q) {
+            const uint32_t chunk = (uint32_t)((2 * kb + q) ^ swz16(r16));
+            ra[q] = lds0 + (uint32_t)((wm * WT + r16) * BK) + (chunk << 4);
+            rb[q] = lds0 + (uint32_t)(BM * BK + (wn * WT + r16) * BK) + (chunk << 4);
+        }
+    }
+    auto flip_read_stage = [&](int to_stage) __attribute__((always_inline)) {
+        const uint32_t delta = to_stage ? (uint32_t)STAGE : (uint32_t)(-STAGE);
+#pragma unroll
+        for (int q = 0; q < 2; ++q) {
+            ra[q] += delta;
+            rb[q] += delta;
+        }
+    };
+    auto read_a = [&](v4i (&f)[2], int tile, int q) __attribute__((always_inline)) {
+        f[q] = *reinterpret_cast<lfrag_t>((uintptr_t)(ra[q] + tile * 16 * BK));
+    };
+    auto read_b = [&](v4i (&f)[2], int tile, int q) __attribute__((always_inline)) {
+        f[q] = *reinterpret_cast<lfrag_t>((uintptr_t)(rb[q] + tile * 16 * BK));
+    };
+
+    // ---- direct loads: wave w fills rows [64 w + 8 p, +8) of each operand, p = 0..7; lane -> row 64 w + 8 p + lr
+    // (lr = lane / 8), position lane % 8, which holds global chunk (lane % 8) ^ swz16(row); swz16(row) is
+    // 4 (p & 1) + lr / 2.  The load's lane offset is a resident register per operand and parity of p (row lr of
+    // the operand plus the chunk) plus a uniform row offset: one vector add next to the load, and few registers
+    // (this kernel runs at the 256-register limit, and a reload from scratch waits on the in-order vector memory
+    // counter, i.e. on every store and direct load before it).
+    const int lr = lane >> 3;
+    uint32_t dv[4];  // [operand][p & 1]
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+        const int64_t ld = k < 2 ? pb.lda : pb.ldb;
+        dv[k] = (uint32_t)((int64_t)lr * ld) + ((uint32_t)((lane & 7) ^ (((k & 1) << 2) | (lr >> 1))) << 4);
+    }
+    // x in 0..15: the first eight -> A rows 8 x, the rest -> B rows 8 (x - 8)
+    auto dma_one = [&](const uint8_t* a_origin, const uint8_t* b_origin, int stage, int x) __attribute__((always_inline)) {
+        const bool is_a = x < kLoads;
+        const int p = x % kLoads;
+        uint32_t rows = (uint32_t)((int64_t)(wave * 64 + 8 * p) * (is_a ? pb.lda : pb.ldb));
+        asm volatile("" : "+s"(rows));  // opaque: the sum stays one add at the load instead of sixteen resident registers
+        const uint32_t o = dv[(is_a ? 0 : 2) + (p & 1)] + rows;
+        const uint8_t* src = (is_a ? a_origin : b_origin) + o;
+        uint8_t* dst = lds + stage * STAGE + (is_a ? 0 : BM * BK) + (wave * 64 + 8 * (x % kLoads)) * BK;
+        __builtin_amdgcn_global_load_lds((gptr_t)src, (lptr_t)dst, 16, 0, 0);
+    };
+
+    // ---- scales.  Nothing in the epilogue may wait on a global load: such a wait also covers the stores of the
+    // previous pass and the operand loads in flight for the next tile (one in-order counter).  Single scales are
+    // read here, once; scale vectors travel through LDS like the operands: when the load cursor reaches a tile,
+    // each wave fetches its 64 row and 64 column scales into slot (tile index % 4) with two direct loads, and the
+    // waits and barriers of the K steps in between make them visible before the tile's epilogue.
+    float inv_single = 1.0f;
+    if constexpr (!Problem::kVecScales) {
+        inv_single = (1.0f / pb.single_sa()) * (1.0f / pb.single_sb());
+        asm volatile("" ::"v"(inv_single));  // the value is complete before the first direct load is issued
+    }
+    auto scale_dma = [&](const TileDesc& d, int tile_idx) __attribute__((always_inline)) {
+        if constexpr (Problem::kVecScales) {
+            uint8_t* slot = lds + 2 * STAGE + OUT_STAGING + (tile_idx & (SCALE_SLOTS - 1)) * SCALE_SLOT + wave * 256;
+            __builtin_amdgcn_global_load_lds((gptr_t)(d.sa + wave * 64 + lane), (lptr_t)slot, 4, 0, 0);
+            __builtin_amdgcn_global_load_lds((gptr_t)(d.sb + wave * 64 + lane), (lptr_t)(slot + 1024), 4, 0, 0);
+        }
+    };
+
+    // ---- this workgroup's tiles (see mi8_gemm_dma8.hip: XCD-contiguous ranges for tiles of equal cost, plain
+    // striding for tiles of unequal cost)
+    const typename Problem::Cache cache = pb.prepare();
+    const int total = pb.total_tiles(cache);
+    int first_tile, tile_stride, my_tiles;
+    if constexpr (Problem::kXcdRanges) {
+        const int per_xcd = (total + 7) / 8;
+        const int xcd = (int)blockIdx.x & 7;
+        const int slot = (int)blockIdx.x >> 3;
+        const int slots = ((int)gridDim.x + 7 - xcd) >> 3;
+        const int first = xcd * per_xcd;
+        int last = first + per_xcd;
+        last = last < total ? last : total;
+        first_tile = first + slot;
+        tile_stride = slots;
+        my_tiles = (first_tile < last) ? (last - first_tile + slots - 1) / slots : 0;
+    } else {
+        first_tile = (int)blockIdx.x;
+        tile_stride = (int)gridDim.x;
+        my_tiles = (first_tile < total) ? (total - first_tile + tile_stride - 1) / tile_stride : 0;
+    }
+    if (my_tiles == 0) return;
+    auto my_tile = [&](int idx) __attribute__((always_inline)) { return pb.tile(first_tile + idx * tile_stride, cache); };
+
+    // load cursor: the K step whose stage is fetched next (two steps ahead of the compute cursor); it skips
+    // tiles without K steps and, past the last tile, keeps fetching valid data nobody reads
+    int ld_tile = -1, ld_kt = 0, ld_nk = 0;
+    const uint8_t* ld_a = nullptr;
+    const uint8_t* ld_b = nullptr;
+    auto next_load_tile = [&]() __attribute__((always_inline)) {
+        while (ld_tile + 1 < my_tiles) {
+            ++ld_tile;
+            const TileDesc d = my_tile(ld_tile);
+            if (d.nk > 0) {
+                ld_a = d.a;
+                ld_b = d.b;
+                ld_nk = d.nk;
+                ld_kt = 0;
+                scale_dma(d, ld_tile);
+                return;
+            }
+        }
+        if (ld_a) {  // no further tile with work: rewind to the start of the current one
+            ld_a -= (int64_t)ld_kt * BK;
+            ld_b -= (int64_t)ld_kt * BK;
+            ld_kt = 0;
+        }
+    };
+    auto advance_load_cursor = [&]() __attribute__((always_inline)) {
+        ++ld_kt;
+        ld_a += BK;
+        ld_b += BK;
+        if (ld_kt >= ld_nk) next_load_tile();
+    };
+    next_load_tile();
+
+    v4f acc[NT][NT];
+    // D' = B . A^T : the first MFMA operand is the B fragment (its type code goes to cbsz).  `fresh`: the tile's
+    // first touch of this accumulator; the MFMA then takes the constant 0 as its addend, so the accumulators
+    // never have to be cleared between tiles.
+    auto mma = [&](const v4i (&a)[2], const v4i (&b)[2], v4f& c, bool fresh) __attribute__((always_inline)) {
+        const v8i fa = __builtin_shufflevector(a[0], a[1], 0, 1, 2, 3, 4, 5, 6, 7);
+        const v8i fb = __builtin_shufflevector(b[0], b[1], 0, 1, 2, 3, 4, 5, 6, 7);
+        const v4f zero = {0, 0, 0, 0};
+        c = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(fb, fa, fresh ? zero : c, BLGP_B, CBSZ_A, 0, 0, 0, 0);
+    };
+
+    // ---- prologue: stages of steps 0 and 1, fragments of step 0 ----------------------------------------
+    if (ld_a != nullptr) {  // uniform
+#pragma unroll
+        for (int s = 0; s < 2; ++s) {
+#pragma unroll
+            for (int x = 0; x < 2 * kLoads; ++x) dma_one(ld_a, ld_b, s, x);
+            advance_load_cursor();
+        }
+    }
+    v4i fa_lo[4][2], fa_hi[4][2], fb[NT][2];  // A tiles 0-3, A tiles 4-7, B tiles 0-7
+    // fragments a step's phase A starts from: A tiles 0-3 and all B tiles of the stage the read addresses point at
+    auto read_step_head = [&]() __attribute__((always_inline)) {
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+            read_a(fa_lo[t], t, 0);
+            read_a(fa_lo[t], t, 1);
+        }
+#pragma unroll
+        for (int t = 0; t < NT; ++t) {
+            read_b(fb[t], t, 0);
+            read_b(fb[t], t, 1);
+        }
+    };
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wave's direct loads have landed
+    __syncthreads();
+    read_step_head();
+
+    int step = 0;
+    for (int cp_tile = 0; cp_tile < my_tiles; ++cp_tile) {
+        const TileDesc td = my_tile(cp_tile);
+        // One 128-byte K step.  `fresh`: the tile's first step; phase A touches the accumulators of A tiles 0-3,
+        // phase B those of A tiles 4-7, so both start from 0 then.  The first step is written out separately
+        // from the loop, not as a branch inside it.
+        auto k_step = [&](bool fresh) __attribute__((always_inline)) {
+            const int cur = step & 1;
+            // every wave has issued its reads of this stage's B rows and A tiles 0-3 (previous phase B)
+            asm volatile("s_barrier" ::: "memory");
+            // phase A: this step's A tiles 4-7 are read behind the first eight MFMAs; the B half of step + 2 is
+            // fetched into the B rows of this stage
+#pragma unroll
+            for (int x = 0; x < 32; ++x) {
+                const int j = x >> 2, i = x & 3;
+                mma(fa_lo[i], fb[j], acc[i][j], fresh);
+                if (x < 8) read_a(fa_hi[x >> 1], 4 + (x >> 1), x & 1);
+                if (x >= 8 && x % 3 == 2) dma_one(ld_a, ld_b, cur, kLoads + (x - 8) / 3);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            // All but this phase's eight loads have landed: the other stage (step + 1) is complete.  (The
+            // compiler does not track direct-to-LDS loads across a barrier.)
+            __builtin_amdgcn_s_waitcnt(0x0F78);  // vmcnt(8)
+            asm volatile("s_barrier" ::: "memory");
+            flip_read_stage(cur ^ 1);
+            // phase B, B tile by B tile: the next step's copy of a B tile is read once its four MFMAs are issued;
+            // the A half of step + 2 is fetched into the A rows of this stage
+#pragma unroll
+            for (int x = 0; x < 32; ++x) {
+                const int j = x >> 2, i = x & 3;
+                mma(fa_hi[i], fb[j], acc[4 + i][j], fresh);
+                if (x < 8) read_a(fa_lo[x >> 1], x >> 1, x & 1);
+                if (i == 3) {
+                    read_b(fb[j], j, 0);
+                    read_b(fb[j], j, 1);
+                }
+                if (i == 1) dma_one(ld_a, ld_b, cur, x >> 2);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            advance_load_cursor();
+            ++step;
+        };
+        if (td.nk > 0) {
+            k_step(true);
+            for (int kt = 1; kt < td.nk; ++kt) k_step(false);
+        } else {  // nothing is accumulated (empty group): the tile is all zeros
+#pragma unroll
+            for (int i = 0; i < NT; ++i)
+#pragma unroll
+                for (int j = 0; j < NT; ++j) acc[i][j] = (v4f){0, 0, 0, 0};
+        }
+
+        // ---- tile finished: epilogue -------------------------------------------------------------------
+        // acc[i][j][e] of lane l is C[row = 16 i + l%16][col = 16 j + 4 (l/16) + e] of the wave tile.
+        // A single scale is inverted with an IEEE division, scale vectors with v_rcp_f32 (exact for the
+        // power-of-two scales of the axiswise recipes, within 1 ulp otherwise).
+        // The wave's output goes through its private staging area 32 rows x 64 columns at a time (4 KB, pitch 128
+        // bytes, 16-byte chunk index XORed with (row >> 1) & 7), i.e. two A tiles by four B tiles per pass.
+        uint8_t* stg = lds + 2 * STAGE + wave * 4096;
+        const uint32_t stg_lds = (uint32_t)(uintptr_t)(lptr_t)stg;
+        const bool zero_tile = td.nk == 0;  // nothing accumulated; the scales may be unset
+        const uint8_t* sc_slot = lds + 2 * STAGE + OUT_STAGING + (cp_tile & (SCALE_SLOTS - 1)) * SCALE_SLOT;
+        const int ldc_bytes = (int)pb.ldc * 2;
+        const uint32_t c_lane_off = (uint32_t)((lane >> 3) * ldc_bytes + (lane & 7) * 16);
+        __amdgpu_buffer_rsrc_t c_rows;
+        if constexpr (Problem::kMaskRows)
+            c_rows = __builtin_amdgcn_make_buffer_rsrc(td.c + (int64_t)td.row_lo * pb.ldc, 0,
+                                                       (td.row_hi - td.row_lo) * ldc_bytes, 0x00020000);
+#pragma unroll
+        for (int jq = 0; jq < 2; ++jq) {
+            float isb[4][4];
+            if constexpr (Problem::kVecScales) {
+#pragma unroll
+                for (int jj = 0; jj < 4; ++jj) {
+                    const float4 s4 =
+                        *reinterpret_cast<const float4*>(sc_slot + 1024 + (wn * WT + jq * 64 + 16 * jj + 4 * kb) * 4);
+                    isb[jj][0] = zero_tile ? 0.0f : __builtin_amdgcn_rcpf(s4.x);
+                    isb[jj][1] = zero_tile ? 0.0f : __builtin_amdgcn_rcpf(s4.y);
+                    isb[jj][2] = zero_tile ? 0.0f : __builtin_amdgcn_rcpf(s4.z);
+                    isb[jj][3] = zero_tile ? 0.0f : __builtin_amdgcn_rcpf(s4.w);
+                }
+            }
+#pragma unroll
+            for (int ih = 0; ih < 4; ++ih) {
+                const int rt = wm * WT + ih * 32;  // first tile row of this pass
+#pragma unroll
+                for (int t = 0; t < 2; ++t) {
+                    // A single scale is made opaque in every pass: with a loop-invariant multiplier the compiler
+                    // forms the products of the whole tile up front and spills accumulators.
+                    float mult = inv_single;
+                    if constexpr (Problem::kVecScales)
+                        mult = __builtin_amdgcn_rcpf(*reinterpret_cast<const float*>(sc_slot + (rt + 16 * t + r16) * 4));
+                    else
+                        asm volatile("" : "+v"(mult));
+                    mult = zero_tile ? 0.0f : mult;
+                    const int row = 16 * t + r16;
+#pragma unroll
+                    for (int jj = 0; jj < 4; ++jj) {
+                        const int cw = 16 * jj + 4 * kb;  // column inside the 64-column pass, multiple of 4
+                        float v[4];
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) {
+                            v[e] = acc[2 * ih + t][4 * jq + jj][e] * mult;
+                            if constexpr (Problem::kVecScales) v[e] *= isb[jj][e];
+                        }
+                        uint2 o;
+                        o.x = pack_bf16x2(v[0], v[1]);
+                        o.y = pack_bf16x2(v[2], v[3]);
+                        const int chunk = (cw >> 3) ^ ((row >> 1) & 7);
+                        // Written as an instruction of its own: before an LDS store it knows of, the compiler
+                        // waits for every direct-to-LDS load in flight (it cannot tell that they target other
+                        // addresses), i.e. for the operand loads already issued for the next tile.
+                        const uint32_t saddr = stg_lds + (uint32_t)(row * 128 + chunk * 16 + (cw & 4) * 2);
+                        asm volatile("ds_write_b64 %0, %1" ::"v"(saddr), "v"(o) : "memory");
+                    }
+                }
+                __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): the wave's own LDS writes have landed
+                __builtin_amdgcn_wave_barrier();
+                v4i staged[4];  // (an ext-vector type: arrays of HIP's uint4 struct end up in scratch)
+#pragma unroll
+                for (int it = 0; it < 4; ++it) {
+                    const int rw = it * 8 + (lane >> 3);
+                    staged[it] = *reinterpret_cast<const v4i*>(stg + rw * 128 + (((lane & 7) ^ ((rw >> 1) & 7)) << 4));
+                }
+                if constexpr (Problem::kMaskRows) {
+                    // Only rows [row_lo, row_hi) of the tile belong to this tile's group.  The stores go through a
+                    // buffer descriptor that spans exactly those rows: a lane whose row lies outside gets an
+                    // offset below zero (huge when read as unsigned) or past the end, and the hardware drops its
+                    // store - no divergent branches around the stores.
+                    const int voff = (rt + (lane >> 3) - td.row_lo) * ldc_bytes + (wn * WT + jq * 64 + (lane & 7) * 8) * 2;
+#pragma unroll
+                    for (int it = 0; it < 4; ++it)
+                        __builtin_amdgcn_raw_buffer_store_b128(staged[it], c_rows, voff + it * 8 * ldc_bytes, 0, 0);
+                } else {
+                    // uniform 64-bit base + one 32-bit lane offset shared by all passes (no per-pass lane pointers)
+#pragma unroll
+                    for (int it = 0; it < 4; ++it) {
+                        uint8_t* base = reinterpret_cast<uint8_t*>(td.c + (int64_t)(rt + it * 8) * pb.ldc + wn * WT + jq * 64);
+                        uint32_t o = c_lane_off;
+                        asm volatile("" : "+v"(o));
+                        *reinterpret_cast<v4i*>(base + o) = staged[it];
+                    }
+                }
+                __builtin_amdgcn_s_waitcnt(0xc07f);  // the reads are done before the next pass overwrites
+                __builtin_amdgcn_wave_barrier();
+            }
+        }
+        // The last step's phase B has read the next tile's first fragments like any other step; reading them
+        // again here makes those 96 registers free during the epilogue, which otherwise spills (and every
+        // reload from scratch waits on the in-order vector memory counter, i.e. on the stores above).
+        read_step_head();
+    }
+    // direct loads issued for steps past the end must have landed before the LDS allocation is released
+    __builtin_amdgcn_s_waitcnt(0x0070);  // vmcnt(0) lgkmcnt(0)
+    __syncthreads();
+}
+
+int num_cus()
+{
+    static int cached = 0;
+    if (cached == 0) {
+        int dev = 0, n = 0;
+        if (hipGetDevice(&dev) != hipSuccess ||
+            hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0)
+            n = 256;
+        cached = n;
+    }
+    return cached;
+}
+
+// persistent: one workgroup per CU walks a static share of the tiles (right when all tiles cost the same);
+// otherwise one workgroup per tile, handed to free CUs by the hardware dispatcher (tiles of unequal cost).
+template <typename Problem, int CBSZ_A, int BLGP_B>
+int launch(const Problem& pb, int max_tiles, bool persistent, hipStream_t st)
+{
+    auto kern = gemm_fp8_m16_kernel<Problem, CBSZ_A, BLGP_B>;
+    static bool configured = false;
+    if (!configured) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES);
+        if (e != hipSuccess) {
+            set_error("mi8 16x16x128 GEMM: cannot reserve %d bytes of LDS: %s", LDS_BYTES, hipGetErrorString(e));
+            return MI8_ERR_LAUNCH;
+        }
+        configured = true;
+    }
+    int blocks = persistent ? num_cus() : max_tiles;
+    if (blocks > max_tiles) blocks = max_tiles;
+    hipLaunchKernelGGL(kern, dim3(blocks), dim3(kThreads), LDS_BYTES, st, pb);
+    return launch_status("mi8 16x16x128 GEMM");
+}
+
+template <typename Problem>
+int launch_typed(const Problem& pb, int max_tiles, bool persistent, int a_dtype, int b_dtype, hipStream_t st)
+{
+    if (a_dtype == MI8_E4M3)
+        return b_dtype == MI8_E4M3 ? launch<Problem, 0, 0>(pb, max_tiles, persistent, st)
+                                   : launch<Problem, 0, 1>(pb, max_tiles, persistent, st);
+    return b_dtype == MI8_E4M3 ? launch<Problem, 1, 0>(pb, max_tiles, persistent, st)
+                               : launch<Problem, 1, 1>(pb, max_tiles, persistent, st);
+}
+
+}  // namespace
+
+int launch_m16(GemmArgs& g, int a_dtype, int b_dtype, hipStream_t st)
+{
+    g.tiles_m = (g.M + BM - 1) / BM;
+    g.tiles_n = (g.N + BN - 1) / BN;
+    if (g.sa_vec) {
+        DenseProblem<true> pb{g, g.lda, g.ldb, g.ldc};
+        return launch_typed(pb, g.tiles_m * g.tiles_n, true, a_dtype, b_dtype, st);
+    }
+    DenseProblem<false> pb{g, g.lda, g.ldb, g.ldc};
+    return launch_typed(pb, g.tiles_m * g.tiles_n, true, a_dtype, b_dtype, st);
+}
+
+int launch_m16_grouped(const uint8_t* a, int a_dtype, int64_t lda, const uint8_t* b, int b_dtype, int64_t ldb,
+                       int64_t b_group_stride, const int64_t* sizes, int E, int64_t T, int N, int K, const float* sa,
+                       const float* sb, int64_t sb_group_stride, uint16_t* out, int64_t ldc, hipStream_t st)
+{
+    const int tiles_n = (N + BN - 1) / BN;
+    GroupedProblem pb{a, b, out, lda, ldb, ldc, b_group_stride, sb_group_stride, sizes, E, T, N, K, tiles_n, sa, sb};
+    const int64_t max_tiles = ((T + BM - 1) / BM + E) * tiles_n;
+    return launch_typed(pb, max_tiles > (1 << 30) ? (1 << 30) : (int)max_tiles, true, a_dtype, b_dtype, st);
+}
+
+int launch_m16_grouped_wgrad(const uint8_t* a_t, int a_dtype, const uint8_t* b_t, int b_dtype, int64_t ld_t,
+                             const int64_t* sizes, int E, int64_t T, int N, int Kl, const float* sa, const float* sb,
+                             uint16_t* out, hipStream_t st)
+{
+    const int tiles_n = (N + BM - 1) / BM, tiles_k = (Kl + BN - 1) / BN;
+    GroupedWgradProblem pb{a_t, b_t, out, ld_t, ld_t, Kl, sizes, E, T, N, Kl, tiles_n, tiles_k, sa, sb};
+    return launch_typed(pb, E * tiles_n * tiles_k, false, a_dtype, b_dtype, st);
+}
+
+}  // namespace gemm
+}  // namespace mi8

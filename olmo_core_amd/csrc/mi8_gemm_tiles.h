@@ -1,0 +1,261 @@
+// Problem policies of the persistent direct-to-LDS fp8 GEMM kernels: how a linear tile index maps to operand
+// panels, scales and output rows for the dense problem and for the ragged grouped problems (forward /
+// grad_input and grad_weight of a dropless-MoE expert layer).  Shared by the 32x32x64 and 16x16x128 kernels.
+#pragma once
+#include "mi8_gemm.h"
+
+namespace mi8 {
+namespace gemm {
+namespace {
+
+constexpr int BM = 256, BN = 256;  // output tile of one workgroup
+
+// ---- what a workgroup needs to know about one output tile ---------------------------------------------
+struct TileDesc {
+    const uint8_t* a;  // first A row of the tile (K offset 0 of the tile's contraction range)
+    const uint8_t* b;  // first B row of the tile
+    int nk;            // 128-byte K steps (0: the tile is all zeros)
+    const float* sa;   // scale of the tile's first row (or the single scale)
+    const float* sb;   // scale of the tile's first column (or the single scale)
+    uint16_t* c;       // C element (first row, first column) of the tile
+    int row_lo, row_hi;  // rows [row_lo, row_hi) of the 256 are stored
+};
+
+struct NoCache {};
+
+// Dense problem: C[M, N] = A[M, K] . B[N, K]^T.  The last tile row / column is shifted back so that every tile
+// is full (M, N >= 256): the overlap is recomputed with the same K order and rewritten with identical values.
+template <bool VEC>
+struct DenseProblem {
+    GemmArgs g;
+    int64_t lda, ldb, ldc;
+    static constexpr bool kVecScales = VEC;  // both scales are vectors (per row / per column) or both single
+    static constexpr bool kMaskRows = false, kXcdRanges = true, kPeelFirstStep = true;
+    using Cache = NoCache;
+    __device__ __forceinline__ Cache prepare() const { return Cache{}; }
+    __device__ __forceinline__ int total_tiles(const Cache&) const { return g.tiles_m * g.tiles_n; }
+    // (single-scale problems only) the two scales, the same for every tile
+    __device__ __forceinline__ float single_sa() const { return g.sa[0]; }
+    __device__ __forceinline__ float single_sb() const { return g.sb[0]; }
+    __device__ __forceinline__ TileDesc tile(int t, const Cache&) const
+    {
+        int tm, tn;
+        tile_coords(g, t, tm, tn);
+        const int m0 = (tm * BM + BM <= g.M) ? tm * BM : g.M - BM;
+        const int n0 = (tn * BN + BN <= g.N) ? tn * BN : g.N - BN;
+        TileDesc d;
+        d.a = g.A + (int64_t)m0 * g.lda;
+        d.b = g.B + (int64_t)n0 * g.ldb;
+        d.nk = g.K / BK;
+        d.sa = g.sa + (VEC ? m0 : 0);
+        d.sb = g.sb + (VEC ? n0 : 0);
+        d.c = reinterpret_cast<uint16_t*>(g.C) + (int64_t)m0 * g.ldc + n0;
+        d.row_lo = 0;
+        d.row_hi = BM;
+        return d;
+    }
+};
+
+// ---- locating a group in the device-resident size list ---------------------------------------------------
+// Groups are consecutive row ranges; sizes are clamped so that their running sum never passes T.  A group of
+// m rows owns ceil(m / U) "units" (row tiles).  The 64 lanes of a wave each take one group of a 64-group chunk
+// and prefix-sum rows and units with shuffles, so a lookup costs one load latency instead of E dependent
+// ones.  Must be called by all lanes of the wave together; the result is wave-uniform.
+struct GroupSpan {
+    int e;                 // group index (E if the key is past the end)
+    int64_t rows_before;   // rows of the groups before it
+    int64_t m;             // its clamped size
+    int64_t units_before;  // units of the groups before it (all units if the key is past the end)
+};
+
+__device__ __forceinline__ int64_t uniform64(int64_t v)
+{
+    const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v);
+    const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)((uint64_t)v >> 32));
+    return (int64_t)(((uint64_t)hi << 32) | lo);
+}
+
+__device__ __forceinline__ int64_t wave_inclusive_sum(int64_t v, int lane)
+{
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+        const int64_t o = __shfl_up(v, d, 64);
+        if (lane >= d) v += o;
+    }
+    return v;
+}
+
+// BY_UNIT: key is a unit index, find the group that owns it; otherwise key is the group index itself.
+template <int U, bool BY_UNIT>
+__device__ __forceinline__ GroupSpan locate_group(const int64_t* sizes, int E, int64_t T, int64_t key)
+{
+    const int lane = (int)threadIdx.x & 63;
+    int64_t rows_c = 0, units_c = 0;
+    for (int base = 0; base < E; base += 64) {
+        const int e = base + lane;
+        int64_t m = (e < E) ? sizes[e] : 0;
+        m = m < 0 ? 0 : (m > T ? T : m);
+        int64_t end = rows_c + wave_inclusive_sum(m, lane);
+        int64_t start = end - m;
+        end = end < T ? end : T;
+        start = start < T ? start : T;
+        const int64_t me = end - start;
+        const int64_t un = (me + U - 1) / U;
+        const int64_t uend = units_c + wave_inclusive_sum(un, lane);
+        const bool hit = (e < E) && (BY_UNIT ? key < uend : key == e);
+        const uint64_t mask = __ballot(hit);
+        if (mask) {
+            const int src = __ffsll((unsigned long long)mask) - 1;
+            GroupSpan r;
+            r.e = base + src;
+            r.rows_before = uniform64(__shfl(start, src, 64));
+            r.m = uniform64(__shfl(me, src, 64));
+            r.units_before = uniform64(__shfl(uend - un, src, 64));
+            return r;
+        }
+        rows_c = uniform64(__shfl(end, 63, 64));
+        units_c = uniform64(__shfl(uend, 63, 64));
+    }
+    return GroupSpan{E, rows_c, 0, units_c};
+}
+
+// Up to 64 groups: the prefix sums live in four registers of every wave for the whole kernel (lane e holds
+// group e), and a lookup is a ballot and three lane reads, with no memory access inside the K loop.
+struct GroupCache {
+    int start, m, ubefore, uend;  // per lane: first row, clamped size, units before, units up to and including
+    bool valid;                   // wave-uniform: E <= 64 (otherwise lookups go to memory)
+};
+
+template <int U>
+__device__ __forceinline__ GroupCache build_group_cache(const int64_t* sizes, int E, int64_t T)
+{
+    GroupCache c{0, 0, 0, 0, E <= 64};
+    if (!c.valid) return c;
+    const int lane = (int)threadIdx.x & 63;
+    int64_t m = (lane < E) ? sizes[lane] : 0;
+    m = m < 0 ? 0 : (m > T ? T : m);
+    int64_t end = wave_inclusive_sum(m, lane);
+    int64_t start = end - m;
+    end = end < T ? end : T;
+    start = start < T ? start : T;
+    const int64_t me = end - start;
+    const int64_t un = (me + U - 1) / U;
+    const int64_t uend = wave_inclusive_sum(un, lane);
+    c.start = (int)start;  // T < 2^30 is checked on the host
+    c.m = (int)me;
+    c.ubefore = (int)(uend - un);
+    c.uend = (int)uend;
+    return c;
+}
+
+template <int U, bool BY_UNIT>
+__device__ __forceinline__ GroupSpan locate_group_cached(const GroupCache& c, const int64_t* sizes, int E, int64_t T,
+                                                         int64_t key)
+{
+    if (!c.valid) return locate_group<U, BY_UNIT>(sizes, E, T, key);
+    int src;
+    if constexpr (BY_UNIT) {
+        const uint64_t mask = __ballot((int64_t)c.uend > key);
+        if (mask == 0) return GroupSpan{E, T, 0, __builtin_amdgcn_readlane(c.uend, 63)};
+        src = __ffsll((unsigned long long)mask) - 1;
+    } else {
+        src = (int)key;
+    }
+    GroupSpan r;
+    r.e = src;
+    r.rows_before = __builtin_amdgcn_readlane(c.start, src);
+    r.m = __builtin_amdgcn_readlane(c.m, src);
+    r.units_before = __builtin_amdgcn_readlane(c.ubefore, src);
+    return r;
+}
+
+// Ragged-M grouped problem (dropless-MoE forward / grad_input): rows of A form consecutive groups, group e
+// multiplies B_e = B + e * b_group_stride.  A tile covers up to 256 rows of ONE group; it always loads a full
+// 256-row window (shifted back at the end of the matrix, T >= 256) and stores only its group's rows.
+struct GroupedProblem {
+    const uint8_t* A;
+    const uint8_t* B;
+    uint16_t* C;
+    int64_t lda, ldb, ldc, b_group_stride, sb_group_stride;
+    const int64_t* sizes;
+    int E;
+    int64_t T;
+    int N, K, tiles_n;
+    const float* sa;
+    const float* sb;
+    static constexpr bool kVecScales = true, kMaskRows = true, kXcdRanges = true, kPeelFirstStep = false;
+    using Cache = GroupCache;
+    __device__ __forceinline__ Cache prepare() const { return build_group_cache<BM>(sizes, E, T); }
+    __device__ __forceinline__ int total_tiles(const Cache& c) const
+    {
+        const GroupSpan s = locate_group_cached<BM, true>(c, sizes, E, T, (int64_t)1 << 60);
+        return (int)s.units_before * tiles_n;
+    }
+    __device__ __forceinline__ TileDesc tile(int t, const Cache& c) const
+    {
+        const int mt = t / tiles_n, nt = t % tiles_n;
+        const GroupSpan s = locate_group_cached<BM, true>(c, sizes, E, T, mt);
+        const int64_t want0 = s.rows_before + (mt - s.units_before) * BM;  // first row this tile is responsible for
+        int64_t want1 = want0 + BM;
+        const int64_t group_end = s.rows_before + s.m;
+        want1 = want1 < group_end ? want1 : group_end;                     // ... up to the group's end
+        const int64_t m0 = (want0 + BM <= T) ? want0 : T - BM;             // loaded window
+        const int n0 = (nt * BN + BN <= N) ? nt * BN : N - BN;
+        TileDesc d;
+        d.a = A + m0 * lda;
+        d.b = B + (int64_t)s.e * b_group_stride + (int64_t)n0 * ldb;
+        d.nk = K / BK;
+        d.sa = sa + m0;
+        d.sb = sb + (int64_t)s.e * sb_group_stride + n0;
+        d.c = C + m0 * ldc + n0;
+        d.row_lo = (int)(want0 - m0);
+        d.row_hi = (int)(want1 - m0);
+        return d;
+    }
+};
+
+// Ragged-K grouped problem (dropless-MoE grad_weight): out[e] = A_t[:, S_e] . B_t[:, S_e]^T over group e's
+// 128-aligned segment S_e of the padded token axis; N, Kl >= 256.  An empty group gives nk = 0: its tiles are
+// written as zeros and its scales (never produced) are ignored.
+struct GroupedWgradProblem {
+    const uint8_t* At;
+    const uint8_t* Bt;
+    uint16_t* C;
+    int64_t lda, ldb, ldc;  // lda = ldb = padded token pitch, ldc = Kl
+    const int64_t* sizes;
+    int E;
+    int64_t T;
+    int N, Kl, tiles_n, tiles_k;
+    const float* sa;  // [E, N]
+    const float* sb;  // [E, Kl]
+    static constexpr bool kVecScales = true, kMaskRows = false, kXcdRanges = false, kPeelFirstStep = true;
+    using Cache = GroupCache;
+    __device__ __forceinline__ Cache prepare() const { return build_group_cache<128>(sizes, E, T); }
+    __device__ __forceinline__ int total_tiles(const Cache&) const { return E * tiles_n * tiles_k; }
+    __device__ __forceinline__ TileDesc tile(int t, const Cache& c) const
+    {
+        const int per_group = tiles_n * tiles_k;
+        const int e = t / per_group, rem = t % per_group;
+        const int tn = rem / tiles_k, tk = rem % tiles_k;
+        const GroupSpan s = locate_group_cached<128, false>(c, sizes, E, T, e);
+        const int64_t seg0 = 128 * s.units_before;
+        int64_t seg = 128 * ((s.m + 127) / 128);
+        if (seg0 + seg > lda) seg = 0;
+        const int n0 = (tn * BM + BM <= N) ? tn * BM : N - BM;
+        const int k0 = (tk * BN + BN <= Kl) ? tk * BN : Kl - BN;
+        TileDesc d;
+        d.a = At + (int64_t)n0 * lda + seg0;
+        d.b = Bt + (int64_t)k0 * ldb + seg0;
+        d.nk = (int)(seg / BK);
+        d.sa = sa + (int64_t)e * N + n0;
+        d.sb = sb + (int64_t)e * Kl + k0;
+        d.c = C + ((int64_t)e * N + n0) * ldc + k0;
+        d.row_lo = 0;
+        d.row_hi = BM;
+        return d;
+    }
+};
+
+}  // namespace
+}  // namespace gemm
+}  // namespace mi8
