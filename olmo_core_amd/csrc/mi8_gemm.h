@@ -81,20 +81,14 @@ int launch_dma8(GemmArgs& g, int a_dtype, int b_dtype, hipStream_t st);
 int launch_dma4(GemmArgs& g, int a_dtype, int b_dtype, hipStream_t st);
 // four waves of 128 x 128 on 16x16x128 MFMAs (mi8_gemm_m16.hip), same requirements
 int launch_m16(GemmArgs& g, int a_dtype, int b_dtype, hipStream_t st);
+// the same kernel over the ragged grouped problems (bf16 output, per-row / per-column scale vectors):
+// forward / grad_input (T, N >= 256, K % 128 == 0) and grad_weight (N, Kl >= 256)
 int launch_m16_grouped(const uint8_t* a, int a_dtype, int64_t lda, const uint8_t* b, int b_dtype, int64_t ldb,
                        int64_t b_group_stride, const int64_t* sizes, int E, int64_t T, int N, int K, const float* sa,
                        const float* sb, int64_t sb_group_stride, uint16_t* out, int64_t ldc, hipStream_t st);
 int launch_m16_grouped_wgrad(const uint8_t* a_t, int a_dtype, const uint8_t* b_t, int b_dtype, int64_t ld_t,
                              const int64_t* sizes, int E, int64_t T, int N, int Kl, const float* sa, const float* sb,
                              uint16_t* out, hipStream_t st);
-// The same kernel over the ragged grouped problems (bf16 output, per-row / per-column scale vectors):
-// forward / grad_input (T, N >= 256, K % 128 == 0) and grad_weight (N, Kl >= 256).
-int launch_dma8_grouped(const uint8_t* a, int a_dtype, int64_t lda, const uint8_t* b, int b_dtype, int64_t ldb,
-                        int64_t b_group_stride, const int64_t* sizes, int E, int64_t T, int N, int K, const float* sa,
-                        const float* sb, int64_t sb_group_stride, uint16_t* out, int64_t ldc, hipStream_t st);
-int launch_dma8_grouped_wgrad(const uint8_t* a_t, int a_dtype, const uint8_t* b_t, int b_dtype, int64_t ld_t,
-                              const int64_t* sizes, int E, int64_t T, int N, int Kl, const float* sa, const float* sb,
-                              uint16_t* out, hipStream_t st);
 
 }  // namespace gemm
 }  // namespace mi8

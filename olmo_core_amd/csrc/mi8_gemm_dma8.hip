@@ -27,7 +27,6 @@ constexpr int WTM = 128, TM = 4;               // two waves along M, each 4 MFMA
 constexpr int STAGE = (BM + BN) * BK;          // 64 KB
 constexpr int OUT_STAGING = 8 * 4096;           // 4 KB of output staging per wave
 constexpr int LDS_BYTES = 2 * STAGE + OUT_STAGING;
-constexpr int kGroupedWN = 2;  // wave layout of the ragged problems (2 x 2 measured faster than 2 x 4)
 
 // The wave layout is 2 x WN.  WN = 4: eight waves of 128 x 64 (two per SIMD, 256 registers each).  WN = 2: four
 // waves of 128 x 128 (one per SIMD, 512 registers: twice the accumulators, a third less LDS read traffic, but no
@@ -473,26 +472,6 @@ int launch_dma4(GemmArgs& g, int a_dtype, int b_dtype, hipStream_t st)
     }
     DenseProblem<false> pb{g, g.lda, g.ldb, g.ldc};
     return launch_typed<DenseProblem<false>, 2>(pb, g.tiles_m * g.tiles_n, true, a_dtype, b_dtype, st);
-}
-
-int launch_dma8_grouped(const uint8_t* a, int a_dtype, int64_t lda, const uint8_t* b, int b_dtype, int64_t ldb,
-                        int64_t b_group_stride, const int64_t* sizes, int E, int64_t T, int N, int K, const float* sa,
-                        const float* sb, int64_t sb_group_stride, uint16_t* out, int64_t ldc, hipStream_t st)
-{
-    const int tiles_n = (N + BN - 1) / BN;
-    GroupedProblem pb{a, b, out, lda, ldb, ldc, b_group_stride, sb_group_stride, sizes, E, T, N, K, tiles_n, sa, sb};
-    const int64_t max_tiles = ((T + BM - 1) / BM + E) * tiles_n;
-    return launch_typed<GroupedProblem, kGroupedWN>(pb, max_tiles > (1 << 30) ? (1 << 30) : (int)max_tiles, true, a_dtype,
-                                                        b_dtype, st);
-}
-
-int launch_dma8_grouped_wgrad(const uint8_t* a_t, int a_dtype, const uint8_t* b_t, int b_dtype, int64_t ld_t,
-                              const int64_t* sizes, int E, int64_t T, int N, int Kl, const float* sa, const float* sb,
-                              uint16_t* out, hipStream_t st)
-{
-    const int tiles_n = (N + BM - 1) / BM, tiles_k = (Kl + BN - 1) / BN;
-    GroupedWgradProblem pb{a_t, b_t, out, ld_t, ld_t, Kl, sizes, E, T, N, Kl, tiles_n, tiles_k, sa, sb};
-    return launch_typed<GroupedWgradProblem, kGroupedWN>(pb, E * tiles_n * tiles_k, false, a_dtype, b_dtype, st);
 }
 
 }  // namespace gemm

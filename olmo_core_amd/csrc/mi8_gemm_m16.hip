@@ -277,6 +277,8 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_fp8_m16_kernel(Problem pb)
         // power-of-two scales of the axiswise recipes, within 1 ulp otherwise).
         // The wave's output goes through its private staging area 32 rows x 64 columns at a time (4 KB, pitch 128
         // bytes, 16-byte chunk index XORed with (row >> 1) & 7), i.e. two A tiles by four B tiles per pass.
+        // (the copies below are opaque to the compiler's hazard handling: the last MFMA has retired after these)
+        asm volatile("s_nop 15\n\ts_nop 15");
         uint8_t* stg = lds + 2 * STAGE + wave * 4096;
         const uint32_t stg_lds = (uint32_t)(uintptr_t)(lptr_t)stg;
         const bool zero_tile = td.nk == 0;  // nothing accumulated; the scales may be unset
@@ -321,7 +323,12 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_fp8_m16_kernel(Problem pb)
                         float v[4];
 #pragma unroll
                         for (int e = 0; e < 4; ++e) {
-                            v[e] = acc[2 * ih + t][4 * jq + jj][e] * mult;
+                            // The copy out of the accumulator file is an instruction of its own, ordered with the
+                            // LDS stores of the passes before it: left to the scheduler, all 256 copies move to
+                            // the top of the epilogue and the kernel spills.
+                            float a_;
+                            asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(a_) : "a"(acc[2 * ih + t][4 * jq + jj][e]));
+                            v[e] = a_ * mult;
                             if constexpr (Problem::kVecScales) v[e] *= isb[jj][e];
                         }
                         uint2 o;
@@ -369,6 +376,7 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_fp8_m16_kernel(Problem pb)
         // The last step's phase B has read the next tile's first fragments like any other step; reading them
         // again here makes those 96 registers free during the epilogue, which otherwise spills (and every
         // reload from scratch waits on the in-order vector memory counter, i.e. on the stores above).
+        __builtin_amdgcn_sched_barrier(0);  // (or the scheduler moves these reads up into the epilogue)
         read_step_head();
     }
     // direct loads issued for steps past the end must have landed before the LDS allocation is released

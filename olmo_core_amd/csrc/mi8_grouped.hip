@@ -208,7 +208,7 @@ extern "C" int mi8_grouped_gemm_fp8(const void* a, int a_dtype, int64_t lda, con
     // full-tile shapes with bf16 output run on the persistent direct-to-LDS kernel
     if (out_dtype == MI8_BF16 && T >= 256 && N >= 256 && K % 128 == 0 && N % 8 == 0 && ldc % 8 == 0 && aligned16(out) &&
         sb_group_stride % 4 == 0 && aligned16(sb) && lda < (1 << 23) && ldb < (1 << 23) && ldc < (1 << 22))
-        return launch_dma8_grouped((const uint8_t*)a, a_dtype, lda, (const uint8_t*)b, b_dtype, ldb, b_group_stride,
+        return launch_m16_grouped((const uint8_t*)a, a_dtype, lda, (const uint8_t*)b, b_dtype, ldb, b_group_stride,
                                    group_sizes, num_groups, T, (int)N, (int)K, sa, sb, sb_group_stride, (uint16_t*)out,
                                    ldc, st);
     if (a_dtype == MI8_E4M3)
@@ -237,7 +237,7 @@ extern "C" int mi8_grouped_wgrad_fp8(const void* a_t, int a_dtype, const void* b
     hipStream_t st = (hipStream_t)stream;
     if (out_dtype == MI8_BF16 && N >= 256 && Kl >= 256 && Kl % 8 == 0 && aligned16(out) && aligned16(sb) &&
         ld_t % 128 == 0 && ld_t < (1 << 23))
-        return launch_dma8_grouped_wgrad((const uint8_t*)a_t, a_dtype, (const uint8_t*)b_t, b_dtype, ld_t, group_sizes,
+        return launch_m16_grouped_wgrad((const uint8_t*)a_t, a_dtype, (const uint8_t*)b_t, b_dtype, ld_t, group_sizes,
                                          num_groups, T, (int)N, (int)Kl, sa, sb, (uint16_t*)out, st);
     if (a_dtype == MI8_E4M3)
         return b_dtype == MI8_E4M3 ? launch_wgrad<0, 0>(g, blocks, st) : launch_wgrad<0, 1>(g, blocks, st);
