@@ -18,10 +18,10 @@
 //
 // Fragment registers: 32 (A 0-3) + 32 (A 4-7) + 64 (B) = 128.
 //
-// LDS: two 64 KB operand stages [row][128 B]; 16-byte chunk position c of row r holds global chunk
-// c ^ ((r >> 1) & 7): the 16 rows one quarter-wave reads (same logical chunk) then cover all banks, and the
-// swizzle of a fragment row does not depend on the tile it belongs to, so two address registers per operand
-// serve all eight tiles through the instruction's offset field.
+// LDS: two 64 KB operand stages [row][128 B]; 16-byte chunk position c of row r holds global chunk c ^ swz16(r)
+// (bank-conflict free for the fragment reads, see swz16).  The swizzle of a fragment row does not depend on the
+// tile it belongs to, so two address registers per operand serve all eight tiles through the instruction's
+// offset field.
 #include "mi8_gemm_tiles.h"
 
 namespace mi8 {
@@ -43,7 +43,13 @@ constexpr int WT = 128;                      // wave tile edge
 constexpr int NT = WT / 16;                  // MFMA tiles per wave tile edge
 constexpr int kLoads = 8;                    // direct loads per operand, step and wave (8 rows each)
 
-__device__ __forceinline__ int swz16(int r) { return (r >> 1) & 7; }
+// The 16-byte chunk index of row r is XORed with swz16(r).  A fragment read has lane l at row l % 16, chunk
+// 2 (l / 16) + q, i.e. four lanes per 128-byte row.  Which swizzles the LDS of gfx950 serves without bank conflicts
+// was found by timing all 4096 GF(2)-linear maps row -> 3 bits in a loop of ds_read_b128 from four waves: a third
+// of them run at the rate of a contiguous read, this is the one with the fewest terms; (r >> 1) & 7, which
+// would be conflict free if 16 consecutive lanes were served together over 64 banks, measured 28 % slower
+// (SQ_LDS_BANK_CONFLICT: half of the LDS cycles of the GEMM).
+__device__ __forceinline__ int swz16(int r) { return ((r >> 2) & 1) | (((r >> 1) & 1) << 2); }
 
 template <typename Problem, int CBSZ_A, int BLGP_B>
 __global__ __launch_bounds__(kThreads, 1) void gemm_fp8_m16_kernel(Problem pb)
@@ -83,8 +89,8 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_fp8_m16_kernel(Problem pb)
     };
 
     // ---- direct loads: wave w fills rows [64 w + 8 p, +8) of each operand, p = 0..7; lane -> row 64 w + 8 p + lr
-    // (lr = lane / 8), position lane % 8, which holds global chunk (lane % 8) ^ swz16(row); swz16(row) is
-    // 4 (p & 1) + lr / 2.  The load's lane offset is a resident register per operand and parity of p (row lr of
+    // (lr = lane / 8), position lane % 8, which holds global chunk (lane % 8) ^ swz16(row); swz16(row) depends on
+    // lr only.  The load's lane offset is a resident register per operand and parity of p (row lr of
     // the operand plus the chunk) plus a uniform row offset: one vector add next to the load, and few registers
     // (this kernel runs at the 256-register limit, and a reload from scratch waits on the in-order vector memory
     // counter, i.e. on every store and direct load before it).
@@ -93,7 +99,7 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_fp8_m16_kernel(Problem pb)
 #pragma unroll
     for (int k = 0; k < 4; ++k) {
         const int64_t ld = k < 2 ? pb.lda : pb.ldb;
-        dv[k] = (uint32_t)((int64_t)lr * ld) + ((uint32_t)((lane & 7) ^ (((k & 1) << 2) | (lr >> 1))) << 4);
+        dv[k] = (uint32_t)((int64_t)lr * ld) + ((uint32_t)((lane & 7) ^ swz16(8 * (k & 1) + lr)) << 4);
     }
     // x in 0..15: the first eight -> A rows 8 x, the rest -> B rows 8 (x - 8)
     auto dma_one = [&](const uint8_t* a_origin, const uint8_t* b_origin, int stage, int x) __attribute__((always_inline)) {
