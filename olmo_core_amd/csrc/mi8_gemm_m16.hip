@@ -116,19 +116,23 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_fp8_m16_kernel(Problem pb)
     // ---- scales.  Nothing in the epilogue may wait on a global load: such a wait also covers the stores of the
     // previous pass and the operand loads in flight for the next tile (one in-order counter).  Single scales are
     // read here, once; scale vectors travel through LDS like the operands: when the load cursor reaches a tile,
-    // each wave fetches its 64 row and 64 column scales into slot (tile index % 4) with two direct loads, and the
-    // waits and barriers of the K steps in between make them visible before the tile's epilogue.
+    // each wave fetches its 64 row and 64 column scales into the next of four slots with two direct loads, and the
+    // waits and barriers of the K steps in between make them visible before the tile's epilogue.  Slots are
+    // counted over tiles that have K steps (the cursor skips the others, however many): the cursor is at most
+    // two steps, hence two such tiles, ahead of the epilogue that reads a slot.
     float inv_single = 1.0f;
     if constexpr (!Problem::kVecScales) {
         inv_single = (1.0f / pb.single_sa()) * (1.0f / pb.single_sb());
         asm volatile("" ::"v"(inv_single));  // the value is complete before the first direct load is issued
     }
-    auto scale_dma = [&](const TileDesc& d, int tile_idx) __attribute__((always_inline)) {
+    int ld_seq = 0, cp_seq = 0;  // tiles with K steps seen by the load cursor / by the epilogue
+    auto scale_dma = [&](const TileDesc& d) __attribute__((always_inline)) {
         if constexpr (Problem::kVecScales) {
-            uint8_t* slot = lds + 2 * STAGE + OUT_STAGING + (tile_idx & (SCALE_SLOTS - 1)) * SCALE_SLOT + wave * 256;
+            uint8_t* slot = lds + 2 * STAGE + OUT_STAGING + (ld_seq & (SCALE_SLOTS - 1)) * SCALE_SLOT + wave * 256;
             __builtin_amdgcn_global_load_lds((gptr_t)(d.sa + wave * 64 + lane), (lptr_t)slot, 4, 0, 0);
             __builtin_amdgcn_global_load_lds((gptr_t)(d.sb + wave * 64 + lane), (lptr_t)(slot + 1024), 4, 0, 0);
         }
+        ++ld_seq;
     };
 
     // ---- this workgroup's tiles (see mi8_gemm_dma8.hip: XCD-contiguous ranges for tiles of equal cost, plain
@@ -169,7 +173,7 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_fp8_m16_kernel(Problem pb)
                 ld_b = d.b;
                 ld_nk = d.nk;
                 ld_kt = 0;
-                scale_dma(d, ld_tile);
+                scale_dma(d);
                 return;
             }
         }
@@ -288,7 +292,8 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_fp8_m16_kernel(Problem pb)
         uint8_t* stg = lds + 2 * STAGE + wave * 4096;
         const uint32_t stg_lds = (uint32_t)(uintptr_t)(lptr_t)stg;
         const bool zero_tile = td.nk == 0;  // nothing accumulated; the scales may be unset
-        const uint8_t* sc_slot = lds + 2 * STAGE + OUT_STAGING + (cp_tile & (SCALE_SLOTS - 1)) * SCALE_SLOT;
+        const uint8_t* sc_slot = lds + 2 * STAGE + OUT_STAGING + (cp_seq & (SCALE_SLOTS - 1)) * SCALE_SLOT;
+        if (!zero_tile) ++cp_seq;
         const int ldc_bytes = (int)pb.ldc * 2;
         const uint32_t c_lane_off = (uint32_t)((lane >> 3) * ldc_bytes + (lane & 7) * 16);
         __amdgpu_buffer_rsrc_t c_rows;

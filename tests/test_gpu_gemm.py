@@ -119,6 +119,28 @@ def test_bf16_integer_exact_all_variants(dev):
             assert torch.equal(out.float().cpu(), want.bfloat16().float()), ops.gemm_variants()[v]
 
 
+@pytest.mark.parametrize("K", [128, 256, 384])
+def test_many_short_tiles_per_workgroup_exact(dev, K):
+    """More tiles than six per compute unit, one to three K steps each, scale vectors: the persistent kernels
+    switch tiles (operand prefetch, scale hand-over, epilogue) every few steps.  Integer data and power-of-two
+    scales make the expected bf16 output exact."""
+    M, N = 8192, 12288
+    g = torch.Generator().manual_seed(31 + K)
+    a = (torch.randint(0, 2, (M, K), generator=g).float())
+    b = (torch.randint(-1, 2, (N, K), generator=g).float())
+    a[:, K // 2:] = 0  # keeps |sum| below 256 for every K
+    ref = a @ b.t()
+    assert ref.abs().max() < 256
+    sa = (2.0 ** torch.randint(-2, 3, (M,), generator=g).float())
+    sb = (2.0 ** torch.randint(-2, 3, (N,), generator=g).float())
+    want = (ref / sa[:, None] / sb[None, :]).bfloat16()
+    out = ops.gemm_fp8(a.to(E4M3).to(dev), sa.to(dev), b.to(E4M3).to(dev), sb.to(dev))
+    assert torch.equal(out.cpu(), want)
+    one = torch.ones(1, device=dev)
+    out1 = ops.gemm_fp8(a.to(E4M3).to(dev), one, b.to(E4M3).to(dev), one)
+    assert torch.equal(out1.cpu(), ref.bfloat16())
+
+
 def test_scaled_mm_library_crosscheck(dev):
     """Tensorwise case against torch-CPU's own _scaled_mm (library routine)."""
     x = seeded((96, 256), 1)
