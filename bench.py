@@ -27,7 +27,7 @@ FP8_MFMA_PEAK_TFLOPS = 5000.0  # MI355X dense fp8 matrix peak
 GEMMS_PER_STEP = 9
 # HBM-side bytes per GEMM launch (L2 fill reads + writes), mean over the 9 launches of a step, from the
 # FETCH_SIZE / WRITE_SIZE counter runs summarised in profiles/gemm_fp8_m16_kernel__mlp7b_traffic_pmc.txt
-GEMM_TRAFFIC_BYTES_PER_LAUNCH = 1.400e9
+GEMM_TRAFFIC_BYTES_PER_LAUNCH = 1.406e9
 
 
 def build_mlp(dev):
