@@ -251,7 +251,12 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_fp8_m16_kernel(Problem pb)
             }
             // All but this phase's eight loads have landed: the other stage (step + 1) is complete.  (The
             // compiler does not track direct-to-LDS loads across a barrier.)
-            __builtin_amdgcn_s_waitcnt(0x0F78);  // vmcnt(8)
+            // A tile's first step follows the previous tile's epilogue, whose 32 stores are younger than the loads
+            // waited for here (one in-order counter): they may stay outstanding as well.
+            if (fresh)
+                __builtin_amdgcn_s_waitcnt(0x8F78);  // vmcnt(40)
+            else
+                __builtin_amdgcn_s_waitcnt(0x0F78);  // vmcnt(8)
             asm volatile("s_barrier" ::: "memory");
             flip_read_stage(cur ^ 1);
             // phase B, B tile by B tile: the next step's copy of a B tile is read once its four MFMAs are issued;
