@@ -305,6 +305,32 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_fp8_m16_kernel(Problem pb)
         if constexpr (Problem::kMaskRows)
             c_rows = __builtin_amdgcn_make_buffer_rsrc(td.c + (int64_t)td.row_lo * pb.ldc, 0,
                                                        (td.row_hi - td.row_lo) * ldc_bytes, 0x00020000);
+        // The passes are software pipelined: the staged rows of a pass are read back into registers, and go to
+        // memory only after the arithmetic of the next pass, so that each pass exposes one LDS round trip instead
+        // of two.
+        v4i staged[4];  // (an ext-vector type: arrays of HIP's uint4 struct end up in scratch)
+        auto store_staged = [&](int jq, int ih) __attribute__((always_inline)) {
+            const int rt = wm * WT + ih * 32;  // first tile row of the pass
+            if constexpr (Problem::kMaskRows) {
+                // Only rows [row_lo, row_hi) of the tile belong to this tile's group.  The stores go through a
+                // buffer descriptor that spans exactly those rows: a lane whose row lies outside gets an offset
+                // below zero (huge when read as unsigned) or past the end, and the hardware drops its store - no
+                // divergent branches around the stores.
+                const int voff = (rt + (lane >> 3) - td.row_lo) * ldc_bytes + (wn * WT + jq * 64 + (lane & 7) * 8) * 2;
+#pragma unroll
+                for (int it = 0; it < 4; ++it)
+                    __builtin_amdgcn_raw_buffer_store_b128(staged[it], c_rows, voff + it * 8 * ldc_bytes, 0, 0);
+            } else {
+                // uniform 64-bit base + one 32-bit lane offset shared by all passes (no per-pass lane pointers)
+#pragma unroll
+                for (int it = 0; it < 4; ++it) {
+                    uint8_t* base = reinterpret_cast<uint8_t*>(td.c + (int64_t)(rt + it * 8) * pb.ldc + wn * WT + jq * 64);
+                    uint32_t o = c_lane_off;
+                    asm volatile("" : "+v"(o));
+                    *reinterpret_cast<v4i*>(base + o) = staged[it];
+                }
+            }
+        };
 #pragma unroll
         for (int jq = 0; jq < 2; ++jq) {
             float isb[4][4];
@@ -322,6 +348,7 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_fp8_m16_kernel(Problem pb)
 #pragma unroll
             for (int ih = 0; ih < 4; ++ih) {
                 const int rt = wm * WT + ih * 32;  // first tile row of this pass
+                uint2 o[2][4];
 #pragma unroll
                 for (int t = 0; t < 2; ++t) {
                     // A single scale is made opaque in every pass: with a loop-invariant multiplier the compiler
@@ -332,10 +359,8 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_fp8_m16_kernel(Problem pb)
                     else
                         asm volatile("" : "+v"(mult));
                     mult = zero_tile ? 0.0f : mult;
-                    const int row = 16 * t + r16;
 #pragma unroll
                     for (int jj = 0; jj < 4; ++jj) {
-                        const int cw = 16 * jj + 4 * kb;  // column inside the 64-column pass, multiple of 4
                         float v[4];
 #pragma unroll
                         for (int e = 0; e < 4; ++e) {
@@ -347,48 +372,41 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_fp8_m16_kernel(Problem pb)
                             v[e] = a_ * mult;
                             if constexpr (Problem::kVecScales) v[e] *= isb[jj][e];
                         }
-                        uint2 o;
-                        o.x = pack_bf16x2(v[0], v[1]);
-                        o.y = pack_bf16x2(v[2], v[3]);
+                        o[t][jj].x = pack_bf16x2(v[0], v[1]);
+                        o[t][jj].y = pack_bf16x2(v[2], v[3]);
+                    }
+                }
+                asm volatile("" ::: "memory");  // the stores below stay behind the arithmetic above
+                if (jq + ih > 0) {
+                    // the previous pass's rows have arrived in registers (so its staging area is free again)
+                    __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0)
+                    store_staged(ih == 0 ? jq - 1 : jq, ih == 0 ? 3 : ih - 1);
+                }
+#pragma unroll
+                for (int t = 0; t < 2; ++t)
+#pragma unroll
+                    for (int jj = 0; jj < 4; ++jj) {
+                        const int row = 16 * t + r16;
+                        const int cw = 16 * jj + 4 * kb;  // column inside the 64-column pass, multiple of 4
                         const int chunk = (cw >> 3) ^ ((row >> 1) & 7);
                         // Written as an instruction of its own: before an LDS store it knows of, the compiler
                         // waits for every direct-to-LDS load in flight (it cannot tell that they target other
                         // addresses), i.e. for the operand loads already issued for the next tile.
                         const uint32_t saddr = stg_lds + (uint32_t)(row * 128 + chunk * 16 + (cw & 4) * 2);
-                        asm volatile("ds_write_b64 %0, %1" ::"v"(saddr), "v"(o) : "memory");
+                        asm volatile("ds_write_b64 %0, %1" ::"v"(saddr), "v"(o[t][jj]) : "memory");
                     }
-                }
                 __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): the wave's own LDS writes have landed
                 __builtin_amdgcn_wave_barrier();
-                v4i staged[4];  // (an ext-vector type: arrays of HIP's uint4 struct end up in scratch)
 #pragma unroll
                 for (int it = 0; it < 4; ++it) {
                     const int rw = it * 8 + (lane >> 3);
                     staged[it] = *reinterpret_cast<const v4i*>(stg + rw * 128 + (((lane & 7) ^ ((rw >> 1) & 7)) << 4));
                 }
-                if constexpr (Problem::kMaskRows) {
-                    // Only rows [row_lo, row_hi) of the tile belong to this tile's group.  The stores go through a
-                    // buffer descriptor that spans exactly those rows: a lane whose row lies outside gets an
-                    // offset below zero (huge when read as unsigned) or past the end, and the hardware drops its
-                    // store - no divergent branches around the stores.
-                    const int voff = (rt + (lane >> 3) - td.row_lo) * ldc_bytes + (wn * WT + jq * 64 + (lane & 7) * 8) * 2;
-#pragma unroll
-                    for (int it = 0; it < 4; ++it)
-                        __builtin_amdgcn_raw_buffer_store_b128(staged[it], c_rows, voff + it * 8 * ldc_bytes, 0, 0);
-                } else {
-                    // uniform 64-bit base + one 32-bit lane offset shared by all passes (no per-pass lane pointers)
-#pragma unroll
-                    for (int it = 0; it < 4; ++it) {
-                        uint8_t* base = reinterpret_cast<uint8_t*>(td.c + (int64_t)(rt + it * 8) * pb.ldc + wn * WT + jq * 64);
-                        uint32_t o = c_lane_off;
-                        asm volatile("" : "+v"(o));
-                        *reinterpret_cast<v4i*>(base + o) = staged[it];
-                    }
-                }
-                __builtin_amdgcn_s_waitcnt(0xc07f);  // the reads are done before the next pass overwrites
-                __builtin_amdgcn_wave_barrier();
+                asm volatile("" ::: "memory");
             }
         }
+        __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0)
+        store_staged(1, 3);
         // The last step's phase B has read the next tile's first fragments like any other step; reading them
         // again here makes those 96 registers free during the epilogue, which otherwise spills (and every
         // reload from scratch waits on the in-order vector memory counter, i.e. on the stores above).
