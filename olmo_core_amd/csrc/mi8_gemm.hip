@@ -120,7 +120,7 @@ extern "C" int mi8_gemm_fp8(const void* a, int a_dtype, int64_t lda, const void*
                         out_dtype == MI8_BF16 && (!sb_is_vector || aligned16(sb)) &&
                         (sa_is_vector != 0) == (sb_is_vector != 0);
     // measured on MI355X on the benchmark configurations' shapes: the four-wave layout beats the eight-wave one
-    // by 0-14 %, and its 16x16x128 form beats its 32x32x64 form by 1-6 % (random operands, power-limited clocks)
+    // by 0-14 %, and its 16x16x128 form beats its 32x32x64 form by 3-9 % (random operands, power-limited clocks)
     if (variant < 0) variant = dma_ok ? (K % 128 == 0 ? kM16 : kDma) : 1;
     if (variant == kDma8 && dma_ok && K % 128 == 0) return launch_dma8(g, a_dtype, b_dtype, st);
     if (variant == kDma4 && dma_ok && K % 128 == 0) return launch_dma4(g, a_dtype, b_dtype, st);

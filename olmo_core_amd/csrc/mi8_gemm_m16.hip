@@ -2,19 +2,20 @@
 // global->LDS loads of full 128-byte rows.  Same problems, tile order and LDS budget as the 32x32x64 kernel
 // (mi8_gemm_dma8.hip); for full 256 x 256 tiles, K % 128 == 0, bf16 output.
 //
-// Why this MFMA shape: an MI355X running fp8 MFMAs on random operands is power limited (it clocks down to about
-// 1.7 GHz), so throughput follows energy per flop, and v_mfma_f32_16x16x128_f8f6f4 needs less of it than
+// Why this MFMA shape: an MI355X running fp8 MFMAs on random operands is power limited (it clocks down to
+// 1.7-1.9 GHz), so throughput follows energy per flop, and v_mfma_f32_16x16x128_f8f6f4 needs less of it than
 // v_mfma_f32_32x32x64_f8f6f4: back-to-back MFMAs on random bytes, nothing else running, measured 4.35 PFLOP/s
 // against 4.0 PFLOP/s (both 4.97 PFLOP/s on all-zero operands, where the clock stays up).
 //
 // A 128-byte K step of a wave is 8 x 8 MFMAs (A tile i: 16 rows, B tile j: 16 columns, 4 accumulator registers
 // each: 256 in all).  The step is split along M so that only half of the A fragments are double buffered:
 //
-//     phase A   32 x { MFMA (A tiles 0-3) x (B tiles 0-7) }; LDS reads of A tiles 4-7 of this step
-//     wait for this wave's loads of step s+1, barrier
+//     barrier (every wave has issued its LDS reads of the previous phase B)
+//     phase A   32 x { MFMA (A tiles 0-3) x (B tiles 0-7) }; LDS reads of A tiles 4-7 of this step; 8 direct loads:
+//               the B rows of step s+2 into the stage of step s, whose B rows are no longer needed
+//     wait for this wave's loads of step s+1 (all but the eight just issued), barrier
 //     phase B   32 x { MFMA (A tiles 4-7) x (B tiles 0-7), B tile by B tile }; LDS reads of step s+1: A tiles 0-3
-//               and each B tile as soon as its four MFMAs are issued; 16 direct loads of step s+2 into the
-//               stage step s has vacated
+//               and each B tile as soon as its four MFMAs are issued; 8 direct loads: the A rows of step s+2
 //
 // Fragment registers: 32 (A 0-3) + 32 (A 4-7) + 64 (B) = 128.
 //
