@@ -48,6 +48,7 @@ typedef enum mi8_hp {
 /* flags shared by the cast entry points */
 #define MI8_FLAG_POW2_SCALE 1u /* round every scale down to a power of two (ao.py:167 round_scales_to_power_of_2) */
 #define MI8_FLAG_SW_CVT 2u     /* convert with integer arithmetic instead of v_cvt_pk_{fp8,bf8}_f32 (same bytes) */
+#define MI8_FLAG_AMAX_READY 4u /* grouped casts: the amax workspaces already hold the amax of x (see mi8_grouped_swiglu_*) */
 
 /* Number of uint32 slots a tensorwise amax workspace must have. */
 #define MI8_AMAX_SLOTS 2048
@@ -170,6 +171,18 @@ int mi8_grouped_cast_rows_and_colwise_t(const void* x, int hp_dtype, int64_t T, 
                                         uint32_t* amax_ws, void* out_t, int64_t ld_t, float* scale_out,
                                         uint32_t* row_amax_ws, void* out_rows, int64_t ld_rows, float* row_scale_out,
                                         void* stream);
+
+/* h = silu(x1) * x2 of the expert layer (src/olmo_core/nn/moe/mlp.py:286-291; bf16 [T, cols], the rounding points
+ * of mi8_swiglu_fwd) together with the amax pass of the cast that follows: amax_ws (uint32 [num_groups * cols]) and
+ * row_amax_ws (uint32 [T]), both ZERO on entry, receive the per-(group, column) and per-row amax of h, so that
+ * mi8_grouped_cast_rows_and_colwise_t(h, ..., flags | MI8_FLAG_AMAX_READY, ...) skips its own first pass.  Rows
+ * beyond the last group are not written.  The backward form writes the gradients g1 (of x1) and g2 (of x2) of that
+ * product for the incoming gradient gh, each with its own pair of amax workspaces. */
+int mi8_grouped_swiglu_fwd(const void* x1, const void* x2, int64_t T, int64_t cols, const int64_t* group_sizes,
+                           int32_t num_groups, void* h, uint32_t* amax_ws, uint32_t* row_amax_ws, void* stream);
+int mi8_grouped_swiglu_bwd(const void* x1, const void* x2, const void* gh, int64_t T, int64_t cols,
+                           const int64_t* group_sizes, int32_t num_groups, void* g1, void* g2, uint32_t* amax_ws1,
+                           uint32_t* row_amax_ws1, uint32_t* amax_ws2, uint32_t* row_amax_ws2, void* stream);
 
 /* out[R_e, :N] = (A[R_e, :K] . B_e[:N, :K]^T) / sa[r] / sb_e[n]   for every group e.
  *   A fp8 [T, lda]; B_e = b + e * b_group_stride (bytes), N rows of pitch ldb; sa float32 [T];

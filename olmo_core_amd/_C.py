@@ -23,6 +23,7 @@ MI8_E4M3, MI8_E5M2 = 0, 1
 MI8_BF16, MI8_F32, MI8_F16, MI8_RAW8 = 0, 1, 2, 3
 FLAG_POW2_SCALE = 1
 FLAG_SW_CVT = 2
+FLAG_AMAX_READY = 4
 AMAX_SLOTS = 2048
 
 # name -> (restype, argtypes); mirrors include/mi8.h one to one
@@ -93,6 +94,15 @@ _SIGNATURES = {
         c_int,
         [c_void_p, c_int, c_int64, c_int64, c_void_p, c_int32, c_int, c_uint32, c_void_p, c_void_p, c_int64, c_void_p,
          c_void_p],
+    ),
+    "mi8_grouped_swiglu_fwd": (
+        c_int,
+        [c_void_p, c_void_p, c_int64, c_int64, c_void_p, c_int32, c_void_p, c_void_p, c_void_p, c_void_p],
+    ),
+    "mi8_grouped_swiglu_bwd": (
+        c_int,
+        [c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_void_p, c_int32, c_void_p, c_void_p, c_void_p, c_void_p,
+         c_void_p, c_void_p, c_void_p],
     ),
     "mi8_grouped_cast_rows_and_colwise_t": (
         c_int,

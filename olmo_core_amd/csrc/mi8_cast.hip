@@ -1,7 +1,7 @@
 // amax reductions and saturating float8 casts (tensorwise, per-row, per-column with transposed output).
 // All kernels are HBM-bound streaming kernels: 16-byte loads per lane, wave-shuffle reductions, an
 // LDS-staged byte transpose for the transposed copy.
-#include "mi8_common.h"
+#include "mi8_swiglu.h"
 
 namespace mi8 {
 namespace {
@@ -491,6 +491,95 @@ __global__ void row_scales_kernel(const uint32_t* __restrict__ row_amax, int64_t
     if (r < T) row_scale[r] = scale_from_amax_bits<FP8>(row_amax[r], pow2);
 }
 
+// SwiGLU of the dropless-MoE expert layer with the first pass of the two-product cast fused in: the kernel
+// writes h = silu(x1) * x2 (or, backward, the gradients g1, g2 of it) in bf16 and takes, of what it writes, the
+// amax per (group, column) and per row, exactly what grouped_colamax_kernel would compute in a pass of its own.
+struct GroupedSwigluArgs {
+    const uint4* x1;
+    const uint4* x2;
+    const uint4* gh;  // backward only
+    uint4* o1;        // forward: h; backward: g1
+    uint4* o2;        // backward: g2
+    int64_t T, cols;
+    const int64_t* sizes;
+    int E;
+    uint32_t* col_amax1;  // [E, cols], zero on entry
+    uint32_t* row_amax1;  // [T], zero on entry
+    uint32_t* col_amax2;  // backward only
+    uint32_t* row_amax2;
+};
+
+template <bool BWD>
+__global__ __launch_bounds__(kThreads) void grouped_swiglu_kernel(GroupedSwigluArgs a)
+{
+    constexpr int NO = BWD ? 2 : 1;
+    __shared__ uint32_t red[NO][16][kTile + 1];
+    int e;
+    int64_t row0, row_end;
+    if (!locate_padded_tile(a.sizes, a.E, a.T, (int)blockIdx.y, e, row0, row_end)) return;
+    const int tid = threadIdx.x;
+    const int cl = tid & 15, rg = tid >> 4;
+    const int64_t col0 = (int64_t)blockIdx.x * kTile;
+    const int64_t c8 = col0 + 8 * cl;
+    uint32_t acc[NO][4];
+#pragma unroll
+    for (int o = 0; o < NO; ++o)
+#pragma unroll
+        for (int k = 0; k < 4; ++k) acc[o][k] = 0;
+    uint32_t* const row_amax[2] = {a.row_amax1, a.row_amax2};
+    uint32_t* const col_amax[2] = {a.col_amax1, a.col_amax2};
+#pragma unroll
+    for (int i = 0; i < kTile / 16; ++i) {
+        const int64_t r = row0 + rg + 16 * i;
+        uint32_t rowacc[NO][4];
+#pragma unroll
+        for (int o = 0; o < NO; ++o)
+#pragma unroll
+            for (int k = 0; k < 4; ++k) rowacc[o][k] = 0;
+        if (c8 < a.cols && r < row_end) {
+            const int64_t v = (r * a.cols + c8) >> 3;
+            uint4 out[2];
+            if constexpr (BWD) {
+                swiglu_bwd8(a.x1[v], a.x2[v], a.gh[v], out[0], out[1]);
+                a.o1[v] = out[0];
+                a.o2[v] = out[1];
+            } else {
+                out[0] = swiglu_fwd8(a.x1[v], a.x2[v]);
+                a.o1[v] = out[0];
+            }
+#pragma unroll
+            for (int o = 0; o < NO; ++o) {
+                absmax_accumulate<MI8_BF16>(out[o], acc[o]);
+                absmax_accumulate<MI8_BF16>(out[o], rowacc[o]);
+            }
+        }
+#pragma unroll
+        for (int o = 0; o < NO; ++o) {  // the 16 lanes that share this row fold their eight columns each
+            uint32_t m = absmax_fold<MI8_BF16>(rowacc[o]);
+#pragma unroll
+            for (int off = 8; off > 0; off >>= 1) m = umax32(m, (uint32_t)__shfl_xor((int)m, off, 16));
+            if (cl == 0 && r < row_end && m) atomicMax(&row_amax[o][r], m);
+        }
+    }
+#pragma unroll
+    for (int o = 0; o < NO; ++o)
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            red[o][rg][8 * cl + 2 * k] = (acc[o][k] & 0xFFFFu) << 16;
+            red[o][rg][8 * cl + 2 * k + 1] = acc[o][k] & 0xFFFF0000u;
+        }
+    __syncthreads();
+    if (tid < kTile && col0 + tid < a.cols) {
+#pragma unroll
+        for (int o = 0; o < NO; ++o) {
+            uint32_t m = 0;
+#pragma unroll
+            for (int k = 0; k < 16; ++k) m = umax32(m, red[o][k][tid]);
+            atomicMax(&col_amax[o][(int64_t)e * a.cols + col0 + tid], m);
+        }
+    }
+}
+
 template <int HP, int FP8, bool SW>
 __global__ __launch_bounds__(kThreads) void grouped_tile_cast_kernel(GroupedCastArgs a)
 {
@@ -839,12 +928,15 @@ int grouped_cast_launch(const char* what, const void* x, int hp_dtype, int64_t T
                       out_rows ? row_amax_ws : nullptr, (uint8_t*)out_rows, ld_rows, row_scale_out};
     hipStream_t st = (hipStream_t)stream;
     dim3 grid((unsigned)ceil_div(cols, kTile), (unsigned)ptiles);
-    if (hp_dtype == MI8_BF16)
-        hipLaunchKernelGGL((grouped_colamax_kernel<MI8_BF16>), grid, dim3(kThreads), 0, st, a);
-    else
-        hipLaunchKernelGGL((grouped_colamax_kernel<MI8_F32>), grid, dim3(kThreads), 0, st, a);
-    int rc = launch_status(what);
-    if (rc != MI8_OK) return rc;
+    int rc = MI8_OK;
+    if (!(flags & MI8_FLAG_AMAX_READY)) {  // otherwise the workspaces already hold the amax of x
+        if (hp_dtype == MI8_BF16)
+            hipLaunchKernelGGL((grouped_colamax_kernel<MI8_BF16>), grid, dim3(kThreads), 0, st, a);
+        else
+            hipLaunchKernelGGL((grouped_colamax_kernel<MI8_F32>), grid, dim3(kThreads), 0, st, a);
+        rc = launch_status(what);
+        if (rc != MI8_OK) return rc;
+    }
     if (out_rows) {
         const dim3 rg((unsigned)ceil_div(T, 256));
         if (fp8_dtype == MI8_E4M3)
@@ -889,4 +981,46 @@ extern "C" int mi8_grouped_cast_rows_and_colwise_t(const void* x, int hp_dtype, 
     return grouped_cast_launch("mi8_grouped_cast_rows_and_colwise_t", x, hp_dtype, T, cols, group_sizes, num_groups,
                                fp8_dtype, flags, amax_ws, out_t, ld_t, scale_out, row_amax_ws, out_rows, ld_rows,
                                row_scale_out, stream);
+}
+
+namespace mi8 {
+namespace {
+
+int grouped_swiglu_launch(const char* what, const GroupedSwigluArgs& a, bool bwd, void* stream)
+{
+    MI8_REQUIRE(a.x1 && a.x2 && a.o1 && a.sizes && a.col_amax1 && a.row_amax1, MI8_ERR_ARG, "%s: null pointer", what);
+    if (bwd) MI8_REQUIRE(a.gh && a.o2 && a.col_amax2 && a.row_amax2, MI8_ERR_ARG, "%s: null pointer", what);
+    MI8_REQUIRE(a.T > 0 && a.cols > 0 && a.E > 0, MI8_ERR_ARG, "%s: empty input", what);
+    MI8_REQUIRE(a.cols % 16 == 0, MI8_ERR_UNSUPPORTED, "%s: cols (%lld) must be a multiple of 16", what, (long long)a.cols);
+    MI8_REQUIRE(aligned16(a.x1) && aligned16(a.x2) && aligned16(a.gh) && aligned16(a.o1) && aligned16(a.o2),
+                MI8_ERR_UNSUPPORTED, "%s: pointers must be 16-byte aligned", what);
+    const int64_t ptiles = ceil_div(a.T, kTile) + a.E;
+    MI8_REQUIRE(ptiles <= 65535, MI8_ERR_UNSUPPORTED, "%s: too many row tiles (%lld)", what, (long long)ptiles);
+    dim3 grid((unsigned)ceil_div(a.cols, kTile), (unsigned)ptiles);
+    if (bwd)
+        hipLaunchKernelGGL((grouped_swiglu_kernel<true>), grid, dim3(kThreads), 0, (hipStream_t)stream, a);
+    else
+        hipLaunchKernelGGL((grouped_swiglu_kernel<false>), grid, dim3(kThreads), 0, (hipStream_t)stream, a);
+    return launch_status(what);
+}
+
+}  // namespace
+}  // namespace mi8
+
+extern "C" int mi8_grouped_swiglu_fwd(const void* x1, const void* x2, int64_t T, int64_t cols, const int64_t* group_sizes,
+                                      int32_t num_groups, void* h, uint32_t* amax_ws, uint32_t* row_amax_ws, void* stream)
+{
+    GroupedSwigluArgs a{(const uint4*)x1, (const uint4*)x2, nullptr, (uint4*)h, nullptr, T, cols, group_sizes, num_groups,
+                        amax_ws, row_amax_ws, nullptr, nullptr};
+    return grouped_swiglu_launch("mi8_grouped_swiglu_fwd", a, false, stream);
+}
+
+extern "C" int mi8_grouped_swiglu_bwd(const void* x1, const void* x2, const void* gh, int64_t T, int64_t cols,
+                                      const int64_t* group_sizes, int32_t num_groups, void* g1, void* g2,
+                                      uint32_t* amax_ws1, uint32_t* row_amax_ws1, uint32_t* amax_ws2,
+                                      uint32_t* row_amax_ws2, void* stream)
+{
+    GroupedSwigluArgs a{(const uint4*)x1, (const uint4*)x2, (const uint4*)gh, (uint4*)g1, (uint4*)g2, T, cols, group_sizes,
+                        num_groups, amax_ws1, row_amax_ws1, amax_ws2, row_amax_ws2};
+    return grouped_swiglu_launch("mi8_grouped_swiglu_bwd", a, true, stream);
 }

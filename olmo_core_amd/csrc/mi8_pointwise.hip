@@ -2,43 +2,12 @@
 // that the tensorwise cast that follows needs no separate pass over the (largest) activation tensor.
 // Rounding points follow torch's eager bf16 evaluation: every elementwise op computes in fp32 and rounds
 // its result to bf16 before the next op reads it.
-#include "mi8_common.h"
+#include "mi8_swiglu.h"
 
 namespace mi8 {
 namespace {
 
 constexpr int kThreads = 256;
-
-__device__ __forceinline__ float bf16_round(float f)
-{
-    __bf16 h = (__bf16)f;
-    return (float)h;
-}
-
-__device__ __forceinline__ uint32_t pack_bf16(float lo, float hi)
-{
-    __bf16 a = (__bf16)lo, b = (__bf16)hi;
-    return (uint32_t)__builtin_bit_cast(uint16_t, a) | ((uint32_t)__builtin_bit_cast(uint16_t, b) << 16);
-}
-
-__device__ __forceinline__ float sigmoid_f32(float x) { return 1.0f / (1.0f + expf(-x)); }
-
-__device__ __forceinline__ void unpack8(uint4 v, float (&f)[8])
-{
-    f[0] = bits_to_f32(v.x << 16);
-    f[1] = bits_to_f32(v.x & 0xFFFF0000u);
-    f[2] = bits_to_f32(v.y << 16);
-    f[3] = bits_to_f32(v.y & 0xFFFF0000u);
-    f[4] = bits_to_f32(v.z << 16);
-    f[5] = bits_to_f32(v.z & 0xFFFF0000u);
-    f[6] = bits_to_f32(v.w << 16);
-    f[7] = bits_to_f32(v.w & 0xFFFF0000u);
-}
-
-__device__ __forceinline__ uint4 pack8(const float (&f)[8])
-{
-    return make_uint4(pack_bf16(f[0], f[1]), pack_bf16(f[2], f[3]), pack_bf16(f[4], f[5]), pack_bf16(f[6], f[7]));
-}
 
 // max over |bf16| of the 8 packed values, as a float32 bit pattern
 __device__ __forceinline__ uint32_t absmax_packed(uint4 v)
@@ -69,15 +38,7 @@ __global__ __launch_bounds__(kThreads) void swiglu_fwd_kernel(const uint4* __res
     uint32_t m = 0;
     const int64_t stride = (int64_t)gridDim.x * kThreads;
     for (int64_t i = (int64_t)blockIdx.x * kThreads + threadIdx.x; i < nvec; i += stride) {
-        float a[8], b[8], o[8];
-        unpack8(x1[i], a);
-        unpack8(x3[i], b);
-#pragma unroll
-        for (int k = 0; k < 8; ++k) {
-            const float s = bf16_round(a[k] * sigmoid_f32(a[k]));  // silu output as a bf16 tensor
-            o[k] = s * b[k];
-        }
-        const uint4 out = pack8(o);
+        const uint4 out = swiglu_fwd8(x1[i], x3[i]);
         h[i] = out;
         m = umax32(m, absmax_packed(out));
     }
@@ -94,19 +55,8 @@ __global__ __launch_bounds__(kThreads) void swiglu_bwd_kernel(const uint4* __res
     uint32_t m1 = 0, m3 = 0;
     const int64_t stride = (int64_t)gridDim.x * kThreads;
     for (int64_t i = (int64_t)blockIdx.x * kThreads + threadIdx.x; i < nvec; i += stride) {
-        float a[8], b[8], g[8], o1[8], o3[8];
-        unpack8(x1[i], a);
-        unpack8(x3[i], b);
-        unpack8(gh[i], g);
-#pragma unroll
-        for (int k = 0; k < 8; ++k) {
-            const float sig = sigmoid_f32(a[k]);
-            const float s = bf16_round(a[k] * sig);   // saved silu output
-            o3[k] = g[k] * s;                         // d/dx3
-            const float gs = bf16_round(g[k] * b[k]); // gradient reaching silu's output
-            o1[k] = gs * (sig * (1.0f + a[k] * (1.0f - sig)));
-        }
-        const uint4 p1 = pack8(o1), p3 = pack8(o3);
+        uint4 p1, p3;
+        swiglu_bwd8(x1[i], x3[i], gh[i], p1, p3);
         g1[i] = p1;
         g3[i] = p3;
         m1 = umax32(m1, absmax_packed(p1));

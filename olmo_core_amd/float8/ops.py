@@ -331,13 +331,62 @@ def grouped_cast_colwise_t(
     return q_t, scale
 
 
+def _grouped_amax_workspace(T: int, cols: int, E: int, device) -> torch.Tensor:
+    """Zeroed ``uint32[E * cols + T]``: the per-(group, column) amax table followed by the per-row one."""
+    return torch.zeros(E * cols + T, dtype=torch.int32, device=device)
+
+
+def grouped_swiglu_fwd(x1: torch.Tensor, x2: torch.Tensor, group_sizes: torch.Tensor):
+    """``h = silu(x1) * x2`` (bf16, ``[T, cols]``, rows grouped by ``group_sizes``) plus the amax workspace of ``h``
+    that :func:`grouped_cast_rows_and_colwise_t` takes as ``amax``: the cast then needs one pass instead of two."""
+    _require_gpu(x1, "grouped_swiglu_fwd")
+    if x1.dtype != torch.bfloat16 or x2.dtype != torch.bfloat16 or x1.shape != x2.shape or x1.dim() != 2:
+        raise ValueError("grouped_swiglu_fwd expects two bfloat16 matrices of one shape")
+    x1, x2 = x1.contiguous(), x2.contiguous()
+    T, cols = x1.shape
+    sizes = _sizes_i64(group_sizes, x1.device)
+    E = sizes.numel()
+    h = torch.empty_like(x1)
+    ws = _grouped_amax_workspace(T, cols, E, x1.device)
+    _C.check(
+        _C.lib().mi8_grouped_swiglu_fwd(x1.data_ptr(), x2.data_ptr(), T, cols, sizes.data_ptr(), E, h.data_ptr(),
+                                        ws.data_ptr(), ws.data_ptr() + 4 * E * cols, _stream(x1)),
+        "mi8_grouped_swiglu_fwd",
+    )
+    return h, ws
+
+
+def grouped_swiglu_bwd(x1: torch.Tensor, x2: torch.Tensor, gh: torch.Tensor, group_sizes: torch.Tensor):
+    """Gradients ``(g1, g2)`` of ``silu(x1) * x2`` for the incoming ``gh`` plus one amax workspace each (see
+    :func:`grouped_swiglu_fwd`)."""
+    _require_gpu(x1, "grouped_swiglu_bwd")
+    if not (x1.dtype == x2.dtype == gh.dtype == torch.bfloat16) or not (x1.shape == x2.shape == gh.shape) or x1.dim() != 2:
+        raise ValueError("grouped_swiglu_bwd expects three bfloat16 matrices of one shape")
+    x1, x2, gh = x1.contiguous(), x2.contiguous(), gh.contiguous()
+    T, cols = x1.shape
+    sizes = _sizes_i64(group_sizes, x1.device)
+    E = sizes.numel()
+    g1, g2 = torch.empty_like(x1), torch.empty_like(x1)
+    ws1 = _grouped_amax_workspace(T, cols, E, x1.device)
+    ws2 = _grouped_amax_workspace(T, cols, E, x1.device)
+    _C.check(
+        _C.lib().mi8_grouped_swiglu_bwd(x1.data_ptr(), x2.data_ptr(), gh.data_ptr(), T, cols, sizes.data_ptr(), E,
+                                        g1.data_ptr(), g2.data_ptr(), ws1.data_ptr(), ws1.data_ptr() + 4 * E * cols,
+                                        ws2.data_ptr(), ws2.data_ptr() + 4 * E * cols, _stream(x1)),
+        "mi8_grouped_swiglu_bwd",
+    )
+    return g1, g2, ws1, ws2
+
+
 def grouped_cast_rows_and_colwise_t(
-    x: torch.Tensor, group_sizes: torch.Tensor, fp8_dtype: torch.dtype, *, pow2: bool = False
+    x: torch.Tensor, group_sizes: torch.Tensor, fp8_dtype: torch.dtype, *, pow2: bool = False,
+    amax: Optional[torch.Tensor] = None,
 ) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]:
     """
     :func:`cast_rowwise` and :func:`grouped_cast_colwise_t` of the same tensor in one pair of passes:
     ``(q [T, cols], row_scale [T], q_t [cols, ld_t], col_scale [E, cols])``.  The group sizes must sum to ``T``
-    (rows after the last group are left unwritten).
+    (rows after the last group are left unwritten).  ``amax``: the workspace returned with ``x`` by
+    :func:`grouped_swiglu_fwd` / :func:`grouped_swiglu_bwd`; the amax pass is then skipped.
     """
     x = _hp2d(x, "grouped_cast_rows_and_colwise_t")
     T, cols = x.shape
@@ -348,10 +397,17 @@ def grouped_cast_rows_and_colwise_t(
     scale = torch.empty((E, cols), dtype=torch.float32, device=x.device)
     q = torch.empty((T, cols), dtype=fp8_dtype, device=x.device)
     row_scale = torch.empty(T, dtype=torch.float32, device=x.device)
-    ws = torch.zeros(E * cols + T, dtype=torch.int32, device=x.device)
+    flags = _flags(pow2)
+    if amax is None:
+        ws = _grouped_amax_workspace(T, cols, E, x.device)
+    else:
+        if amax.numel() != E * cols + T or amax.dtype != torch.int32 or amax.device != x.device:
+            raise ValueError("amax must be the workspace returned by grouped_swiglu_fwd/bwd for this tensor")
+        ws = amax
+        flags |= _C.FLAG_AMAX_READY
     _C.check(
         _C.lib().mi8_grouped_cast_rows_and_colwise_t(
-            x.data_ptr(), _HP_CODE[x.dtype], T, cols, sizes.data_ptr(), E, _FP8_CODE[fp8_dtype], _flags(pow2),
+            x.data_ptr(), _HP_CODE[x.dtype], T, cols, sizes.data_ptr(), E, _FP8_CODE[fp8_dtype], flags,
             ws.data_ptr(), q_t.data_ptr(), ld_t, scale.data_ptr(), ws.data_ptr() + 4 * E * cols, q.data_ptr(), cols,
             row_scale.data_ptr(), _stream(x),
         ),

@@ -53,10 +53,12 @@ class _Float8DroplessMLP(torch.autograd.Function):
             w3q, s3 = ops.cast_rowwise(w3, _E4M3, pow2=pow2)
         x1 = ops.grouped_gemm_fp8(xq, sx, w1q, s1, sizes, n=H, k=D, b_group_stride=H * w1q.stride(0), sb_group_stride=H)
         x2 = ops.grouped_gemm_fp8(xq, sx, w3q, s3, sizes, n=H, k=D, b_group_stride=H * w3q.stride(0), sb_group_stride=H)
-        h, _ = ops.swiglu_fwd(x1, x2, want_amax=False)
         if need[2]:
-            hq, sh, ht, shc = ops.grouped_cast_rows_and_colwise_t(h, sizes, _E4M3, pow2=pow2)
+            # the pointwise kernel also takes the amax of h per row and per (expert, column): the cast is one pass
+            h, h_amax = ops.grouped_swiglu_fwd(x1, x2, sizes)
+            hq, sh, ht, shc = ops.grouped_cast_rows_and_colwise_t(h, sizes, _E4M3, pow2=pow2, amax=h_amax)
         else:
+            h, _ = ops.swiglu_fwd(x1, x2, want_amax=False)
             hq, sh = ops.cast_rowwise(h, _E4M3, pow2=pow2)
         del h
         # w2[e] is [H, D] and is used as-is (h_e @ w2[e]): its output channel is the column -> transposed copy
@@ -95,20 +97,25 @@ class _Float8DroplessMLP(torch.autograd.Function):
             # gh_e = gy_e @ w2[e]^T : contraction over D, the right operand is w2[e] itself, one scale per row
             gh = ops.grouped_gemm_fp8(gyq, sgy, w2q, s2r, sizes, n=H, k=D, b_group_stride=H * w2q.stride(0),
                                       sb_group_stride=H)
-            g1, g2, _, _ = ops.swiglu_bwd(x1, x2, gh, want_amax=False)
+            fused_amax = need_x and (need_w1 or need_w3)
+            if fused_amax:
+                g1, g2, amax1, amax2 = ops.grouped_swiglu_bwd(x1, x2, gh, sizes)
+            else:
+                g1, g2, _, _ = ops.swiglu_bwd(x1, x2, gh, want_amax=False)
+                amax1 = amax2 = None
             del gh
 
-            def both(g, want_rows, want_cols):
+            def both(g, want_rows, want_cols, amax):
                 if want_rows and want_cols:
-                    return ops.grouped_cast_rows_and_colwise_t(g, sizes, _E4M3, pow2=pow2)
+                    return ops.grouped_cast_rows_and_colwise_t(g, sizes, _E4M3, pow2=pow2, amax=amax)
                 if want_rows:
                     return (*ops.cast_rowwise(g, _E4M3, pow2=pow2), None, None)
                 if want_cols:
                     return (None, None, *ops.grouped_cast_colwise_t(g, sizes, _E4M3, pow2=pow2))
                 return None, None, None, None
 
-            g1q, sg1, g1t, sg1c = both(g1, need_x, need_w1)
-            g2q, sg2, g2t, sg2c = both(g2, need_x, need_w3)
+            g1q, sg1, g1t, sg1c = both(g1, need_x, need_w1, amax1)
+            g2q, sg2, g2t, sg2c = both(g2, need_x, need_w3, amax2)
             del g1, g2
             if need_x:
                 # gx_e = g_e @ w[e] : contraction over H, the right operand is w[e]^T [D, H], one scale per input channel

@@ -77,6 +77,35 @@ def test_rows_and_grouped_colwise_cast_bit_exact(dev, sizes, pow2):
 
 
 @pytest.mark.parametrize("sizes", SIZE_CASES, ids=lambda s: "-".join(map(str, s)))
+def test_grouped_swiglu_with_amax_matches_separate_kernels(dev, sizes):
+    """The group-aware SwiGLU kernels write the bytes of the flat ones, and the cast that takes their amax
+    workspace gives the bytes and scales of the cast that computes the amax itself (forward and backward)."""
+    T, C = sum(sizes), 272
+    x1, x2, gh = (seeded((T, C), s, std=1.0).to(dev) for s in (21, 22, 23))
+    sz = torch.tensor(sizes)
+    h_ref, _ = ops.swiglu_fwd(x1, x2, want_amax=False)
+    h, ws = ops.grouped_swiglu_fwd(x1, x2, sz)
+    assert torch.equal(h.view(torch.int16), h_ref.view(torch.int16))
+    want = ops.grouped_cast_rows_and_colwise_t(h_ref, sz, E4M3, pow2=True)
+    got = ops.grouped_cast_rows_and_colwise_t(h, sz, E4M3, pow2=True, amax=ws)
+    g1_ref, g2_ref, _, _ = ops.swiglu_bwd(x1, x2, gh, want_amax=False)
+    g1, g2, ws1, ws2 = ops.grouped_swiglu_bwd(x1, x2, gh, sz)
+    assert torch.equal(g1.view(torch.int16), g1_ref.view(torch.int16))
+    assert torch.equal(g2.view(torch.int16), g2_ref.view(torch.int16))
+    pairs = [(want, got)]
+    for g_ref, g, w in ((g1_ref, g1, ws1), (g2_ref, g2, ws2)):
+        pairs.append((ops.grouped_cast_rows_and_colwise_t(g_ref, sz, E4M3, pow2=True),
+                      ops.grouped_cast_rows_and_colwise_t(g, sz, E4M3, pow2=True, amax=w)))
+    for want, got in pairs:
+        (q, rs, q_t, cs), (q2, rs2, q_t2, cs2) = want, got
+        assert torch.equal(u8(q), u8(q2)) and torch.equal(rs, rs2)
+        for e, (m, p0) in enumerate(zip(sizes, _padded_starts(sizes))):
+            if m:
+                seg = slice(p0, p0 + 128 * ((m + 127) // 128))
+                assert torch.equal(u8(q_t[:, seg]), u8(q_t2[:, seg])) and torch.equal(cs[e], cs2[e])
+
+
+@pytest.mark.parametrize("sizes", SIZE_CASES, ids=lambda s: "-".join(map(str, s)))
 def test_grouped_gemm_exact_integers(dev, sizes):
     """Integer operands: the grouped forward GEMM must reproduce the per-expert integer matmul exactly, for both
     weight layouts (stacked rows / transposed with a column offset per expert)."""
