@@ -183,6 +183,29 @@ def test_full_size_row_sample(dev):
     assert torch.equal(out2[rows.to(dev)].float() * 2, out[rows.to(dev)].float())
 
 
+@pytest.mark.parametrize("shape", [(16384, 4096, 11008), (11008, 4096, 16384), (4096, 11008, 16384)],
+                         ids=lambda s: "x".join(map(str, s)))
+def test_full_size_gradient_shapes_row_sample(dev, shape):
+    """The grad_input and grad_weight GEMMs of the 7B MLP at full size (e5m2 left operand, as grad_output is cast):
+    a sample of output rows against the oracle, for the default kernel and every persistent variant that
+    takes the shape held to the same bar."""
+    M, N, K = shape
+    a = seeded((M, K), 2001, std=1e-3)
+    b = seeded((N, K), 2002)
+    aq, _, sa = ops.cast_tensorwise(a.to(dev), E5M2)
+    bq, _, sb = ops.cast_tensorwise(b.to(dev), E4M3)
+    out = ops.gemm_fp8(aq, sa, bq, sb)
+    rows = torch.arange(3, M, max(M // 13, 1))
+    ref = O.emulated_mm_f32(aq[rows.to(dev)].cpu(), sa.cpu()[0], bq.cpu().t(), sb.cpu()[0])
+    assert_gemm_close(out[rows.to(dev)], ref, "row sample")
+    names = ops.gemm_variants()
+    for v, name in enumerate(names):
+        if "dma" in name and "k64" not in name:
+            other = ops.gemm_fp8(aq, sa, bq, sb, variant=v)
+            # (the fp32 summation order inside a 128-byte K step differs between the MFMA shapes)
+            assert_gemm_close(other[rows.to(dev)], ref, name)
+
+
 def test_argument_errors(dev):
     from olmo_core_amd.exceptions import MI8KernelError
 
