@@ -211,6 +211,16 @@ int mi8_swiglu_fwd(const void* x1, const void* x3, void* h, int64_t n, uint32_t*
 int mi8_swiglu_bwd(const void* x1, const void* x3, const void* gh, void* g1, void* g3, int64_t n,
                    uint32_t* slots_g1, uint32_t* slots_g3, void* stream);
 
+/* The feed-forward block's backward needs g1 and g3 only as fp8 operands.  Two passes that never write them in bf16:
+ * mi8_swiglu_bwd with g1 = g3 = NULL leaves just the amax partials of what it would have written; this entry point
+ * then recomputes the gradients tile by tile and writes the tensorwise casts of both (row-major [rows, ld_out]
+ * and/or transposed [cols, ld_t] copies, the layouts of mi8_cast_tensorwise; the same layouts for both outputs) with
+ * the scales taken from those partials.  Bytes and scales equal mi8_swiglu_bwd + mi8_cast_tensorwise on each output. */
+int mi8_swiglu_bwd_cast(const void* x1, const void* x3, const void* gh, int64_t rows, int64_t cols,
+                        const uint32_t* slots_g1, const uint32_t* slots_g3, int32_t n_slots, int fp8_dtype, uint32_t flags,
+                        void* out1, void* out3, int64_t ld_out, void* out1_t, void* out3_t, int64_t ld_t,
+                        float* scale_out1, float* scale_out3, void* stream);
+
 /* ---------------------------------------------------------------------------------------------
  * Token permutation around the expert GEMMs of a mixture-of-experts layer.  These replace the copy kernels of
  * src/olmo_core/kernels/moe.py (gather :101-139, padded_scatter / scatter :142-192, scatter_wgrad :251-298,

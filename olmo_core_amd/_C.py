@@ -63,6 +63,11 @@ _SIGNATURES = {
         c_int,
         [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_void_p, c_void_p, c_void_p],
     ),
+    "mi8_swiglu_bwd_cast": (
+        c_int,
+        [c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_void_p, c_void_p, c_int32, c_int, c_uint32, c_void_p, c_void_p,
+         c_int64, c_void_p, c_void_p, c_int64, c_void_p, c_void_p, c_void_p],
+    ),
     "mi8_moe_gather": (
         c_int,
         [c_void_p, c_int, c_int64, c_int64, c_void_p, c_void_p, c_int, c_int32, c_void_p, c_void_p],

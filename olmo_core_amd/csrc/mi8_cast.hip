@@ -491,6 +491,122 @@ __global__ void row_scales_kernel(const uint32_t* __restrict__ row_amax, int64_t
     if (r < T) row_scale[r] = scale_from_amax_bits<FP8>(row_amax[r], pow2);
 }
 
+// Second pass of the SwiGLU backward of the dense feed-forward block when its two outputs are only ever needed
+// in fp8: with the amax of g1 and g3 known (first pass: swiglu_bwd_kernel without outputs), the gradients are
+// recomputed from x1, x3, gh tile by tile and go straight to their row-major and transposed fp8 copies - the bf16
+// tensors g1 and g3 are never written or read back.  Same arithmetic as swiglu_bwd_kernel followed by
+// tile_cast_kernel on each output (the values pass through the same bf16 rounding).
+struct SwigluBwdCastArgs {
+    const uint4* x1;
+    const uint4* x3;
+    const uint4* gh;
+    int64_t rows, cols;
+    const uint32_t* slots1;  // partial maxima of g1 / g3
+    const uint32_t* slots3;
+    int n_slots;
+    bool pow2;
+    uint8_t* out1;    // [rows, ld_out] or null
+    uint8_t* out3;
+    int64_t ld_out;
+    uint8_t* out1_t;  // [cols, ld_t] or null
+    uint8_t* out3_t;
+    int64_t ld_t;
+    float* scale_out1;  // [1]
+    float* scale_out3;
+};
+
+template <int FP8, bool SW>
+__global__ __launch_bounds__(kThreads) void swiglu_bwd_cast_kernel(SwigluBwdCastArgs a)
+{
+    __shared__ __attribute__((aligned(16))) uint32_t lds_t[2][kTile * kTile / 4];
+    __shared__ uint32_t smem[4];
+
+    const int tid = threadIdx.x;
+    const int wave = tid >> 6, lane = tid & 63;
+    const int cl = lane & 15, g = lane >> 4;
+    const int64_t row0 = (int64_t)blockIdx.y * kTile;
+    const int64_t col0 = (int64_t)blockIdx.x * kTile;
+    const int64_t c8 = col0 + 8 * cl;
+    const bool col_ok = c8 < a.cols;
+    const bool first = tid == 0 && blockIdx.x == 0 && blockIdx.y == 0;
+
+    float sc[2];
+    {
+        uint32_t m1 = 0, m3 = 0;
+        for (int i = tid; i < a.n_slots; i += kThreads) {
+            m1 = umax32(m1, a.slots1[i]);
+            m3 = umax32(m3, a.slots3[i]);
+        }
+        m1 = block_umax(m1, smem);
+        __syncthreads();
+        m3 = block_umax(m3, smem);
+        sc[0] = scale_from_amax_bits<FP8>(m1, a.pow2);  // every lane: same bits in, same bits out
+        sc[1] = scale_from_amax_bits<FP8>(m3, a.pow2);
+        if (first) {
+            a.scale_out1[0] = sc[0];
+            a.scale_out3[0] = sc[1];
+        }
+    }
+    uint8_t* const out[2] = {a.out1, a.out3};
+    uint8_t* const out_t[2] = {a.out1_t, a.out3_t};
+    const bool want_t = a.out1_t != nullptr;
+
+#pragma unroll
+    for (int it = 0; it < 2; ++it) {
+        uint4 p[2][4];  // the two gradients of the thread's four rows, eight packed bf16 each
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int64_t r = row0 + 32 * wave + 16 * it + 4 * g + j;
+            p[0][j] = p[1][j] = make_uint4(0, 0, 0, 0);
+            if (col_ok && r < a.rows) {
+                const int64_t v = (r * a.cols + c8) >> 3;
+                swiglu_bwd8(a.x1[v], a.x3[v], a.gh[v], p[0][j], p[1][j]);
+            }
+        }
+#pragma unroll
+        for (int o = 0; o < 2; ++o) {
+            uint32_t lo[4], hi[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const int64_t r = row0 + 32 * wave + 16 * it + 4 * g + j;
+                const bool ok = col_ok && r < a.rows;
+                float v[8];
+                unpack8(p[o][j], v);
+                lo[j] = quant4<FP8, SW>(v[0], v[1], v[2], v[3], sc[o], sc[o], sc[o], sc[o]);
+                hi[j] = quant4<FP8, SW>(v[4], v[5], v[6], v[7], sc[o], sc[o], sc[o], sc[o]);
+                if (!ok) lo[j] = hi[j] = 0;  // padding is zero bytes whatever the scale is (0 * NaN is NaN)
+                if (out[o] && ok) *reinterpret_cast<uint2*>(out[o] + r * a.ld_out + c8) = make_uint2(lo[j], hi[j]);
+            }
+            if (want_t) {
+                uint32_t t[8];
+                transpose4x4_bytes(lo[0], lo[1], lo[2], lo[3], t[0], t[1], t[2], t[3]);
+                transpose4x4_bytes(hi[0], hi[1], hi[2], hi[3], t[4], t[5], t[6], t[7]);
+                const int rd = 8 * wave + 4 * it + g;  // which dword of the column's 32 row-dwords
+#pragma unroll
+                for (int i = 0; i < 8; ++i) {
+                    const int col = 8 * cl + i;
+                    lds_t[o][tile_lds_chunk(col, rd >> 2) * 4 + (rd & 3)] = t[i];
+                }
+            }
+        }
+    }
+    if (want_t) {
+        __syncthreads();
+        const int64_t dst_end = (a.rows + 15) / 16 * 16;
+#pragma unroll
+        for (int o = 0; o < 2; ++o)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int q = tid + kThreads * i;
+                const int col = q >> 3, part = q & 7;
+                const uint4 v = reinterpret_cast<const uint4*>(lds_t[o])[tile_lds_chunk(col, part)];
+                const int64_t c = col0 + col;
+                const int64_t d = row0 + 16 * part;
+                if (c < a.cols && d < dst_end) *reinterpret_cast<uint4*>(out_t[o] + c * a.ld_t + d) = v;
+            }
+    }
+}
+
 // SwiGLU of the dropless-MoE expert layer with the first pass of the two-product cast fused in: the kernel
 // writes h = silu(x1) * x2 (or, backward, the gradients g1, g2 of it) in bf16 and takes, of what it writes, the
 // amax per (group, column) and per row, exactly what grouped_colamax_kernel would compute in a pass of its own.
@@ -831,6 +947,45 @@ extern "C" int mi8_cast_tensorwise(const void* x, int hp_dtype, int64_t rows, in
     dispatch_tile_cast(hp_dtype, fp8_dtype, (flags & MI8_FLAG_SW_CVT) != 0, slots ? kScalarFromSlots : kScalarFromPtr,
                        a, (hipStream_t)stream);
     return launch_status("mi8_cast_tensorwise");
+}
+
+extern "C" int mi8_swiglu_bwd_cast(const void* x1, const void* x3, const void* gh, int64_t rows, int64_t cols,
+                                   const uint32_t* slots_g1, const uint32_t* slots_g3, int32_t n_slots, int fp8_dtype,
+                                   uint32_t flags, void* out1, void* out3, int64_t ld_out, void* out1_t, void* out3_t,
+                                   int64_t ld_t, float* scale_out1, float* scale_out3, void* stream)
+{
+    MI8_REQUIRE(x1 && x3 && gh && slots_g1 && slots_g3 && scale_out1 && scale_out3, MI8_ERR_ARG,
+                "mi8_swiglu_bwd_cast: null pointer");
+    MI8_REQUIRE((out1 != nullptr) == (out3 != nullptr) && (out1_t != nullptr) == (out3_t != nullptr) && (out1 || out1_t),
+                MI8_ERR_ARG, "mi8_swiglu_bwd_cast: request the same layouts (row-major and/or transposed) of both outputs");
+    MI8_REQUIRE(valid_fp8(fp8_dtype), MI8_ERR_ARG, "mi8_swiglu_bwd_cast: unknown dtype");
+    MI8_REQUIRE(rows > 0 && cols > 0, MI8_ERR_ARG, "mi8_swiglu_bwd_cast: empty input");
+    MI8_REQUIRE(n_slots > 0 && n_slots <= MI8_AMAX_SLOTS, MI8_ERR_ARG, "mi8_swiglu_bwd_cast: n_slots %d out of range", n_slots);
+    MI8_REQUIRE(cols % 16 == 0, MI8_ERR_UNSUPPORTED, "mi8_swiglu_bwd_cast: cols (%lld) must be a multiple of 16",
+                (long long)cols);
+    MI8_REQUIRE(aligned16(x1) && aligned16(x3) && aligned16(gh) && aligned16(out1) && aligned16(out3) && aligned16(out1_t) &&
+                    aligned16(out3_t),
+                MI8_ERR_UNSUPPORTED, "mi8_swiglu_bwd_cast: pointers must be 16-byte aligned");
+    if (out1)
+        MI8_REQUIRE(ld_out >= cols && ld_out % 16 == 0, MI8_ERR_UNSUPPORTED,
+                    "mi8_swiglu_bwd_cast: ld_out (%lld) must be a multiple of 16 and at least cols", (long long)ld_out);
+    if (out1_t)
+        MI8_REQUIRE(ld_t >= rows && ld_t % 16 == 0, MI8_ERR_UNSUPPORTED,
+                    "mi8_swiglu_bwd_cast: ld_t (%lld) must be a multiple of 16 and at least rows", (long long)ld_t);
+    SwigluBwdCastArgs a{(const uint4*)x1, (const uint4*)x3, (const uint4*)gh, rows, cols, slots_g1, slots_g3, n_slots,
+                        (flags & MI8_FLAG_POW2_SCALE) != 0, (uint8_t*)out1, (uint8_t*)out3, ld_out, (uint8_t*)out1_t,
+                        (uint8_t*)out3_t, ld_t, scale_out1, scale_out3};
+    const dim3 grid((unsigned)ceil_div(cols, kTile), (unsigned)ceil_div(rows, kTile));
+    hipStream_t st = (hipStream_t)stream;
+    const bool sw = flags & MI8_FLAG_SW_CVT;
+    if (fp8_dtype == MI8_E4M3) {
+        if (sw) hipLaunchKernelGGL((swiglu_bwd_cast_kernel<MI8_E4M3, true>), grid, dim3(kThreads), 0, st, a);
+        else hipLaunchKernelGGL((swiglu_bwd_cast_kernel<MI8_E4M3, false>), grid, dim3(kThreads), 0, st, a);
+    } else {
+        if (sw) hipLaunchKernelGGL((swiglu_bwd_cast_kernel<MI8_E5M2, true>), grid, dim3(kThreads), 0, st, a);
+        else hipLaunchKernelGGL((swiglu_bwd_cast_kernel<MI8_E5M2, false>), grid, dim3(kThreads), 0, st, a);
+    }
+    return launch_status("mi8_swiglu_bwd_cast");
 }
 
 extern "C" int mi8_cast_rowwise(const void* x, int hp_dtype, int64_t rows, int64_t cols, int fp8_dtype,

@@ -57,8 +57,10 @@ __global__ __launch_bounds__(kThreads) void swiglu_bwd_kernel(const uint4* __res
     for (int64_t i = (int64_t)blockIdx.x * kThreads + threadIdx.x; i < nvec; i += stride) {
         uint4 p1, p3;
         swiglu_bwd8(x1[i], x3[i], gh[i], p1, p3);
-        g1[i] = p1;
-        g3[i] = p3;
+        if (g1) {  // (without outputs: only the amax of what would be written)
+            g1[i] = p1;
+            g3[i] = p3;
+        }
         m1 = umax32(m1, absmax_packed(p1));
         m3 = umax32(m3, absmax_packed(p3));
     }
@@ -90,7 +92,9 @@ extern "C" int mi8_swiglu_fwd(const void* x1, const void* x3, void* h, int64_t n
 extern "C" int mi8_swiglu_bwd(const void* x1, const void* x3, const void* gh, void* g1, void* g3, int64_t n,
                               uint32_t* slots_g1, uint32_t* slots_g3, void* stream)
 {
-    MI8_REQUIRE(x1 && x3 && gh && g1 && g3, MI8_ERR_ARG, "mi8_swiglu_bwd: null pointer");
+    MI8_REQUIRE(x1 && x3 && gh, MI8_ERR_ARG, "mi8_swiglu_bwd: null pointer");
+    MI8_REQUIRE((g1 != nullptr) == (g3 != nullptr), MI8_ERR_ARG, "mi8_swiglu_bwd: give both outputs or neither");
+    MI8_REQUIRE(g1 || (slots_g1 && slots_g3), MI8_ERR_ARG, "mi8_swiglu_bwd: nothing to compute");
     MI8_REQUIRE(n > 0 && n % 8 == 0, MI8_ERR_UNSUPPORTED, "mi8_swiglu_bwd: n (%lld) must be a positive multiple of 8",
                 (long long)n);
     MI8_REQUIRE(aligned16(x1) && aligned16(x3) && aligned16(gh) && aligned16(g1) && aligned16(g3),

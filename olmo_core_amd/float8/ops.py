@@ -290,6 +290,48 @@ def swiglu_bwd(x1: torch.Tensor, x3: torch.Tensor, gh: torch.Tensor, want_amax: 
     return g1, g3, ((s1, used) if want_amax else None), ((s3, used) if want_amax else None)
 
 
+def swiglu_bwd_cast(
+    x1: torch.Tensor, x3: torch.Tensor, gh: torch.Tensor, fp8_dtype: torch.dtype, *, pow2: bool = False,
+    want_rowmajor: bool = True, want_transposed: bool = False,
+):
+    """
+    ``swiglu_bwd`` followed by ``cast_tensorwise`` of both gradients, without ever writing them in bf16: a first
+    pass takes only their amax, a second recomputes them tile by tile and writes the fp8 copies.  Returns
+    ``(g1q, g1q_t, scale1, g3q, g3q_t, scale3)`` with the bytes and scales of the two-step route.
+    """
+    _require_gpu(x1, "swiglu_bwd_cast")
+    if not (x1.dtype == x3.dtype == gh.dtype == torch.bfloat16) or not (x1.shape == x3.shape == gh.shape) or x1.dim() != 2:
+        raise ValueError("swiglu_bwd_cast expects three bfloat16 matrices of one shape")
+    if not (want_rowmajor or want_transposed):
+        raise ValueError("swiglu_bwd_cast: no output requested")
+    x1, x3, gh = x1.contiguous(), x3.contiguous(), gh.contiguous()
+    rows, cols = x1.shape
+    dev = x1.device
+    n = x1.numel()
+    s1 = torch.empty(_C.AMAX_SLOTS, dtype=torch.int32, device=dev)
+    s3 = torch.empty(_C.AMAX_SLOTS, dtype=torch.int32, device=dev)
+    _C.check(
+        _C.lib().mi8_swiglu_bwd(x1.data_ptr(), x3.data_ptr(), gh.data_ptr(), None, None, n, s1.data_ptr(), s3.data_ptr(),
+                                _stream(x1)),
+        "mi8_swiglu_bwd",
+    )
+    used = _C.lib().mi8_amax_slots_for(n)
+    q = [_operand((rows, cols), fp8_dtype, dev) if want_rowmajor else None for _ in range(2)]
+    q_t = [_operand((cols, pad16(rows)), fp8_dtype, dev) if want_transposed else None for _ in range(2)]
+    scales = [torch.empty(1, dtype=torch.float32, device=dev) for _ in range(2)]
+    ptr = lambda t: t.data_ptr() if t is not None else None  # noqa: E731
+    _C.check(
+        _C.lib().mi8_swiglu_bwd_cast(
+            x1.data_ptr(), x3.data_ptr(), gh.data_ptr(), rows, cols, s1.data_ptr(), s3.data_ptr(), used,
+            _FP8_CODE[fp8_dtype], _flags(pow2), ptr(q[0]), ptr(q[1]), q[0].stride(0) if want_rowmajor else 0,
+            ptr(q_t[0]), ptr(q_t[1]), q_t[0].stride(0) if want_transposed else 0,
+            scales[0].data_ptr(), scales[1].data_ptr(), _stream(x1),
+        ),
+        "mi8_swiglu_bwd_cast",
+    )
+    return q[0], q_t[0], scales[0], q[1], q_t[1], scales[1]
+
+
 # ---- ragged grouped operations (dropless-MoE expert layer) -------------------------------------------
 
 

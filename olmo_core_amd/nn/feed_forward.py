@@ -94,12 +94,11 @@ class _Float8SwiGLUMLP(torch.autograd.Function):
         gx = gw1 = gw3 = None
         if need_gh:
             gh = ops.gemm_fp8(gyq, sgy, w2q_t, s2, k=D, out_dtype=x_dt)
-            g1, g3, slots1, slots3 = ops.swiglu_bwd(x1, x3, gh, want_amax=True)
-            del gh
             need_t = need_w1 or need_w3
-            g1q, g1q_t, sg1 = ops.cast_tensorwise(g1, go_dt, pow2=pow2, want_rowmajor=need_x, want_transposed=need_t, slots=slots1)
-            g3q, g3q_t, sg3 = ops.cast_tensorwise(g3, go_dt, pow2=pow2, want_rowmajor=need_x, want_transposed=need_t, slots=slots3)
-            del g1, g3
+            # g1 and g3 are needed in fp8 only: amax pass, then recompute-and-cast pass (no bf16 round trip)
+            g1q, g1q_t, sg1, g3q, g3q_t, sg3 = ops.swiglu_bwd_cast(
+                x1, x3, gh, go_dt, pow2=pow2, want_rowmajor=need_x, want_transposed=need_t)
+            del gh
             if need_x:
                 gx = ops.gemm_fp8(g1q, sg1, w1q_t, s1, k=H, out_dtype=x_dt)
                 gx = gx + ops.gemm_fp8(g3q, sg3, w3q_t, s3, k=H, out_dtype=x_dt)

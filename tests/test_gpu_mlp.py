@@ -4,7 +4,7 @@ bits), both vs the oracle's composition (tolerance), and the fused amax against 
 import pytest
 import torch
 
-from helpers import E4M3, assert_gemm_close, assert_scale_equal, gemm_errors, seeded
+from helpers import E4M3, E5M2, assert_gemm_close, assert_scale_equal, gemm_errors, seeded
 from oracle import float8_oracle as O
 
 pytestmark = pytest.mark.gpu
@@ -82,3 +82,28 @@ def test_swiglu_kernels_and_fused_amax(dev):
     q_b, _, s_b = ops.cast_tensorwise(h, E4M3)
     assert torch.equal(q_a.view(torch.uint8), q_b.view(torch.uint8))
     assert_scale_equal(s_a, s_b)
+
+
+@pytest.mark.parametrize("shape", [(333, 528), (128, 128), (1, 16), (1000, 2064)], ids=lambda s: "x".join(map(str, s)))
+@pytest.mark.parametrize("layouts", [(True, True), (True, False), (False, True)], ids=["both", "rows", "transposed"])
+@pytest.mark.parametrize("fp8", [E5M2, E4M3], ids=["e5m2", "e4m3"])
+def test_swiglu_backward_cast_equals_two_steps(dev, shape, layouts, fp8):
+    """The recompute-and-cast route writes the bytes and scales of swiglu_bwd followed by cast_tensorwise on each
+    gradient, in both layouts, including the zero padding of the transposed copies."""
+    x1, x3, gh = seeded(shape, 11).to(dev), seeded(shape, 12).to(dev), seeded(shape, 13, std=1e-3).to(dev)
+    rowmajor, transposed = layouts
+    g1, g3, s1, s3 = ops.swiglu_bwd(x1, x3, gh)
+    want = []
+    for g, sl in ((g1, s1), (g3, s3)):
+        want.append(ops.cast_tensorwise(g, fp8, want_rowmajor=rowmajor, want_transposed=transposed, slots=sl))
+    q1, q1t, sc1, q3, q3t, sc3 = ops.swiglu_bwd_cast(x1, x3, gh, fp8, want_rowmajor=rowmajor, want_transposed=transposed)
+    for (wq, wqt, ws), (q, qt, sc) in zip(want, ((q1, q1t, sc1), (q3, q3t, sc3))):
+        assert_scale_equal(sc, ws)
+        if rowmajor:
+            assert torch.equal(q.view(torch.uint8), wq.view(torch.uint8))
+        else:
+            assert q is None
+        if transposed:
+            assert torch.equal(qt.view(torch.uint8), wqt.view(torch.uint8))
+        else:
+            assert qt is None
