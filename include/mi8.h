@@ -148,7 +148,7 @@ const char* mi8_gemm_variant_name(int variant);
  * ------------------------------------------------------------------------------------------- */
 
 /* Upper bound of the padded token axis used by the grouped transposed layouts: every group's segment starts at a
- * multiple of 128. */
+ * multiple of 128 (T rounded up to 128, plus 128 per group after the first). */
 int64_t mi8_grouped_padded_rows(int64_t T, int32_t num_groups);
 
 /* Per-group, per-column dynamic cast with transposed output: for group e (rows R_e of x[T, cols]) the scale of

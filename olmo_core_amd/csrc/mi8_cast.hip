@@ -1053,7 +1053,8 @@ extern "C" int mi8_cast_colwise_t(const void* x, int hp_dtype, int64_t rows, int
 extern "C" int64_t mi8_grouped_padded_rows(int64_t T, int32_t num_groups)
 {
     if (T < 0 || num_groups < 0) return 0;
-    return round_up(T, kTile) + (int64_t)kTile * num_groups;
+    // sum of ceil(m_e / 128) over groups whose sizes sum to at most T is at most ceil(T / 128) + num_groups - 1
+    return round_up(T, kTile) + (int64_t)kTile * (num_groups > 0 ? num_groups - 1 : 0);
 }
 
 namespace mi8 {

@@ -14,7 +14,7 @@ from typing import Optional, Tuple
 import torch
 
 from . import ops
-from .linear import _COMPILED_CONFIGS, _backward_impl, _forward_impl, _saves_quantised
+from .linear import _COMPILED_CONFIGS, _backward_impl, _forward_impl, _is_axiswise, _saves_quantised
 
 _CONFIGS = _COMPILED_CONFIGS  # configs travel through the operators as indices into this list
 
@@ -36,13 +36,16 @@ def _(x2, weight, weight_scale, cfg, need_gx, need_gw):
     N = weight.shape[0]
     x_is_q, w_is_q = _saves_quantised(c, need_gx, need_gw)
 
-    def saved(is_q, rows, cols, dtype):
+    def saved(is_q, rows, cols, cast):
         if not is_q:
             return x2.new_empty(0), x2.new_empty(0)
-        return x2.new_empty((cols, (rows + 15) // 16 * 16), dtype=dtype), x2.new_empty(1, dtype=torch.float32)
+        if _is_axiswise(cast):  # transposed copy padded to 128 rows, one scale per column
+            return (x2.new_empty((cols, (rows + 127) // 128 * 128), dtype=cast.target_dtype),
+                    x2.new_empty(cols, dtype=torch.float32))
+        return x2.new_empty((cols, (rows + 15) // 16 * 16), dtype=cast.target_dtype), x2.new_empty(1, dtype=torch.float32)
 
-    xa, xb = saved(x_is_q, M, K, c.cast_config_input.target_dtype)
-    wa, wb = saved(w_is_q, N, K, c.cast_config_weight.target_dtype)
+    xa, xb = saved(x_is_q, M, K, c.cast_config_input)
+    wa, wb = saved(w_is_q, N, K, c.cast_config_weight)
     return x2.new_empty((M, N)), xa, xb, wa, wb
 
 

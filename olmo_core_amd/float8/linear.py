@@ -49,6 +49,12 @@ def _shared_tensorwise(a: CastConfig, b: CastConfig) -> bool:
     return _is_tensorwise(a) and _is_tensorwise(b) and a.target_dtype == b.target_dtype
 
 
+def _shared_axiswise(a: CastConfig, b: CastConfig) -> bool:
+    """Two uses of one tensor, one scaled per row and one per column, in the same fp8 type: both copies come out
+    of one two-product cast."""
+    return _is_axiswise(a) and _is_axiswise(b) and a.target_dtype == b.target_dtype
+
+
 def _rows_operand(x: torch.Tensor, c: CastConfig, pow2: bool) -> Tuple[torch.Tensor, torch.Tensor]:
     """Operand reduced along its rows' elements (K = last dim of x): row-major fp8 + scale [1] or [rows]."""
     if _is_tensorwise(c):
@@ -70,8 +76,10 @@ def _saves_quantised(c: Float8LinearConfig, need_gx: bool, need_gw: bool) -> Tup
     of the high-precision tensor: possible when forward and backward quantise that tensor identically."""
     if _is_disabled(c.cast_config_input):
         return False, False
-    x_is_q = need_gw and _shared_tensorwise(c.cast_config_input, c.cast_config_input_for_grad_weight)
-    w_is_q = need_gx and _shared_tensorwise(c.cast_config_weight, c.cast_config_weight_for_grad_input)
+    ci, ciw = c.cast_config_input, c.cast_config_input_for_grad_weight
+    cw, cwi = c.cast_config_weight, c.cast_config_weight_for_grad_input
+    x_is_q = need_gw and (_shared_tensorwise(ci, ciw) or _shared_axiswise(ci, ciw))
+    w_is_q = need_gx and (_shared_tensorwise(cw, cwi) or _shared_axiswise(cw, cwi))
     return x_is_q, w_is_q
 
 
@@ -89,6 +97,9 @@ def _forward_impl(x2, weight, c: Float8LinearConfig, weight_scale, need_gx: bool
         )
         if share_x:
             x_saved = (xq_t, sx)
+    elif share_x:  # per-row copy for this GEMM, per-column transposed copy for grad_weight, one cast
+        xq, sx, xq_t, sxc = ops.cast_rows_and_colwise_t(x2, c.cast_config_input.target_dtype, pow2=pow2)
+        x_saved = (xq_t, sxc)
     else:
         xq, sx = ops.cast_rowwise(x2, c.cast_config_input.target_dtype, pow2=pow2)
     if _is_tensorwise(c.cast_config_weight):
@@ -98,6 +109,9 @@ def _forward_impl(x2, weight, c: Float8LinearConfig, weight_scale, need_gx: bool
         )
         if share_w:
             w_saved = (wq_t, sw)
+    elif share_w:
+        wq, sw, wq_t, swc = ops.cast_rows_and_colwise_t(weight, c.cast_config_weight.target_dtype, pow2=pow2)
+        w_saved = (wq_t, swc)
     else:
         wq, sw = ops.cast_rowwise(weight, c.cast_config_weight.target_dtype, pow2=pow2)
     return ops.gemm_fp8(xq, sx, wq, sw, out_dtype=x2.dtype), x_saved, w_saved
@@ -116,6 +130,9 @@ def _backward_impl(go2, c: Float8LinearConfig, N: int, x_dtype, w_dtype, x_part,
     if need_gx and need_gw and _shared_tensorwise(cg, cgw):
         q, q_t, s = ops.cast_tensorwise(go2, cg.target_dtype, pow2=pow2, want_rowmajor=True, want_transposed=True)
         go_rows, go_cols = (q, s), (q_t, s)
+    elif need_gx and need_gw and _shared_axiswise(cg, cgw):
+        q, rs, q_t, cs = ops.cast_rows_and_colwise_t(go2, cg.target_dtype, pow2=pow2)
+        go_rows, go_cols = (q, rs), (q_t, cs)
 
     gx = gw = None
     if need_gx:

@@ -458,6 +458,27 @@ def grouped_cast_rows_and_colwise_t(
     return q, row_scale, q_t, scale
 
 
+_ONE_GROUP: dict = {}
+
+
+def cast_rows_and_colwise_t(
+    x: torch.Tensor, fp8_dtype: torch.dtype, *, pow2: bool = False
+) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]:
+    """
+    :func:`cast_rowwise` and :func:`cast_colwise_t` of one tensor from one pair of passes (the grouped two-product
+    cast with a single group): ``(q [rows, cols], row_scale [rows], q_t [cols, rows rounded up to 128], col_scale
+    [cols])``; ``q_t`` is zero beyond ``rows``.  Bytes and scales are those of the two separate casts.
+    """
+    x = _hp2d(x, "cast_rows_and_colwise_t")
+    rows = x.shape[0]
+    key = (rows, x.device)
+    sizes = _ONE_GROUP.get(key)
+    if sizes is None:
+        sizes = _ONE_GROUP[key] = torch.tensor([rows], dtype=torch.int64, device=x.device)
+    q, row_scale, q_t, col_scale = grouped_cast_rows_and_colwise_t(x, sizes, fp8_dtype, pow2=pow2)
+    return q, row_scale, q_t, col_scale.reshape(-1)
+
+
 def grouped_gemm_fp8(
     a: torch.Tensor,
     sa: torch.Tensor,
