@@ -83,9 +83,11 @@ def _saves_quantised(c: Float8LinearConfig, need_gx: bool, need_gw: bool) -> Tup
     return x_is_q, w_is_q
 
 
-def _forward_impl(x2, weight, c: Float8LinearConfig, weight_scale, need_gx: bool, need_gw: bool):
+def _forward_impl(x2, weight, c: Float8LinearConfig, weight_scale, need_gx: bool, need_gw: bool, weight_ops=None):
     """y = x2 @ weight^T in float8.  Returns ``(y, x_saved, w_saved)``: the tensors the backward needs for x and
-    for the weight, each either ``(q_t, scale)`` (see :func:`_saves_quantised`) or ``None`` (keep the input)."""
+    for the weight, each either ``(q_t, scale)`` (see :func:`_saves_quantised`) or ``None`` (keep the input).
+    ``weight_ops``: ``(q, q_t, scale)`` of the weight kept by the module (:meth:`Float8Linear.weight_operands`);
+    the weight is then not quantised here."""
     pow2 = c.round_scales_to_power_of_2
     share_x, share_w = _saves_quantised(c, need_gx, need_gw)
     x_saved = w_saved = None
@@ -102,7 +104,11 @@ def _forward_impl(x2, weight, c: Float8LinearConfig, weight_scale, need_gx: bool
         x_saved = (xq_t, sxc)
     else:
         xq, sx = ops.cast_rowwise(x2, c.cast_config_input.target_dtype, pow2=pow2)
-    if _is_tensorwise(c.cast_config_weight):
+    if weight_ops is not None:
+        wq, wq_t, sw = weight_ops
+        if share_w:
+            w_saved = (wq_t, sw)
+    elif _is_tensorwise(c.cast_config_weight):
         wq, wq_t, sw = ops.cast_tensorwise(
             weight, c.cast_config_weight.target_dtype, pow2=pow2, want_rowmajor=True, want_transposed=share_w,
             scale=weight_scale,
@@ -160,9 +166,10 @@ class _Float8Matmul(torch.autograd.Function):
     """y = x @ W^T with float8 operands; x [M, K] and W [N, K] in high precision."""
 
     @staticmethod
-    def forward(ctx, x2: torch.Tensor, weight: torch.Tensor, config: Float8LinearConfig, weight_scale=None):
+    def forward(ctx, x2: torch.Tensor, weight: torch.Tensor, config: Float8LinearConfig, weight_scale=None,
+                weight_ops=None):
         need_gx, need_gw = ctx.needs_input_grad[0], ctx.needs_input_grad[1]
-        y, x_saved, w_saved = _forward_impl(x2, weight, config, weight_scale, need_gx, need_gw)
+        y, x_saved, w_saved = _forward_impl(x2, weight, config, weight_scale, need_gx, need_gw, weight_ops)
         ctx.config = config
         ctx.x_dtype, ctx.w_dtype = x2.dtype, weight.dtype
         ctx.shapes = (x2.shape[0], x2.shape[1], weight.shape[0])
@@ -184,7 +191,7 @@ class _Float8Matmul(torch.autograd.Function):
             go.reshape(M, N), ctx.config, N, ctx.x_dtype, ctx.w_dtype, saved[: ctx.n_x], saved[ctx.n_x :],
             ctx.x_is_q, ctx.w_is_q, ctx.needs_input_grad[0], ctx.needs_input_grad[1],
         )
-        return gx, gw, None, None
+        return gx, gw, None, None, None
 
 
 # Operator arguments must be plain values: under torch.compile a config travels as its index in this list.  Configs
@@ -202,17 +209,20 @@ def _register_config(c: Float8LinearConfig) -> int:
 
 
 @torch.compiler.disable
-def _eager_matmul(x2, weight, config, weight_scale):
-    return _Float8Matmul.apply(x2, weight, config, weight_scale)
+def _eager_matmul(x2, weight, config, weight_scale, weight_ops=None):
+    return _Float8Matmul.apply(x2, weight, config, weight_scale, weight_ops)
 
 
 def float8_linear_function(
-    x: torch.Tensor, weight: torch.Tensor, config: Float8LinearConfig, weight_scale: Optional[torch.Tensor] = None
+    x: torch.Tensor, weight: torch.Tensor, config: Float8LinearConfig, weight_scale: Optional[torch.Tensor] = None,
+    weight_ops: Optional[Tuple[torch.Tensor, torch.Tensor, torch.Tensor]] = None,
 ) -> torch.Tensor:
     """``x [*, K] @ weight[N, K].T`` through the float8 path, differentiable in x and weight.
 
     ``weight_scale``: a precomputed tensorwise scale of ``weight`` (float32 ``[1]``), used instead of reducing the
     weight's amax again; ignored unless the weight cast is tensorwise.
+    ``weight_ops``: float8 copies of ``weight`` made earlier (``(q [N, K], q_t [K, pad16(N)], scale [1])``, as
+    :meth:`Float8Linear.weight_operands` returns them), used instead of quantising ``weight`` again; eager only.
 
     Under ``torch.compile`` the call becomes a pair of registered custom operators (forward, backward) with shape
     functions, so a compiled block keeps one graph; eagerly it is an ordinary ``autograd.Function``.
@@ -227,7 +237,7 @@ def float8_linear_function(
 
         y = compiled.linear(x2, weight, cfg_id, weight_scale)
     else:  # eager, or a config no module registered: a graph break
-        y = _eager_matmul(x2, weight, config, weight_scale)
+        y = _eager_matmul(x2, weight, config, weight_scale, weight_ops)
     return y.reshape(*x.shape[:-1], weight.shape[0])
 
 
@@ -253,8 +263,10 @@ class Float8Linear(nn.Linear):
         if torch.is_autocast_enabled():
             input = input.to(torch.get_autocast_dtype(input.device.type))
         # (the stored scale is checked against the weight's address and version counter: not traceable)
-        scale = None if torch.compiler.is_compiling() else self.precomputed_weight_scale()
-        out = float8_linear_function(input, self.weight, self.config, scale)
+        compiling = torch.compiler.is_compiling()
+        scale = None if compiling else self.precomputed_weight_scale()
+        w_ops = None if compiling else self.weight_operands()
+        out = float8_linear_function(input, self.weight, self.config, scale, w_ops)
         if self.bias is not None:
             out = out + self.bias.to(out.dtype)
         return out
@@ -270,6 +282,39 @@ class Float8Linear(nn.Linear):
         if w.data_ptr() != ptr or w._version != version or not _is_tensorwise(self.config.cast_config_weight):
             return None
         return scale
+
+    def weight_operands(self) -> Optional[Tuple[torch.Tensor, torch.Tensor, torch.Tensor]]:
+        """Float8 copies of the weight that outlive one call: ``(q [N, K], q_t [K, pad16(N)], scale [1])``, made
+        on first use and kept until the weight is modified or replaced (address and version counter), so that
+        the micro-batches of one optimizer step, or the steps of a generation loop, quantise each weight once.
+
+        Only with ``config.enable_fsdp_float8_all_gather``: upstream that switch makes FSDP hold and communicate
+        the float8 weight (computed from the precomputed scale, ``src/olmo_core/float8/__init__.py:54-62``,
+        ``src/olmo_core/float8/ao.py:173-180``); on one device what remains of it is that the float8 weight is
+        materialised once per weight update rather than once per forward.  Costs two bytes per parameter.
+        ``None`` when the switch is off, the weight is not a contiguous GPU tensor, or forward and grad_input
+        quantise the weight differently.  Bytes and scale equal those a forward would make itself.  (A write
+        through ``weight.data`` moves no version counter and goes unnoticed, as for the precomputed scales;
+        :func:`precompute_float8_dynamic_scale_for_fsdp` drops the copies.)"""
+        c = self.config
+        if not c.enable_fsdp_float8_all_gather:
+            return None
+        w = self.weight
+        if not _shared_tensorwise(c.cast_config_weight, c.cast_config_weight_for_grad_input):
+            return None
+        if not w.is_cuda or not w.is_contiguous() or w.dtype not in (torch.bfloat16, torch.float32):
+            return None
+        key = (w.data_ptr(), w._version, w.dtype, tuple(w.shape))
+        entry = getattr(self, "_weight_operands", None)
+        if entry is not None and entry[0] == key:
+            return entry[1]
+        with torch.no_grad():
+            made = ops.cast_tensorwise(
+                w.detach(), c.cast_config_weight.target_dtype, pow2=c.round_scales_to_power_of_2,
+                want_rowmajor=True, want_transposed=True, scale=self.precomputed_weight_scale(),
+            )
+        self._weight_operands = (key, made)
+        return made
 
     def extra_repr(self) -> str:
         c = self.config
@@ -355,6 +400,7 @@ def precompute_float8_dynamic_scale_for_fsdp(module: nn.Module) -> None:
         if not isinstance(m, Float8Linear):
             continue
         m._precomputed_weight_scale = None
+        m._weight_operands = None
         c = m.config
         w = m.weight
         if not _is_tensorwise(c.cast_config_weight) or not w.is_cuda or not w.is_contiguous():

@@ -46,7 +46,7 @@ class _Float8SwiGLUMLP(torch.autograd.Function):
     """y = (silu(x W1^T) * (x W3^T)) W2^T with tensorwise float8 GEMMs; x [M, D], W1/W3 [H, D], W2 [D, H]."""
 
     @staticmethod
-    def forward(ctx, x, w1, w2, w3, config, ws1=None, ws2=None, ws3=None):
+    def forward(ctx, x, w1, w2, w3, config, ws1=None, ws2=None, ws3=None, wo1=None, wo2=None, wo3=None):
         c = config
         pow2 = c.round_scales_to_power_of_2
         in_dt, w_dt, go_dt = (
@@ -57,10 +57,11 @@ class _Float8SwiGLUMLP(torch.autograd.Function):
         need = ctx.needs_input_grad
         any_grad = any(need[:4])
         xq, xq_t, sx = ops.cast_tensorwise(x, in_dt, pow2=pow2, want_transposed=need[1] or need[3])
-        # ws*: weight scales precomputed after the optimizer step (None: reduce the amax here)
-        w1q, w1q_t, s1 = ops.cast_tensorwise(w1, w_dt, pow2=pow2, want_transposed=need[0], scale=ws1)
-        w3q, w3q_t, s3 = ops.cast_tensorwise(w3, w_dt, pow2=pow2, want_transposed=need[0], scale=ws3)
-        w2q, w2q_t, s2 = ops.cast_tensorwise(w2, w_dt, pow2=pow2, want_transposed=any_grad, scale=ws2)
+        # ws*: weight scales precomputed after the optimizer step (None: reduce the amax here);
+        # wo*: float8 copies the modules keep between calls (None: quantise the weight here)
+        w1q, w1q_t, s1 = wo1 or ops.cast_tensorwise(w1, w_dt, pow2=pow2, want_transposed=need[0], scale=ws1)
+        w3q, w3q_t, s3 = wo3 or ops.cast_tensorwise(w3, w_dt, pow2=pow2, want_transposed=need[0], scale=ws3)
+        w2q, w2q_t, s2 = wo2 or ops.cast_tensorwise(w2, w_dt, pow2=pow2, want_transposed=any_grad, scale=ws2)
         x1 = ops.gemm_fp8(xq, sx, w1q, s1, out_dtype=x.dtype)
         x3 = ops.gemm_fp8(xq, sx, w3q, s3, out_dtype=x.dtype)
         h, h_slots = ops.swiglu_fwd(x1, x3, want_amax=True)
@@ -110,7 +111,7 @@ class _Float8SwiGLUMLP(torch.autograd.Function):
         def as_param(g, dt):
             return g if g is None or g.dtype == dt else g.to(dt)
 
-        return gx, as_param(gw1, w1_dt), as_param(gw2, w2_dt), as_param(gw3, w3_dt), None, None, None, None
+        return (gx, as_param(gw1, w1_dt), as_param(gw2, w2_dt), as_param(gw3, w3_dt)) + (None,) * 7
 
 
 def _fusable(ff: "FeedForward", x: torch.Tensor) -> bool:
@@ -129,8 +130,8 @@ def _fusable(ff: "FeedForward", x: torch.Tensor) -> bool:
 
 
 @torch.compiler.disable
-def _fused_mlp(x2, w1, w2, w3, config, ws1=None, ws2=None, ws3=None):
-    return _Float8SwiGLUMLP.apply(x2, w1, w2, w3, config, ws1, ws2, ws3)
+def _fused_mlp(x2, w1, w2, w3, config, ws1=None, ws2=None, ws3=None, wo1=None, wo2=None, wo3=None):
+    return _Float8SwiGLUMLP.apply(x2, w1, w2, w3, config, ws1, ws2, ws3, wo1, wo2, wo3)
 
 
 class FeedForward(nn.Module):
@@ -160,7 +161,8 @@ class FeedForward(nn.Module):
             x2 = x.reshape(-1, x.shape[-1])
             y = _fused_mlp(x2, self.w1.weight, self.w2.weight, self.w3.weight, self.w1.config,
                            self.w1.precomputed_weight_scale(), self.w2.precomputed_weight_scale(),
-                           self.w3.precomputed_weight_scale())
+                           self.w3.precomputed_weight_scale(), self.w1.weight_operands(), self.w2.weight_operands(),
+                           self.w3.weight_operands())
             return y.reshape(*x.shape[:-1], self.w2.weight.shape[0])
         x1, x3 = self.w1(x), self.w3(x)
         if x1.is_cuda and x1.dtype == torch.bfloat16 and not compiling:
