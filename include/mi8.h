@@ -135,6 +135,21 @@ int mi8_gemm_fp8(const void* a, int a_dtype, int64_t lda, const void* b, int b_d
                  int64_t N, int64_t K, const float* sa, int sa_is_vector, const float* sb, int sb_is_vector,
                  void* out, int out_dtype, int64_t ldc, int variant, void* stream);
 
+/* The same product with K cut into `splits` slices, for problems whose few output tiles would leave most of the
+ * GPU idle (a few hundred rows of A against a weight matrix): every slice is summed by its own workgroups into
+ * an fp32 plane of `workspace`, a second kernel adds the planes in slice order (results do not depend on
+ * scheduling), applies the scales and rounds.  Arguments as mi8_gemm_fp8; splits in 1..min(64, ceil(K/128));
+ * workspace: 16-byte aligned device memory of mi8_gemm_splitk_workspace_bytes(M, N, splits) bytes, owned by the
+ * caller, free for reuse once the call's work on `stream` is done.  mi8_gemm_splitk_suggest returns the number
+ * of slices the library would use for a shape (1: call mi8_gemm_fp8 instead).  No counterpart upstream: the
+ * reference leaves the choice of GEMM algorithm to torch._scaled_mm's backend. */
+int mi8_gemm_fp8_splitk(const void* a, int a_dtype, int64_t lda, const void* b, int b_dtype, int64_t ldb,
+                        int64_t M, int64_t N, int64_t K, const float* sa, int sa_is_vector, const float* sb,
+                        int sb_is_vector, void* out, int out_dtype, int64_t ldc, int splits, void* workspace,
+                        int64_t workspace_bytes, void* stream);
+int mi8_gemm_splitk_suggest(int64_t M, int64_t N, int64_t K);
+int64_t mi8_gemm_splitk_workspace_bytes(int64_t M, int64_t N, int splits);
+
 /* Number of GEMM kernel variants compiled in (variant ids 0..n-1; -1 lets the library choose by shape). */
 int mi8_gemm_num_variants(void);
 const char* mi8_gemm_variant_name(int variant);

@@ -56,6 +56,13 @@ _SIGNATURES = {
         [c_void_p, c_int, c_int64, c_void_p, c_int, c_int64, c_int64, c_int64, c_int64, c_void_p, c_int, c_void_p,
          c_int, c_void_p, c_int, c_int64, c_int, c_void_p],
     ),
+    "mi8_gemm_fp8_splitk": (
+        c_int,
+        [c_void_p, c_int, c_int64, c_void_p, c_int, c_int64, c_int64, c_int64, c_int64, c_void_p, c_int, c_void_p,
+         c_int, c_void_p, c_int, c_int64, c_int, c_void_p, c_int64, c_void_p],
+    ),
+    "mi8_gemm_splitk_suggest": (c_int, [c_int64, c_int64, c_int64]),
+    "mi8_gemm_splitk_workspace_bytes": (c_int64, [c_int64, c_int64, c_int]),
     "mi8_gemm_num_variants": (c_int, []),
     "mi8_gemm_variant_name": (c_char_p, [c_int]),
     "mi8_swiglu_fwd": (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_void_p, c_void_p]),

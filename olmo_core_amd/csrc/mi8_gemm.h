@@ -81,6 +81,10 @@ int launch_dma8(GemmArgs& g, int a_dtype, int b_dtype, hipStream_t st);
 int launch_dma4(GemmArgs& g, int a_dtype, int b_dtype, hipStream_t st);
 // four waves of 128 x 128 on 16x16x128 MFMAs (mi8_gemm_m16.hip), same requirements
 int launch_m16(GemmArgs& g, int a_dtype, int b_dtype, hipStream_t st);
+// a few rows of A (M <= kSkinnyMaxM) against all of B, bound by reading B once (mi8_gemm_skinny.hip): any N,
+// K % 16 == 0, any mix of single scales and scale vectors, bf16 or fp32 output
+constexpr int kSkinnyMaxM = 64;
+int launch_skinny(GemmArgs& g, int a_dtype, int b_dtype, hipStream_t st);
 // the same kernel over the ragged grouped problems (bf16 output, per-row / per-column scale vectors):
 // forward / grad_input (T, N >= 256, K % 128 == 0) and grad_weight (N, Kl >= 256)
 int launch_m16_grouped(const uint8_t* a, int a_dtype, int64_t lda, const uint8_t* b, int b_dtype, int64_t ldb,

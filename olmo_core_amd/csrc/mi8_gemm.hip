@@ -22,6 +22,115 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_fp8_kernel(GemmArgs g)
     gemm_tile_body<BM, BN, WM, WN, CBSZ, BLGP>(g, tm * BM, tn * BN, lds);
 }
 
+// ---- split K ---------------------------------------------------------------------------------------
+// A problem with few output tiles and a long K leaves most compute units idle while every busy one pays a
+// memory latency per 128-byte K step.  Here blockIdx.y cuts K into slices: every (tile, slice) workgroup runs
+// the same tile routine on its slice (operand pointers moved along the rows, which are K-contiguous) and stores
+// the raw fp32 sums into its own plane of a workspace; a second kernel adds the planes in a fixed order (the
+// result does not depend on scheduling), applies the scales and rounds.
+
+constexpr int kSplitTile = 128;
+
+struct SplitArgs {
+    GemmArgs g;          // the problem; C, ldc, scales describe the final output
+    float* planes;       // [splits][M][ld_plane] fp32
+    int64_t ld_plane;    // round_up(N, 4)
+    int steps_per_split; // 128-byte K steps per slice; the last slice may be shorter, none is empty
+    int splits;
+};
+
+template <int CBSZ, int BLGP>
+__global__ __launch_bounds__(256, 1) void gemm_fp8_splitk_kernel(SplitArgs a)
+{
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+    GemmArgs g = a.g;
+    int tm, tn;
+    if (!tile_of_block(g, tm, tn)) return;
+    const int split = (int)blockIdx.y;
+    const int k0 = split * a.steps_per_split * BK;
+    const int left = g.K - k0;
+    g.A += k0;
+    g.B += k0;
+    g.K = left < a.steps_per_split * BK ? left : a.steps_per_split * BK;
+    g.C = a.planes + (int64_t)split * g.M * a.ld_plane;
+    g.c_f32 = 1;
+    g.ldc = a.ld_plane;
+    g.sa = g.sb = nullptr;
+    g.sa_vec = g.sb_vec = 0;
+    gemm_tile_body<kSplitTile, kSplitTile, 2, 2, CBSZ, BLGP>(g, tm * kSplitTile, tn * kSplitTile, lds);
+}
+
+// out[m][n] = round( (sum over planes, in plane order) * (1/sa) * (1/sb) ); four columns per thread
+__global__ __launch_bounds__(256) void splitk_reduce_kernel(SplitArgs a)
+{
+    const GemmArgs& g = a.g;
+    const int64_t quads_per_row = a.ld_plane / 4;
+    const int64_t q = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (q >= (int64_t)g.M * quads_per_row) return;
+    const int m = (int)(q / quads_per_row);
+    const int n = (int)(q % quads_per_row) * 4;
+    const int64_t plane = (int64_t)g.M * a.ld_plane;
+    const float* p = a.planes + (int64_t)m * a.ld_plane + n;
+    float4 s = *reinterpret_cast<const float4*>(p);
+    for (int i = 1; i < a.splits; ++i) {
+        const float4 t = *reinterpret_cast<const float4*>(p + i * plane);
+        s.x += t.x;
+        s.y += t.y;
+        s.z += t.z;
+        s.w += t.w;
+    }
+    // same scale arithmetic as the tile routine's own epilogue
+    const float isa = g.sa_vec ? __builtin_amdgcn_rcpf(g.sa[m]) : 1.0f / g.sa[0];
+    const float isb_scalar = g.sb_vec ? 0.0f : 1.0f / g.sb[0];
+    const float v[4] = {s.x, s.y, s.z, s.w};
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        if (n + j >= g.N) break;
+        const float isb = g.sb_vec ? __builtin_amdgcn_rcpf(g.sb[n + j]) : isb_scalar;
+        const float r = v[j] * isa * isb;
+        if (g.c_f32)
+            reinterpret_cast<float*>(g.C)[(int64_t)m * g.ldc + n + j] = r;
+        else
+            reinterpret_cast<uint16_t*>(g.C)[(int64_t)m * g.ldc + n + j] = f32_to_bf16_bits(r);
+    }
+}
+
+template <int CBSZ, int BLGP>
+int launch_splitk_typed(const SplitArgs& a, hipStream_t st)
+{
+    auto kern = gemm_fp8_splitk_kernel<CBSZ, BLGP>;
+    constexpr int lds_bytes = 2 * (kSplitTile + kSplitTile) * BK;
+    static bool configured = false;
+    if (!configured) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
+        if (e != hipSuccess) {
+            set_error("mi8_gemm_fp8_splitk: cannot reserve %d bytes of LDS: %s", lds_bytes, hipGetErrorString(e));
+            return MI8_ERR_LAUNCH;
+        }
+        configured = true;
+    }
+    const int total = a.g.tiles_m * a.g.tiles_n;
+    hipLaunchKernelGGL(kern, dim3(((total + 7) / 8) * 8, a.splits), dim3(256), lds_bytes, st, a);
+    const int64_t quads = (int64_t)a.g.M * (a.ld_plane / 4);
+    hipLaunchKernelGGL(splitk_reduce_kernel, dim3((unsigned)((quads + 255) / 256)), dim3(256), 0, st, a);
+    return launch_status("mi8_gemm_fp8_splitk");
+}
+
+// slices for a problem, 1 = do not split: aim at two workgroups per compute unit, at least four K steps a slice
+int suggested_splits(int64_t M, int64_t N, int64_t K)
+{
+    const int64_t tiles = ((M + kSplitTile - 1) / kSplitTile) * ((N + kSplitTile - 1) / kSplitTile);
+    const int64_t steps = (K + BK - 1) / BK;
+    if (M <= 16 || tiles >= 256 || steps < 8) return 1;  // (up to 16 rows: the few-rows kernel reads B once)
+    int64_t s = 512 / tiles;
+    if (s > steps / 4) s = steps / 4;
+    if (s > 32) s = 32;
+    if (s < 2) return 1;
+    const int64_t per = (steps + s - 1) / s;
+    return (int)((steps + per - 1) / per);  // no empty slice
+}
+
 // ---- variants --------------------------------------------------------------------------------------
 
 struct Variant {
@@ -39,8 +148,9 @@ constexpr Variant kVariants[] = {
     {"256x256_dma_w8_k128x2", 256, 256, 512},
     {"256x256_dma_w4x128_k128x2", 256, 256, 256},
     {"256x256_dma_w4x128_m16x128", 256, 256, 256},
+    {"rows64x16_k8_m16x128", 64, 16, 512},
 };
-constexpr int kDma = 5, kDma8 = 6, kDma4 = 7, kM16 = 8;
+constexpr int kSmallTile = 2, kDma = 5, kDma8 = 6, kDma4 = 7, kM16 = 8, kSkinny = 9;
 constexpr int kNumVariants = sizeof(kVariants) / sizeof(kVariants[0]);
 
 template <int BM, int BN, int WM, int WN, int CBSZ, int BLGP>
@@ -120,8 +230,20 @@ extern "C" int mi8_gemm_fp8(const void* a, int a_dtype, int64_t lda, const void*
                         out_dtype == MI8_BF16 && (!sb_is_vector || aligned16(sb)) &&
                         (sa_is_vector != 0) == (sb_is_vector != 0);
     // measured on MI355X on the benchmark configurations' shapes: the four-wave layout beats the eight-wave one
-    // by 0-14 %, and its 16x16x128 form beats its 32x32x64 form by 3-9 % (random operands, power-limited clocks)
-    if (variant < 0) variant = dma_ok ? (K % 128 == 0 ? kM16 : kDma) : 1;
+    // by 0-14 %, and its 16x16x128 form beats its 32x32x64 form by 3-9 % (random operands, power-limited clocks).
+    // Problems with few 256 x 256 tiles leave most compute units idle and pay one memory latency per K step:
+    // 128 x 128 tiles put four times the workgroups to work (512 x 11008 x 4096: 42 us against 70 us), and a few
+    // rows of A go to the kernel that streams B once.
+    if (variant < 0) {
+        const int64_t tiles256 = ((M + 255) / 256) * ((N + 255) / 256);
+        if (M <= kSkinnyMaxM)
+            variant = kSkinny;
+        else if (dma_ok)
+            variant = tiles256 <= 96 ? kSmallTile : (K % 128 == 0 ? kM16 : kDma);
+        else
+            variant = tiles256 <= 384 ? kSmallTile : 1;
+    }
+    if (variant == kSkinny) return launch_skinny(g, a_dtype, b_dtype, st);
     if (variant == kDma8 && dma_ok && K % 128 == 0) return launch_dma8(g, a_dtype, b_dtype, st);
     if (variant == kDma4 && dma_ok && K % 128 == 0) return launch_dma4(g, a_dtype, b_dtype, st);
     if (variant == kM16 && dma_ok && K % 128 == 0) return launch_m16(g, a_dtype, b_dtype, st);
@@ -135,4 +257,60 @@ extern "C" int mi8_gemm_fp8(const void* a, int a_dtype, int64_t lda, const void*
     if (a_dtype == MI8_E4M3)
         return b_dtype == MI8_E4M3 ? launch_variant<0, 0>(variant, g, st) : launch_variant<0, 1>(variant, g, st);
     return b_dtype == MI8_E4M3 ? launch_variant<1, 0>(variant, g, st) : launch_variant<1, 1>(variant, g, st);
+}
+
+extern "C" int mi8_gemm_splitk_suggest(int64_t M, int64_t N, int64_t K)
+{
+    if (M <= 0 || N <= 0 || K <= 0) return 1;
+    return suggested_splits(M, N, K);
+}
+
+extern "C" int64_t mi8_gemm_splitk_workspace_bytes(int64_t M, int64_t N, int splits)
+{
+    if (M <= 0 || N <= 0 || splits <= 0) return 0;
+    return (int64_t)splits * M * ((N + 3) / 4 * 4) * (int64_t)sizeof(float);
+}
+
+extern "C" int mi8_gemm_fp8_splitk(const void* a, int a_dtype, int64_t lda, const void* b, int b_dtype, int64_t ldb,
+                                   int64_t M, int64_t N, int64_t K, const float* sa, int sa_is_vector,
+                                   const float* sb, int sb_is_vector, void* out, int out_dtype, int64_t ldc,
+                                   int splits, void* workspace, int64_t workspace_bytes, void* stream)
+{
+    MI8_REQUIRE(a && b && sa && sb && out && workspace, MI8_ERR_ARG, "mi8_gemm_fp8_splitk: null pointer");
+    MI8_REQUIRE((a_dtype == MI8_E4M3 || a_dtype == MI8_E5M2) && (b_dtype == MI8_E4M3 || b_dtype == MI8_E5M2),
+                MI8_ERR_ARG, "mi8_gemm_fp8_splitk: unknown fp8 dtype");
+    MI8_REQUIRE(M > 0 && N > 0 && K > 0, MI8_ERR_ARG, "mi8_gemm_fp8_splitk: empty problem %lld x %lld x %lld",
+                (long long)M, (long long)N, (long long)K);
+    MI8_REQUIRE(K % 16 == 0 && lda % 16 == 0 && ldb % 16 == 0 && lda >= K && ldb >= K, MI8_ERR_UNSUPPORTED,
+                "mi8_gemm_fp8_splitk: K (%lld), lda (%lld), ldb (%lld) must be multiples of 16 with lda, ldb >= K",
+                (long long)K, (long long)lda, (long long)ldb);
+    MI8_REQUIRE(ldc >= N, MI8_ERR_UNSUPPORTED, "mi8_gemm_fp8_splitk: ldc (%lld) < N (%lld)", (long long)ldc,
+                (long long)N);
+    MI8_REQUIRE(aligned16(a) && aligned16(b) && aligned16(workspace), MI8_ERR_UNSUPPORTED,
+                "mi8_gemm_fp8_splitk: operands and workspace must be 16-byte aligned");
+    MI8_REQUIRE(M * lda < (int64_t)1 << 32 && N * ldb < (int64_t)1 << 32 && M < (1 << 30) && N < (1 << 30) &&
+                    K < (1 << 30),
+                MI8_ERR_UNSUPPORTED, "mi8_gemm_fp8_splitk: operand larger than 4 GiB");
+    MI8_REQUIRE(out_dtype == MI8_BF16 || out_dtype == MI8_F32, MI8_ERR_ARG,
+                "mi8_gemm_fp8_splitk: unknown output dtype %d", out_dtype);
+    const int64_t steps = (K + BK - 1) / BK;
+    MI8_REQUIRE(splits >= 1 && splits <= 64 && splits <= steps, MI8_ERR_ARG,
+                "mi8_gemm_fp8_splitk: splits (%d) must be in 1..min(64, K steps = %lld)", splits, (long long)steps);
+    const int64_t per = (steps + splits - 1) / splits;
+    const int used = (int)((steps + per - 1) / per);  // slices that are not empty
+    MI8_REQUIRE(workspace_bytes >= mi8_gemm_splitk_workspace_bytes(M, N, used), MI8_ERR_ARG,
+                "mi8_gemm_fp8_splitk: workspace of %lld bytes, %lld needed", (long long)workspace_bytes,
+                (long long)mi8_gemm_splitk_workspace_bytes(M, N, used));
+    SplitArgs s{};
+    s.g = GemmArgs{(const uint8_t*)a, (const uint8_t*)b, out, out_dtype == MI8_F32 ? 1 : 0, lda, ldb, ldc, (int)M,
+                   (int)N, (int)K, sa, sb, sa_is_vector ? 1 : 0, sb_is_vector ? 1 : 0,
+                   (int)((M + kSplitTile - 1) / kSplitTile), (int)((N + kSplitTile - 1) / kSplitTile)};
+    s.planes = (float*)workspace;
+    s.ld_plane = (N + 3) / 4 * 4;
+    s.steps_per_split = (int)per;
+    s.splits = used;
+    hipStream_t st = (hipStream_t)stream;
+    if (a_dtype == MI8_E4M3)
+        return b_dtype == MI8_E4M3 ? launch_splitk_typed<0, 0>(s, st) : launch_splitk_typed<0, 1>(s, st);
+    return b_dtype == MI8_E4M3 ? launch_splitk_typed<1, 0>(s, st) : launch_splitk_typed<1, 1>(s, st);
 }

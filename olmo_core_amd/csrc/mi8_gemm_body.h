@@ -142,9 +142,9 @@ __device__ __forceinline__ void gemm_tile_body(const GemmArgs& g, const int m0, 
     for (int j = 0; j < TN; ++j) {
         const int col = n0 + wn * WTN + j * 32 + l32;
         col_ok[j] = col < g.N;
-        isb[j] = g.sb_vec ? (col_ok[j] ? __builtin_amdgcn_rcpf(g.sb[col]) : 0.0f) : 1.0f / g.sb[0];
+        isb[j] = g.sb_vec ? (col_ok[j] ? __builtin_amdgcn_rcpf(g.sb[col]) : 0.0f) : g.sb ? 1.0f / g.sb[0] : 1.0f;
     }
-    const float isa_scalar = g.sa_vec ? 0.0f : 1.0f / g.sa[0];
+    const float isa_scalar = g.sa_vec ? 0.0f : g.sa ? 1.0f / g.sa[0] : 1.0f;  // (null: the raw sums are wanted)
 #pragma unroll
     for (int i = 0; i < TM; ++i) {
 #pragma unroll

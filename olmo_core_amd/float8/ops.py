@@ -212,10 +212,15 @@ def gemm_fp8(
     k: Optional[int] = None,
     out_dtype: torch.dtype = torch.bfloat16,
     variant: int = -1,
+    out: Optional[torch.Tensor] = None,
+    splits: int = -1,
 ) -> torch.Tensor:
     """
     ``out[M, N] = (a[M, :k] @ b[N, :k].T) / sa / sb`` with fp32 accumulation on the fp8 matrix cores.
     ``a`` and ``b`` are fp8 tensors whose rows are K-contiguous; ``sa`` / ``sb`` hold one scale or one per row.
+    ``out``: an ``[M, N]`` tensor of ``out_dtype`` with contiguous rows (any row pitch) to write into.
+    ``splits``: slices of K summed separately and added afterwards (for problems with few output tiles);
+    -1 lets the library decide from the shape, 1 forbids splitting; a forced ``variant`` is never split.
     """
     _require_gpu(a, "gemm_fp8")
     if a.dim() != 2 or b.dim() != 2 or a.stride(1) != 1 or b.stride(1) != 1:
@@ -228,20 +233,42 @@ def gemm_fp8(
     K = min(a.shape[1], b.shape[1]) if k is None else k
     if sa.numel() not in (1, M) or sb.numel() not in (1, N):
         raise ValueError(f"gemm_fp8: scale sizes {sa.numel()}, {sb.numel()} do not match M={M}, N={N}")
-    out = torch.empty((M, N), dtype=out_dtype, device=a.device)
+    if out is None:
+        out = torch.empty((M, N), dtype=out_dtype, device=a.device)
+    elif tuple(out.shape) != (M, N) or out.dtype != out_dtype or out.stride(1) != 1 or out.device != a.device:
+        raise ValueError(f"gemm_fp8: out must be a [{M}, {N}] {out_dtype} tensor with contiguous rows on {a.device}")
     sink = GEMM_EVENT_SINK
     if sink is not None:
         ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         ev0.record()
-    _C.check(
-        _C.lib().mi8_gemm_fp8(
-            a.data_ptr(), _FP8_CODE[a.dtype], a.stride(0), b.data_ptr(), _FP8_CODE[b.dtype], b.stride(0), M, N, K,
-            sa.data_ptr(), int(sa.numel() != 1),
-            sb.data_ptr(), int(sb.numel() != 1),
-            out.data_ptr(), _HP_CODE[out_dtype], out.stride(0), variant, _stream(a),
-        ),
-        "mi8_gemm_fp8",
-    )
+    L = _C.lib()
+    if variant >= 0:
+        splits = 1
+    elif splits < 0:
+        splits = L.mi8_gemm_splitk_suggest(M, N, K)
+    if splits > 1:
+        # the planes come from torch's caching allocator: reuse is ordered on the stream like any other tensor
+        planes = torch.empty(L.mi8_gemm_splitk_workspace_bytes(M, N, splits), dtype=torch.uint8, device=a.device)
+        _C.check(
+            L.mi8_gemm_fp8_splitk(
+                a.data_ptr(), _FP8_CODE[a.dtype], a.stride(0), b.data_ptr(), _FP8_CODE[b.dtype], b.stride(0), M, N, K,
+                sa.data_ptr(), int(sa.numel() != 1),
+                sb.data_ptr(), int(sb.numel() != 1),
+                out.data_ptr(), _HP_CODE[out_dtype], out.stride(0), splits, planes.data_ptr(), planes.numel(),
+                _stream(a),
+            ),
+            "mi8_gemm_fp8_splitk",
+        )
+    else:
+        _C.check(
+            L.mi8_gemm_fp8(
+                a.data_ptr(), _FP8_CODE[a.dtype], a.stride(0), b.data_ptr(), _FP8_CODE[b.dtype], b.stride(0), M, N, K,
+                sa.data_ptr(), int(sa.numel() != 1),
+                sb.data_ptr(), int(sb.numel() != 1),
+                out.data_ptr(), _HP_CODE[out_dtype], out.stride(0), variant, _stream(a),
+            ),
+            "mi8_gemm_fp8",
+        )
     if sink is not None:
         ev1.record()
         sink.append((ev0, ev1, (M, N, K)))

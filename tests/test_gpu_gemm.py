@@ -23,7 +23,7 @@ def _gemm(a, sa, b, sb, variant, **kw):
     try:
         return ops.gemm_fp8(a, sa, b, sb, variant=variant, **kw)
     except MI8KernelError as e:
-        if "direct-to-LDS variant needs" in str(e):
+        if "direct-to-LDS variant needs" in str(e) or "few-rows variant takes" in str(e):
             return None
         raise
 
@@ -34,7 +34,9 @@ def _int_operand(shape, seed, dtype):
 
 
 EXACT_SHAPES = [(32, 32, 64), (1, 16, 16), (33, 48, 144), (256, 256, 128), (300, 272, 1040), (257, 513, 4096), (512, 768, 16),
-                (264, 520, 384), (256, 256, 256), (1024, 768, 1152), (2304, 2816, 128)]
+                (264, 520, 384), (256, 256, 256), (1024, 768, 1152), (2304, 2816, 128),
+                # a few rows of A: the kernel that streams B once (K split over eight waves, ragged N and K)
+                (1, 4096, 4096), (7, 1000, 2064), (16, 24, 16), (17, 40, 1040), (48, 1032, 4096), (64, 528, 11008)]
 
 
 @pytest.mark.parametrize("mnk", EXACT_SHAPES, ids=lambda s: "x".join(map(str, s)))
@@ -53,6 +55,71 @@ def test_integer_operands_exact(dev, mnk):
             if out is None:
                 continue
             assert torch.equal(out.cpu(), ref), f"variant {ops.gemm_variants()[v]} {da} x {db}: max diff {(out.cpu() - ref).abs().max()}"
+
+
+@pytest.mark.parametrize("M", [1, 5, 16, 31, 64])
+def test_few_rows_scales_and_outputs(dev, M):
+    """The default route for M <= 64: every mix of single scales and scale vectors, both output types, padded row
+    pitches; integer operands and power-of-two scales make the expected result exact."""
+    N, K, lda, ldb, ldc = 200, 400, 448, 416, 208
+    g = torch.Generator().manual_seed(40 + M)
+    a = torch.zeros(M, lda)
+    a[:, :K] = torch.randint(-2, 3, (M, K), generator=g).float()
+    a[:, K:] = 3.0  # bytes past K must not be read into the sum
+    b = torch.zeros(N, ldb)
+    b[:, :K] = torch.randint(-2, 3, (N, K), generator=g).float()
+    b[:, K:] = 3.0
+    ref = a[:, :K] @ b[:, :K].t()
+    aq, bq = a.to(E5M2).to(dev)[:, :K], b.to(E4M3).to(dev)[:, :K]
+    sa_v = (2.0 ** torch.randint(-3, 4, (M,), generator=g).float())
+    sb_v = (2.0 ** torch.randint(-3, 4, (N,), generator=g).float())
+    for sa, sb in ((torch.tensor([4.0]), torch.tensor([0.5])), (sa_v, sb_v), (sa_v, torch.tensor([2.0])),
+                   (torch.tensor([0.25]), sb_v)):
+        want = ref / (sa[:, None] if sa.numel() > 1 else sa) / (sb[None, :] if sb.numel() > 1 else sb)
+        for dt in (torch.float32, torch.bfloat16):
+            out = torch.full((M, ldc), 7.0, device=dev, dtype=dt)
+            res = ops.gemm_fp8(aq, sa.to(dev), bq, sb.to(dev), out_dtype=dt, out=out[:, :N])
+            assert res.data_ptr() == out.data_ptr()
+            assert torch.equal(out[:, :N].float().cpu(), want.to(dt).float())
+            assert bool((out[:, N:] == 7.0).all())  # nothing stored past column N
+
+
+@pytest.mark.parametrize("mnk", [(100, 200, 1040), (257, 130, 4096), (64, 72, 256), (130, 1000, 2048)],
+                         ids=lambda s: "x".join(map(str, s)))
+@pytest.mark.parametrize("splits", [2, 3, 8])
+def test_split_k_exact(dev, mnk, splits):
+    """K cut into slices that are summed separately and added in slice order: integer operands make every slice
+    and their sum exact, so a slice that is dropped, counted twice or cut at the wrong byte changes the result.
+    Scale vectors of powers of two, both output types, an output with padded rows."""
+    M, N, K = mnk
+    splits = min(splits, (K + 127) // 128)
+    g = torch.Generator().manual_seed(M + splits)
+    a, b = _int_operand((M, K), 11, E5M2), _int_operand((N, K), 12, E4M3)
+    sa = (2.0 ** torch.randint(-3, 4, (M,), generator=g).float())
+    sb = (2.0 ** torch.randint(-3, 4, (N,), generator=g).float())
+    ref = (a.float() @ b.float().t())
+    for sa_t, sb_t in ((torch.ones(1), torch.ones(1)), (sa, sb)):
+        want = ref / (sa_t[:, None] if sa_t.numel() > 1 else sa_t) / (sb_t[None, :] if sb_t.numel() > 1 else sb_t)
+        for dt in (torch.float32, torch.bfloat16):
+            out = torch.full((M, N + 8), 7.0, device=dev, dtype=dt)
+            ops.gemm_fp8(a.to(dev), sa_t.to(dev), b.to(dev), sb_t.to(dev), out_dtype=dt, out=out[:, :N], splits=splits)
+            assert torch.equal(out[:, :N].float().cpu(), want.to(dt).float()), (dt, sa_t.numel())
+            assert bool((out[:, N:] == 7.0).all())
+    # the library's own choice for the shape gives the same numbers
+    auto = ops.gemm_fp8(a.to(dev), sa.to(dev), b.to(dev), sb.to(dev), out_dtype=torch.float32)
+    assert torch.equal(auto.cpu(), ref / sa[:, None] / sb[None, :])
+
+
+def test_split_k_matches_single_pass_on_real_data(dev):
+    """Random operands: the sliced sum differs from the single-pass sum only by fp32 summation order."""
+    M, N, K = 384, 1024, 4096
+    a, b = seeded((M, K), 5).to(E4M3).to(dev), seeded((N, K), 6).to(E4M3).to(dev)
+    one = torch.ones(1, device=dev)
+    whole = ops.gemm_fp8(a, one, b, one, out_dtype=torch.float32, splits=1)
+    cut = ops.gemm_fp8(a, one, b, one, out_dtype=torch.float32, splits=8)
+    again = ops.gemm_fp8(a, one, b, one, out_dtype=torch.float32, splits=8)
+    assert torch.equal(cut, again)  # fixed summation order
+    assert float((cut - whole).abs().max()) <= 1e-4 * float(whole.abs().max())
 
 
 def test_integer_operands_exact_padded_pitch(dev):
@@ -217,3 +284,14 @@ def test_argument_errors(dev):
         ops.gemm_fp8(a.view(torch.uint8), one, a, one)
     with pytest.raises(ValueError):
         ops.gemm_fp8(torch.zeros(16, 32, dtype=E4M3, device=dev), torch.ones(3, device=dev), a, one)
+    b = torch.zeros(16, 256, dtype=E4M3, device=dev)
+    with pytest.raises(MI8KernelError, match="splits"):
+        ops.gemm_fp8(b, one, b, one, splits=3)  # more slices than 128-byte K steps
+    L = ops._C.lib()
+    assert L.mi8_gemm_splitk_workspace_bytes(100, 30, 4) == 4 * 100 * 32 * 4
+    assert L.mi8_gemm_splitk_suggest(16384, 11008, 4096) == 1 and L.mi8_gemm_splitk_suggest(256, 4096, 11008) > 1
+    small = torch.empty(64, dtype=torch.uint8, device=dev)
+    out = torch.empty(16, 16, dtype=torch.bfloat16, device=dev)
+    rc = L.mi8_gemm_fp8_splitk(b.data_ptr(), 0, 256, b.data_ptr(), 0, 256, 16, 16, 256, one.data_ptr(), 0, one.data_ptr(), 0,
+                               out.data_ptr(), 0, 16, 2, small.data_ptr(), small.numel(), 0)
+    assert rc != 0 and b"workspace" in L.mi8_last_error()
