@@ -232,10 +232,14 @@ def float8_linear_function(
         raise ValueError(f"float8 linear: input features {K} do not match weight {tuple(weight.shape)}")
     x2 = x.reshape(-1, K)
     cfg_id = getattr(config, "_compiled_id", -1)
-    if torch.compiler.is_compiling() and cfg_id >= 0:
+    compiling = torch.compiler.is_compiling()
+    if compiling and cfg_id >= 0:
         from . import compiled
 
         y = compiled.linear(x2, weight, cfg_id, weight_scale)
+    elif not compiling and not (torch.is_grad_enabled() and (x2.requires_grad or weight.requires_grad)):
+        # nothing to differentiate (evaluation, generation): no autograd node, nothing kept for a backward
+        y = _forward_impl(x2, weight, config, weight_scale, False, False, weight_ops)[0]
     else:  # eager, or a config no module registered: a graph break
         y = _eager_matmul(x2, weight, config, weight_scale, weight_ops)
     return y.reshape(*x.shape[:-1], weight.shape[0])

@@ -353,3 +353,36 @@ def test_kept_weight_operands(dev, monkeypatch):
         for x in xs:
             assert torch.equal(kept["proj"](kept["ff"](x)), plain["proj"](plain["ff"](x)))
     assert len(casts) == 8
+
+
+@pytest.mark.parametrize("tokens", [16, 300], ids=["few_rows", "split_k"])
+def test_forward_replays_from_a_captured_graph(dev, tokens):
+    """A generation loop captures one step in a HIP graph and replays it: every launch of the forward (casts,
+    SwiGLU, the few-rows / split-K / tiled GEMMs) goes to the capturing stream, nothing synchronises or reads
+    back, so each replay on new input equals the eager result bit for bit.  Eager work runs between replays."""
+    from olmo_core_amd.nn import FeedForward
+
+    torch.manual_seed(11)
+    model = nn.Sequential(
+        FeedForward(d_model=1024, hidden_size=2048, bias=False, dtype=torch.bfloat16),
+        nn.Linear(1024, 512, bias=True, dtype=torch.bfloat16),
+    ).to(dev)
+    Float8Config(ao=AOFloat8LinearConfig.recommended()).apply_float8_linear(model)
+    x_static = torch.randn(tokens, 1024, device=dev, dtype=torch.bfloat16)
+    with torch.no_grad():
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            for _ in range(3):  # first calls configure kernels and fill the kept weight copies
+                model(x_static)
+        torch.cuda.current_stream().wait_stream(side)
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            y_static = model(x_static)
+        for i in range(4):
+            x_new = torch.randn(tokens, 1024, device=dev, dtype=torch.bfloat16) * (i + 1)
+            x_static.copy_(x_new)
+            graph.replay()
+            torch.cuda.synchronize()
+            eager = model(x_new)
+            assert torch.equal(y_static, eager), i
