@@ -166,6 +166,16 @@ __device__ __forceinline__ void tile_cast_body(const void* x, int64_t row_end, i
             HpVec<HP>::load8(xb + (r * cols + c8) * HpVec<HP>::kBytes, ok, f[it][j]);
         }
 
+    // the rows' own scales, read with the data (a read placed between the stores below would wait for them)
+    float srow[2][4];
+#pragma unroll
+    for (int it = 0; it < 2; ++it)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int64_t r = row0 + 32 * wave + 16 * it + 4 * g + j;
+            srow[it][j] = (out_r && r < row_end) ? row_scale[r] : 0.0f;
+        }
+
 #pragma unroll
     for (int it = 0; it < 2; ++it) {
         uint32_t lo[4], hi[4];
@@ -179,7 +189,7 @@ __device__ __forceinline__ void tile_cast_body(const void* x, int64_t row_end, i
             if (!ok) lo[j] = hi[j] = 0;  // padding is zero bytes whatever the scale is (0 * NaN is NaN)
             if (out && ok) *reinterpret_cast<uint2*>(out + r * ld_out + c8) = make_uint2(lo[j], hi[j]);
             if (out_r && ok) {  // the same values quantised with the row's own scale
-                const float sr = row_scale[r];
+                const float sr = srow[it][j];
                 const uint32_t rl = quant4<FP8, SW>(v[0], v[1], v[2], v[3], sr, sr, sr, sr);
                 const uint32_t rh = quant4<FP8, SW>(v[4], v[5], v[6], v[7], sr, sr, sr, sr);
                 *reinterpret_cast<uint2*>(out_r + r * ld_r + c8) = make_uint2(rl, rh);
@@ -404,23 +414,75 @@ struct GroupedCastArgs {
 // Tile p of the padded row space (128 rows each; group e owns ceil(m_e / 128) consecutive tiles) -> its group,
 // its rows [row0, row_end) in x (row_end = the group's end) and its destination column 128 p in out_t.
 // Sizes are clamped so that nothing past row T is ever read.
+__device__ __forceinline__ int64_t shfl64(int64_t v, int src)
+{
+    const int lo = __shfl((int)(uint32_t)v, src, 64), hi = __shfl((int)(v >> 32), src, 64);
+    return ((int64_t)hi << 32) | (uint32_t)lo;
+}
+__device__ __forceinline__ int64_t shfl_up64(int64_t v, int off)
+{
+    const int lo = __shfl_up((int)(uint32_t)v, off, 64), hi = __shfl_up((int)(v >> 32), off, 64);
+    return ((int64_t)hi << 32) | (uint32_t)lo;
+}
+
+// Every wave finds the tile's group on its own, 64 groups at a time: one coalesced load of the sizes, prefix sums
+// of rows and of tiles across the lanes, a ballot for the group whose tile range holds p.  (Walking the sizes one
+// by one cost 35 us per launch at 64 groups: every step waits for its own load.)  All lanes return the same
+// values.  Must be called by full waves in uniform control flow.
 __device__ __forceinline__ bool locate_padded_tile(const int64_t* sizes, int E, int64_t T, int p, int& e,
                                                    int64_t& row0, int64_t& row_end)
 {
-    int64_t rows_before = 0;
+    if (E <= 4) {  // a handful of groups (one: the dense two-product cast): walking them is cheaper than a scan
+        int64_t before = 0;
+        int tiles = 0;
+        for (e = 0; e < E; ++e) {
+            int64_t m = sizes[e];
+            m = m < 0 ? 0 : m;
+            m = before + m > T ? T - before : m;
+            const int t = (int)((m + kTile - 1) / kTile);
+            if (p < tiles + t) {
+                row0 = before + (int64_t)kTile * (p - tiles);
+                row_end = before + m;
+                return true;
+            }
+            tiles += t;
+            before += m;
+        }
+        return false;
+    }
+    const int lane = threadIdx.x & 63;
+    int64_t rows_before = 0;  // unclamped sum of the sizes of earlier chunks
     int tiles_before = 0;
-    for (e = 0; e < E; ++e) {
-        int64_t m = sizes[e];
+    for (int base = 0; base < E; base += 64) {
+        int64_t m = base + lane < E ? sizes[base + lane] : 0;
         m = m < 0 ? 0 : m;
-        m = (rows_before + m > T) ? T - rows_before : m;
-        const int t = (int)((m + kTile - 1) / kTile);
-        if (p < tiles_before + t) {
-            row0 = rows_before + (int64_t)kTile * (p - tiles_before);
-            row_end = rows_before + m;
+        int64_t incl = m;  // inclusive prefix sum over the chunk
+#pragma unroll
+        for (int off = 1; off < 64; off <<= 1) {
+            const int64_t t = shfl_up64(incl, off);
+            if (lane >= off) incl += t;
+        }
+        // a running sum clamped to T step by step equals the clamped running sum (sizes are not negative)
+        const int64_t end = rows_before + incl < T ? rows_before + incl : T;
+        const int64_t beg = rows_before + incl - m < T ? rows_before + incl - m : T;
+        const int t = (int)((end - beg + kTile - 1) / kTile);
+        int tincl = t;
+#pragma unroll
+        for (int off = 1; off < 64; off <<= 1) {
+            const int u = __shfl_up(tincl, off, 64);
+            if (lane >= off) tincl += u;
+        }
+        const int first = tiles_before + tincl - t;  // this group's first tile
+        const unsigned long long hit = __ballot(p >= first && p < first + t);
+        if (hit) {
+            const int src = __ffsll((long long)hit) - 1;
+            e = base + src;
+            row0 = shfl64(beg, src) + (int64_t)kTile * (p - __shfl(first, src, 64));
+            row_end = shfl64(end, src);
             return true;
         }
-        tiles_before += t;
-        rows_before += m;
+        rows_before += shfl64(incl, 63);
+        tiles_before += __shfl(tincl, 63, 64);
     }
     return false;
 }
