@@ -1,6 +1,7 @@
 // amax reductions and saturating float8 casts (tensorwise, per-row, per-column with transposed output).
 // All kernels are HBM-bound streaming kernels: 16-byte loads per lane, wave-shuffle reductions, an
 // LDS-staged byte transpose for the transposed copy.
+#include "mi8_groups.h"
 #include "mi8_swiglu.h"
 
 namespace mi8 {
@@ -414,21 +415,9 @@ struct GroupedCastArgs {
 // Tile p of the padded row space (128 rows each; group e owns ceil(m_e / 128) consecutive tiles) -> its group,
 // its rows [row0, row_end) in x (row_end = the group's end) and its destination column 128 p in out_t.
 // Sizes are clamped so that nothing past row T is ever read.
-__device__ __forceinline__ int64_t shfl64(int64_t v, int src)
-{
-    const int lo = __shfl((int)(uint32_t)v, src, 64), hi = __shfl((int)(v >> 32), src, 64);
-    return ((int64_t)hi << 32) | (uint32_t)lo;
-}
-__device__ __forceinline__ int64_t shfl_up64(int64_t v, int off)
-{
-    const int lo = __shfl_up((int)(uint32_t)v, off, 64), hi = __shfl_up((int)(v >> 32), off, 64);
-    return ((int64_t)hi << 32) | (uint32_t)lo;
-}
-
-// Every wave finds the tile's group on its own, 64 groups at a time: one coalesced load of the sizes, prefix sums
-// of rows and of tiles across the lanes, a ballot for the group whose tile range holds p.  (Walking the sizes one
-// by one cost 35 us per launch at 64 groups: every step waits for its own load.)  All lanes return the same
-// values.  Must be called by full waves in uniform control flow.
+// The search is a wave-wide prefix scan over the sizes (gemm::locate_group); walking the sizes one by one cost
+// 35 us per launch at 64 groups, every step waiting for its own load.  All lanes return the same values; must be
+// called by full waves in uniform control flow.
 __device__ __forceinline__ bool locate_padded_tile(const int64_t* sizes, int E, int64_t T, int p, int& e,
                                                    int64_t& row0, int64_t& row_end)
 {
@@ -450,41 +439,12 @@ __device__ __forceinline__ bool locate_padded_tile(const int64_t* sizes, int E, 
         }
         return false;
     }
-    const int lane = threadIdx.x & 63;
-    int64_t rows_before = 0;  // unclamped sum of the sizes of earlier chunks
-    int tiles_before = 0;
-    for (int base = 0; base < E; base += 64) {
-        int64_t m = base + lane < E ? sizes[base + lane] : 0;
-        m = m < 0 ? 0 : m;
-        int64_t incl = m;  // inclusive prefix sum over the chunk
-#pragma unroll
-        for (int off = 1; off < 64; off <<= 1) {
-            const int64_t t = shfl_up64(incl, off);
-            if (lane >= off) incl += t;
-        }
-        // a running sum clamped to T step by step equals the clamped running sum (sizes are not negative)
-        const int64_t end = rows_before + incl < T ? rows_before + incl : T;
-        const int64_t beg = rows_before + incl - m < T ? rows_before + incl - m : T;
-        const int t = (int)((end - beg + kTile - 1) / kTile);
-        int tincl = t;
-#pragma unroll
-        for (int off = 1; off < 64; off <<= 1) {
-            const int u = __shfl_up(tincl, off, 64);
-            if (lane >= off) tincl += u;
-        }
-        const int first = tiles_before + tincl - t;  // this group's first tile
-        const unsigned long long hit = __ballot(p >= first && p < first + t);
-        if (hit) {
-            const int src = __ffsll((long long)hit) - 1;
-            e = base + src;
-            row0 = shfl64(beg, src) + (int64_t)kTile * (p - __shfl(first, src, 64));
-            row_end = shfl64(end, src);
-            return true;
-        }
-        rows_before += shfl64(incl, 63);
-        tiles_before += __shfl(tincl, 63, 64);
-    }
-    return false;
+    const gemm::GroupSpan g = gemm::locate_group<kTile, true>(sizes, E, T, p);
+    if (g.e >= E) return false;
+    e = g.e;
+    row0 = g.rows_before + (int64_t)kTile * (p - g.units_before);
+    row_end = g.rows_before + g.m;
+    return true;
 }
 
 template <int HP>
