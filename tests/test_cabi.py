@@ -37,6 +37,18 @@ def test_host_only_entry_points():
     assert L.mi8_amax_slots_for(1) == 1
     assert L.mi8_amax_slots_for(1 << 40) == _C.AMAX_SLOTS
     assert L.mi8_colamax_workspace_slots(16384, 4096) % 4096 == 0
+    # split-K planning: large problems are not split, a few rows go to the kernel that streams the weight once,
+    # few output tiles with a long K are cut so that no slice is empty and each keeps at least four K steps
+    assert L.mi8_gemm_splitk_suggest(16384, 11008, 4096) == 1
+    assert L.mi8_gemm_splitk_suggest(16, 4096, 4096) == 1
+    assert L.mi8_gemm_splitk_suggest(256, 256, 512) == 1
+    for (m, n, k) in ((256, 4096, 11008), (100, 200, 1040), (384, 1024, 4096), (64, 11008, 4096)):
+        s = L.mi8_gemm_splitk_suggest(m, n, k)
+        steps = -(-k // 128)
+        per = -(-steps // s)
+        assert 2 <= s <= 32 and per >= 4 - 1 and (s - 1) * per < steps, (m, n, k, s)
+    assert L.mi8_gemm_splitk_workspace_bytes(100, 30, 4) == 4 * 100 * 32 * 4
+    assert L.mi8_gemm_splitk_workspace_bytes(0, 30, 4) == 0
 
 
 def test_argument_validation_happens_before_any_gpu_call():
@@ -44,5 +56,6 @@ def test_argument_validation_happens_before_any_gpu_call():
     assert L.mi8_cast_rowwise(None, 0, 4, 16, 0, 0, None, 16, None, None) == -1
     assert "null" in _C.last_error()
     assert L.mi8_gemm_fp8(None, 0, 16, None, 0, 16, 1, 1, 16, None, 0, None, 0, None, 0, 16, -1, None) == -1
+    assert L.mi8_gemm_fp8_splitk(None, 0, 16, None, 0, 16, 1, 1, 16, None, 0, None, 0, None, 0, 16, 2, None, 0, None) == -1
     with pytest.raises(Exception):
         _C.check(-2, "x")

@@ -264,3 +264,18 @@ def test_no_cpu_path():
     Float8Config().apply_float8_linear(m, modules_to_ignore={"lm_head"})
     with pytest.raises(RuntimeError, match="no CPU path"):
         m.blocks[0]["w1"](torch.randn(4, 32))
+
+
+def test_kept_weight_operands_need_the_switch_and_a_gpu_weight():
+    """Float8Linear.weight_operands(): nothing is kept without enable_fsdp_float8_all_gather, and a weight that
+    is not on the GPU is never quantised ahead of the forward (which then raises: there is no CPU path)."""
+    import torch.nn as nn
+
+    from olmo_core_amd.float8 import AOFloat8LinearConfig, Float8Config
+    from olmo_core_amd.float8.linear import Float8Linear
+
+    for cfg in (AOFloat8LinearConfig(), AOFloat8LinearConfig.recommended()):
+        model = nn.Sequential(nn.Linear(32, 48, bias=False))
+        Float8Config(ao=cfg).apply_float8_linear(model)
+        assert isinstance(model[0], Float8Linear)
+        assert model[0].weight_operands() is None
