@@ -122,7 +122,7 @@ int suggested_splits(int64_t M, int64_t N, int64_t K)
 {
     const int64_t tiles = ((M + kSplitTile - 1) / kSplitTile) * ((N + kSplitTile - 1) / kSplitTile);
     const int64_t steps = (K + BK - 1) / BK;
-    if (M <= 16 || tiles >= 256 || steps < 8) return 1;  // (up to 16 rows: the few-rows kernel reads B once)
+    if (M <= 16 || tiles > 256 || steps < 8) return 1;  // (up to 16 rows: the few-rows kernel reads B once)
     int64_t s = 512 / tiles;
     if (s > steps / 4) s = steps / 4;
     if (s > 32) s = 32;

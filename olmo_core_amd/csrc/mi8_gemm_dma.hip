@@ -300,7 +300,8 @@ int launch(GemmArgs& g, hipStream_t st)
     g.tiles_n = (g.N + BN - 1) / BN;
     const int total = g.tiles_m * g.tiles_n;
     int blocks = num_cus();
-    if (blocks > total) blocks = total;
+    const int wanted = (total + 7) / 8 * 8;  // every XCD gets as many workgroups as it has tiles
+    if (blocks > wanted) blocks = wanted;
     hipLaunchKernelGGL(kern, dim3(blocks), dim3(NT), LDS_BYTES, st, g);
     return launch_status("mi8_gemm_fp8(direct-to-LDS)");
 }

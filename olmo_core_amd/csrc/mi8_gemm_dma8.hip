@@ -432,8 +432,12 @@ int launch(const Problem& pb, int max_tiles, bool persistent, hipStream_t st)
         }
         configured = true;
     }
+    // Persistent: one workgroup per compute unit, or, for fewer tiles, as many as the tiles need - rounded up to
+    // a multiple of 8, because every XCD takes an eighth of the tiles (rounded up) and needs that many
+    // workgroups to finish in one round (43 tiles on 43 workgroups: XCDs with 5 workgroups for 6 tiles).
     int blocks = persistent ? num_cus() : max_tiles;
-    if (blocks > max_tiles) blocks = max_tiles;
+    const int wanted = persistent ? (max_tiles + 7) / 8 * 8 : max_tiles;
+    if (blocks > wanted) blocks = wanted;
     hipLaunchKernelGGL(kern, dim3(blocks), dim3(Layout<WN>::kThreads), LDS_BYTES, st, pb);
     return launch_status("mi8 direct-to-LDS GEMM (8 waves)");
 }
