@@ -156,6 +156,31 @@ def run_other_config(n, steps, warmup):
                       "pct_fp8_mfma_peak": round(100 * flops / ms / 1e9 / FP8_MFMA_PEAK_TFLOPS, 2), "steps": steps}), flush=True)
 
 
+def gemm_shapes(shapes, steps, warmup):
+    """One line per shape: a single e4m3 x e4m3 GEMM with bf16 output and single scales, the kernel chosen by the
+    library (few rows: the weight-streaming kernel; few tiles: split K; otherwise the tiled kernels)."""
+    from olmo_core_amd.float8 import ops
+
+    dev = torch.device("cuda:0")
+    one = torch.ones(1, device=dev)
+    g = torch.Generator().manual_seed(7)
+    for (m, n, k) in shapes:
+        a = torch.randn(m, k, generator=g).to(torch.float8_e4m3fn).to(dev)
+        b = torch.randn(n, k, generator=g).to(torch.float8_e4m3fn).to(dev)
+        for _ in range(warmup):
+            ops.gemm_fp8(a, one, b, one)
+        start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        start.record()
+        for _ in range(steps):
+            ops.gemm_fp8(a, one, b, one)
+        end.record()
+        torch.cuda.synchronize()
+        us = start.elapsed_time(end) / steps * 1e3
+        print(json.dumps({"gemm": f"{m}x{n}x{k}", "us_per_call": round(us, 2), "TFLOP/s": round(2.0 * m * n * k / us / 1e6, 1),
+                          "operand_GB/s": round((m * k + n * k + 2 * m * n) / us / 1e3, 1), "steps": steps}), flush=True)
+
+
 def traffic_probe():
     """Workload for the rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs: a plain 256 MiB device copy (the
     calibration: 268435456 bytes read and written), then the three GEMM shapes of the benchmark step and the
@@ -240,6 +265,8 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--config", type=int, default=2, help="benchmark configuration 1..5 (2 is the headline line)")
     ap.add_argument("--traffic-probe", action="store_true", help="workload for the FETCH_SIZE/WRITE_SIZE counter runs")
+    ap.add_argument("--gemm", type=str, default=None, metavar="M,N,K[;M,N,K...]",
+                    help="time single scaled GEMMs of these shapes (library's choice of kernel) instead of a step")
     ns = ap.parse_args()
     if ns.gpus != 1:
         print("bench.py: this build measures the float8 linear path on ONE GPU; --gpus must be 1", file=sys.stderr)
@@ -252,6 +279,9 @@ def main():
 
     if ns.traffic_probe:
         traffic_probe()
+        return
+    if ns.gemm:
+        gemm_shapes([tuple(int(v) for v in part.split(",")) for part in ns.gemm.split(";")], ns.steps, ns.warmup)
         return
     if ns.config != 2:
         run_other_config(ns.config, ns.steps, ns.warmup)
