@@ -7,6 +7,11 @@
 // LDS stage layout: [row][128 bytes]; the 16-byte chunk c of row r sits at chunk position c ^ swz(r),
 // swz(r) = (r ^ (r >> 3)) & 7, so that the 16-byte fragment reads of 32 different rows spread over all banks
 // while the stores (8 lanes per row) stay contiguous.
+//
+// This file holds that general tile kernel (any M, N; K % 16 == 0; bf16 or fp32 output), its split-K form for
+// problems with few output tiles, and the entry points, which pick a kernel by shape: the persistent direct-to-LDS
+// kernels of mi8_gemm_m16.hip / mi8_gemm_dma8.hip / mi8_gemm_dma.hip for large problems, the weight-streaming
+// kernel of mi8_gemm_skinny.hip for a few rows of A.
 #include "mi8_gemm_body.h"
 
 namespace mi8 {

@@ -24,11 +24,7 @@ __device__ __forceinline__ uint32_t pack_bf16(float lo, float hi)
 // e^-x overflowing to +inf gives 0, underflowing to 0 gives 1, NaN stays NaN.
 __device__ __forceinline__ float sigmoid_f32(float x)
 {
-#ifdef MI8_SLOW_SIGMOID
-    return 1.0f / (1.0f + expf(-x));
-#else
     return __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(x * -1.44269504088896341f));
-#endif
 }
 
 __device__ __forceinline__ void unpack8(uint4 v, float (&f)[8])
