@@ -89,7 +89,9 @@ int mi8_multi_tensor_scales(const void* const* ptrs, const int64_t* numels, int3
 /* Saturating cast of x[rows, cols] with one scale for the whole tensor.
  *   scale source: if slots != NULL the scale is reduced from slots[0..n_slots) exactly as
  *   mi8_scale_from_partials does (and written to scale_out[0] if scale_out != NULL);
- *   otherwise it is read from scale_in[0] (device float32).
+ *   otherwise, if scale_in != NULL, it is read from scale_in[0] (device float32);
+ *   with neither (tensors of at most 65536 elements, row-major output only: the activations of a generation
+ *   step) one workgroup takes the amax, derives the scale and converts in a single launch.
  *   out   (may be NULL): fp8 [rows, ld_out], row-major with row pitch ld_out >= cols, ld_out % 16 == 0;
  *                        bytes cols..ld_out-1 of a row are not touched.
  *   out_t (may be NULL): fp8 [cols, ld_t], the transposed copy; ld_t >= rows, ld_t % 16 == 0; columns

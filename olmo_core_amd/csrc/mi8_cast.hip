@@ -811,6 +811,64 @@ int64_t colamax_rows_per_chunk(int64_t rows)
     return rpc < 256 ? 256 : rpc;
 }
 
+// ---- small tensors: amax, scale and cast in one launch --------------------------------------------------
+// A few rows of activations (a generation step) are cast by ONE workgroup: every lane keeps its share of the
+// tensor in registers between the amax reduction and the conversion, so the tensorwise cast is one launch
+// instead of two and reads x once.  Same helpers as the two-kernel route: same scale, same bytes.
+constexpr int kSmallThreads = 1024;
+constexpr int kSmallVecs = 8;  // 8-element groups per lane
+constexpr int64_t kSmallCastElems = (int64_t)kSmallThreads * kSmallVecs * 8;
+
+template <int HP, int FP8, bool SW>
+__global__ __launch_bounds__(kSmallThreads) void small_cast_kernel(const void* __restrict__ x, int64_t rows,
+                                                                   int64_t cols, bool pow2, uint8_t* __restrict__ out,
+                                                                   int64_t ld_out, float* __restrict__ scale_out)
+{
+    __shared__ uint32_t smem[kSmallThreads / 64];
+    const int tid = threadIdx.x;
+    const int64_t groups = rows * cols / 8;  // cols % 16 == 0
+    const char* xb = reinterpret_cast<const char*>(x);
+    float f[kSmallVecs][8];
+    uint32_t m = 0;
+#pragma unroll
+    for (int i = 0; i < kSmallVecs; ++i) {
+        const int64_t g = tid + (int64_t)kSmallThreads * i;
+        HpVec<HP>::load8(xb + g * 8 * HpVec<HP>::kBytes, g < groups, f[i]);  // zeros past the end
+        m = umax32(m, absmax8_bits(f[i]));
+    }
+    m = wave_umax(m);
+    if ((tid & 63) == 0) smem[tid >> 6] = m;
+    __syncthreads();
+    m = 0;
+#pragma unroll
+    for (int w = 0; w < kSmallThreads / 64; ++w) m = umax32(m, smem[w]);
+    const float s = scale_from_amax_bits<FP8>(m, pow2);  // every lane: same bits in, same bits out
+    if (tid == 0 && scale_out) scale_out[0] = s;
+#pragma unroll
+    for (int i = 0; i < kSmallVecs; ++i) {
+        const int64_t g = tid + (int64_t)kSmallThreads * i;
+        if (g >= groups) continue;
+        const int64_t e = g * 8, r = e / cols, c = e % cols;
+        const uint32_t lo = quant4<FP8, SW>(f[i][0], f[i][1], f[i][2], f[i][3], s, s, s, s);
+        const uint32_t hi = quant4<FP8, SW>(f[i][4], f[i][5], f[i][6], f[i][7], s, s, s, s);
+        *reinterpret_cast<uint2*>(out + r * ld_out + c) = make_uint2(lo, hi);
+    }
+}
+
+template <int HP>
+void launch_small_cast(int fp8_dtype, bool sw, const void* x, int64_t rows, int64_t cols, bool pow2, uint8_t* out,
+                       int64_t ld_out, float* scale_out, hipStream_t st)
+{
+    const dim3 grid(1), block(kSmallThreads);
+    if (fp8_dtype == MI8_E4M3) {
+        if (sw) hipLaunchKernelGGL((small_cast_kernel<HP, MI8_E4M3, true>), grid, block, 0, st, x, rows, cols, pow2, out, ld_out, scale_out);
+        else hipLaunchKernelGGL((small_cast_kernel<HP, MI8_E4M3, false>), grid, block, 0, st, x, rows, cols, pow2, out, ld_out, scale_out);
+    } else {
+        if (sw) hipLaunchKernelGGL((small_cast_kernel<HP, MI8_E5M2, true>), grid, block, 0, st, x, rows, cols, pow2, out, ld_out, scale_out);
+        else hipLaunchKernelGGL((small_cast_kernel<HP, MI8_E5M2, false>), grid, block, 0, st, x, rows, cols, pow2, out, ld_out, scale_out);
+    }
+}
+
 }  // namespace
 }  // namespace mi8
 
@@ -950,8 +1008,12 @@ extern "C" int mi8_cast_tensorwise(const void* x, int hp_dtype, int64_t rows, in
     MI8_REQUIRE(valid_hp(hp_dtype) && valid_fp8(fp8_dtype), MI8_ERR_ARG, "mi8_cast_tensorwise: unknown dtype");
     MI8_REQUIRE(rows > 0 && cols > 0, MI8_ERR_ARG, "mi8_cast_tensorwise: empty input (%lld x %lld)", (long long)rows,
                 (long long)cols);
-    MI8_REQUIRE((slots != nullptr) != (scale_in != nullptr), MI8_ERR_ARG,
-                "mi8_cast_tensorwise: give exactly one of slots / scale_in");
+    MI8_REQUIRE(!(slots && scale_in), MI8_ERR_ARG, "mi8_cast_tensorwise: give slots or scale_in, not both");
+    const bool fused_amax = !slots && !scale_in;  // small tensors: amax taken by the cast kernel itself
+    MI8_REQUIRE(!fused_amax || (rows * cols <= kSmallCastElems && out && !out_t), MI8_ERR_ARG,
+                "mi8_cast_tensorwise: without slots or scale_in the tensor may have at most %lld elements and only "
+                "the row-major output (%lld x %lld)",
+                (long long)kSmallCastElems, (long long)rows, (long long)cols);
     MI8_REQUIRE(!slots || (n_slots > 0 && n_slots <= MI8_AMAX_SLOTS), MI8_ERR_ARG,
                 "mi8_cast_tensorwise: n_slots %d out of range", n_slots);
     MI8_REQUIRE(cols % 16 == 0, MI8_ERR_UNSUPPORTED, "mi8_cast_tensorwise: cols (%lld) must be a multiple of 16",
@@ -964,6 +1026,14 @@ extern "C" int mi8_cast_tensorwise(const void* x, int hp_dtype, int64_t rows, in
     if (out_t)
         MI8_REQUIRE(ld_t >= rows && ld_t % 16 == 0, MI8_ERR_UNSUPPORTED,
                     "mi8_cast_tensorwise: ld_t (%lld) must be a multiple of 16 and at least rows", (long long)ld_t);
+    if (fused_amax) {
+        const bool sw = (flags & MI8_FLAG_SW_CVT) != 0, pow2 = (flags & MI8_FLAG_POW2_SCALE) != 0;
+        if (hp_dtype == MI8_BF16)
+            launch_small_cast<MI8_BF16>(fp8_dtype, sw, x, rows, cols, pow2, (uint8_t*)out, ld_out, scale_out, (hipStream_t)stream);
+        else
+            launch_small_cast<MI8_F32>(fp8_dtype, sw, x, rows, cols, pow2, (uint8_t*)out, ld_out, scale_out, (hipStream_t)stream);
+        return launch_status("mi8_cast_tensorwise");
+    }
     TileCastArgs a{x, rows, cols, slots, n_slots, scale_in, (flags & MI8_FLAG_POW2_SCALE) != 0,
                    (uint8_t*)out, ld_out, (uint8_t*)out_t, ld_t, scale_out};
     dispatch_tile_cast(hp_dtype, fp8_dtype, (flags & MI8_FLAG_SW_CVT) != 0, slots ? kScalarFromSlots : kScalarFromPtr,

@@ -59,6 +59,9 @@ def _hp2d(x: torch.Tensor, what: str) -> torch.Tensor:
     return x
 
 
+_SMALL_CAST = 65536  # elements up to which mi8_cast_tensorwise takes the amax itself
+
+
 def pad16(n: int) -> int:
     return (n + 15) // 16 * 16
 
@@ -151,7 +154,9 @@ def cast_tensorwise(
     x = _hp2d(x, "cast_tensorwise")
     rows, cols = x.shape
     dev = x.device
-    if scale is None and slots is None:
+    # small tensors with only the row-major copy: the cast kernel takes the amax itself (one launch)
+    fused_amax = scale is None and slots is None and want_rowmajor and not want_transposed and x.numel() <= _SMALL_CAST
+    if scale is None and slots is None and not fused_amax:
         slots = amax_partials(x)
     q = _operand((rows, cols), fp8_dtype, dev, pitch) if want_rowmajor else None
     q_t = _operand((cols, pad16(rows)), fp8_dtype, dev, pitch_t) if want_transposed else None
@@ -161,7 +166,8 @@ def cast_tensorwise(
     _C.check(
         _C.lib().mi8_cast_tensorwise(
             x.data_ptr(), _HP_CODE[x.dtype], rows, cols,
-            slots[0].data_ptr() if scale is None else None, slots[1] if scale is None else 0,
+            slots[0].data_ptr() if slots is not None and scale is None else None,
+            slots[1] if slots is not None and scale is None else 0,
             scale.data_ptr() if scale is not None else None,
             _FP8_CODE[fp8_dtype], _flags(pow2),
             q.data_ptr() if q is not None else None, q.stride(0) if q is not None else 0,

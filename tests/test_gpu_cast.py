@@ -69,6 +69,40 @@ def test_tensorwise_dynamic(dev, shape, fp8, pow2, cvt_mode):
     assert int(u8(q_t[:, rows:]).max() if q_t.shape[1] > rows else 0) == 0, "padding must be zero bytes"
 
 
+@pytest.mark.parametrize("shape", [(1, 16), (1, 4096), (7, 528), (16, 4096), (64, 1024), (33, 1040)],
+                         ids=lambda s: f"{s[0]}x{s[1]}")
+@pytest.mark.parametrize("fp8", [E4M3, E5M2], ids=["e4m3", "e5m2"])
+@pytest.mark.parametrize("pow2", [False, True], ids=["", "pow2"])
+def test_tensorwise_small_single_launch(dev, shape, fp8, pow2, cvt_mode):
+    """Up to 65536 elements with only the row-major copy wanted: the cast takes the amax itself (one launch).
+    Bytes and scale equal the oracle's and those of the two-kernel route (amax partials, then cast); float32
+    input, NaN, an all-zero tensor and a padded output pitch included."""
+    x = seeded(shape, seed=shape[0] * 13 + shape[1], std=0.7)
+    ref_q, ref_s = O.cast(x, fp8, O.TENSORWISE, None, pow2)
+    xd = x.to(dev)
+    q, q_t, s = ops.cast_tensorwise(xd, fp8, pow2=pow2)  # the single-launch route
+    assert q_t is None
+    assert_scale_equal(s, ref_s, "scale")
+    assert_bytes_equal(q, ref_q, what="row-major")
+    q2, _, s2 = ops.cast_tensorwise(xd, fp8, pow2=pow2, slots=ops.amax_partials(xd))  # the two-kernel route
+    assert torch.equal(u8(q), u8(q2)) and torch.equal(s, s2)
+    # float32 input and a wider output pitch
+    x32 = x.float() * 1.0009765625
+    ref_q32, ref_s32 = O.cast(x32, fp8, O.TENSORWISE, None, pow2)
+    q32, _, s32 = ops.cast_tensorwise(x32.to(dev), fp8, pow2=pow2, pitch=shape[1] + 32)
+    assert q32.stride(0) == shape[1] + 32
+    assert_scale_equal(s32, ref_s32, "scale (float32 input)")
+    assert_bytes_equal(q32, ref_q32, what="row-major (float32 input)")
+    # NaN and all zeros behave as on the two-kernel route
+    for special in (torch.zeros(shape, dtype=torch.bfloat16), x.clone()):
+        if special.abs().max() > 0:
+            special.view(-1)[special.numel() // 2] = float("nan")
+        sd = special.to(dev)
+        qa, _, sa = ops.cast_tensorwise(sd, fp8, pow2=pow2)
+        qb, _, sb = ops.cast_tensorwise(sd, fp8, pow2=pow2, slots=ops.amax_partials(sd))
+        assert torch.equal(u8(qa), u8(qb)) and torch.equal(sa.view(torch.int32), sb.view(torch.int32))
+
+
 @pytest.mark.parametrize("std", [0.02, 1e-3, 50.0, 1e-20])
 def test_tensorwise_magnitudes(dev, std):
     x = seeded((333, 528), seed=11, std=std)
