@@ -510,11 +510,11 @@ def cast_rows_and_colwise_t(
     [cols])``; ``q_t`` is zero beyond ``rows``.  Bytes and scales are those of the two separate casts.
     """
     x = _hp2d(x, "cast_rows_and_colwise_t")
-    rows = x.shape[0]
-    key = (rows, x.device)
-    sizes = _ONE_GROUP.get(key)
+    # one group that takes every row: the kernels clamp group sizes to the rows that exist, so one device-resident
+    # "all of them" serves every shape (no host-to-device copy per call, none at all after the first)
+    sizes = _ONE_GROUP.get(x.device)
     if sizes is None:
-        sizes = _ONE_GROUP[key] = torch.tensor([rows], dtype=torch.int64, device=x.device)
+        sizes = _ONE_GROUP[x.device] = torch.tensor([1 << 62], dtype=torch.int64, device=x.device)
     q, row_scale, q_t, col_scale = grouped_cast_rows_and_colwise_t(x, sizes, fp8_dtype, pow2=pow2)
     return q, row_scale, q_t, col_scale.reshape(-1)
 
