@@ -148,7 +148,8 @@ template <int HP, int FP8, bool SW>
 __device__ __forceinline__ void tile_cast_body(const void* x, int64_t row_end, int64_t cols, int64_t row0, int64_t col0,
                                                const float (&sc)[8], uint8_t* out, int64_t ld_out, uint8_t* out_t, int64_t ld_t,
                                                int64_t dst0, int64_t dst_end, uint32_t* lds_t,
-                                               uint8_t* out_r = nullptr, int64_t ld_r = 0, const float* row_scale = nullptr)
+                                               uint8_t* out_r = nullptr, int64_t ld_r = 0, const float* row_scale = nullptr,
+                                               int64_t row_scale_row0 = 0)
 {
     const int tid = threadIdx.x;
     const int wave = tid >> 6, lane = tid & 63;
@@ -167,14 +168,14 @@ __device__ __forceinline__ void tile_cast_body(const void* x, int64_t row_end, i
             HpVec<HP>::load8(xb + (r * cols + c8) * HpVec<HP>::kBytes, ok, f[it][j]);
         }
 
-    // the rows' own scales, read with the data (a read placed between the stores below would wait for them)
+    // the rows' own scales, read ahead of the stores below (a read placed between them would wait for them)
     float srow[2][4];
 #pragma unroll
     for (int it = 0; it < 2; ++it)
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
             const int64_t r = row0 + 32 * wave + 16 * it + 4 * g + j;
-            srow[it][j] = (out_r && r < row_end) ? row_scale[r] : 0.0f;
+            srow[it][j] = (out_r && r < row_end) ? row_scale[r - row_scale_row0] : 0.0f;  // (row_scale[0] = row row_scale_row0)
         }
 
 #pragma unroll
@@ -506,13 +507,6 @@ __global__ __launch_bounds__(kThreads) void grouped_colamax_kernel(GroupedCastAr
     }
 }
 
-template <int FP8>
-__global__ void row_scales_kernel(const uint32_t* __restrict__ row_amax, int64_t T, bool pow2, float* __restrict__ row_scale)
-{
-    const int64_t r = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (r < T) row_scale[r] = scale_from_amax_bits<FP8>(row_amax[r], pow2);
-}
-
 // Second pass of the SwiGLU backward of the dense feed-forward block when its two outputs are only ever needed
 // in fp8: with the amax of g1 and g3 known (first pass: swiglu_bwd_kernel without outputs), the gradients are
 // recomputed from x1, x3, gh tile by tile and go straight to their row-major and transposed fp8 copies - the bf16
@@ -723,6 +717,7 @@ __global__ __launch_bounds__(kThreads) void grouped_tile_cast_kernel(GroupedCast
 {
     __shared__ __attribute__((aligned(16))) uint32_t lds_t[kTile * kTile / 4];
     __shared__ float s_scale[kTile];
+    __shared__ float s_row_scale[kTile];
     int e;
     int64_t row0, row_end;
     if (!locate_padded_tile(a.sizes, a.E, a.T, (int)blockIdx.y, e, row0, row_end)) return;
@@ -737,6 +732,16 @@ __global__ __launch_bounds__(kThreads) void grouped_tile_cast_kernel(GroupedCast
             a.scale_out[(int64_t)e * a.cols + c] = s;  // every tile of the group writes the same value
         }
         s_scale[tid] = s;
+    } else if (a.out_r) {
+        // the other half of the workgroup: the scales of the tile's rows from their amax (every column tile
+        // derives the same values; the first one publishes them) - no separate launch for [T] scales
+        const int64_t r = row0 + tid - kTile;
+        float s = 0.0f;
+        if (r < row_end) {
+            s = scale_from_amax_bits<FP8>(a.row_amax[r], a.pow2);
+            if (blockIdx.x == 0) a.row_scale[r] = s;
+        }
+        s_row_scale[tid - kTile] = s;
     }
     __syncthreads();
     float sc[8];
@@ -744,7 +749,7 @@ __global__ __launch_bounds__(kThreads) void grouped_tile_cast_kernel(GroupedCast
     for (int i = 0; i < 8; ++i) sc[i] = s_scale[8 * cl + i];
     const int64_t dst0 = (int64_t)kTile * blockIdx.y;
     tile_cast_body<HP, FP8, SW>(a.x, row_end, a.cols, row0, col0, sc, nullptr, 0, a.out_t, a.ld_t, dst0, a.ld_t, lds_t,
-                                a.out_r, a.ld_r, a.row_scale);
+                                a.out_r, a.ld_r, s_row_scale, row0);
 }
 
 // ---- dispatch helpers ------------------------------------------------------------------------------
@@ -1184,13 +1189,6 @@ int grouped_cast_launch(const char* what, const void* x, int hp_dtype, int64_t T
             hipLaunchKernelGGL((grouped_colamax_kernel<MI8_F32>), grid, dim3(kThreads), 0, st, a);
         rc = launch_status(what);
         if (rc != MI8_OK) return rc;
-    }
-    if (out_rows) {
-        const dim3 rg((unsigned)ceil_div(T, 256));
-        if (fp8_dtype == MI8_E4M3)
-            hipLaunchKernelGGL((row_scales_kernel<MI8_E4M3>), rg, dim3(256), 0, st, row_amax_ws, T, pow2, row_scale_out);
-        else
-            hipLaunchKernelGGL((row_scales_kernel<MI8_E5M2>), rg, dim3(256), 0, st, row_amax_ws, T, pow2, row_scale_out);
     }
     const bool sw = flags & MI8_FLAG_SW_CVT;
 #define MI8_GC(HP_, FP8_)                                                                                   \
