@@ -181,6 +181,43 @@ def gemm_shapes(shapes, steps, warmup):
                           "operand_GB/s": round((m * k + n * k + 2 * m * n) / us / 1e3, 1), "steps": steps}), flush=True)
 
 
+HBM_PEAK_GBS = 8000.0
+
+
+def cast_rates(iters: int = 10):
+    """The HBM-bound half of the path, outside the timed region: the fused tensorwise cast (amax pass, then one pass
+    that writes the row-major and the transposed fp8 copy) of the step's largest activation, h [tokens, hidden] bf16.
+    Algorithmic bytes per element: 4 (2 read, 1 + 1 written); as the two passes stream it: 6 (the amax pass
+    reads x once more)."""
+    from olmo_core_amd.float8 import ops
+
+    dev = torch.device("cuda:0")
+    h = torch.randn(TOKENS, HIDDEN, device=dev, dtype=torch.bfloat16)
+    n = h.numel()
+
+    def run():
+        slots = ops.amax_partials(h)
+        ops.cast_tensorwise(h, torch.float8_e4m3fn, want_rowmajor=True, want_transposed=True, slots=slots)
+
+    for _ in range(3):
+        run()
+    start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    start.record()
+    for _ in range(iters):
+        run()
+    end.record()
+    torch.cuda.synchronize()
+    us = start.elapsed_time(end) / iters * 1e3
+    return {
+        "tensor": f"{TOKENS}x{HIDDEN} bf16 -> e4m3 row-major + transposed, tensorwise (amax pass + cast pass)",
+        "us": round(us, 1),
+        "GB/s_algorithmic_4B_per_elem": round(4.0 * n / us / 1e3, 1),
+        "GB/s_streamed_6B_per_elem": round(6.0 * n / us / 1e3, 1),
+        "frac_hbm_peak_streamed": round(6.0 * n / us / 1e3 / HBM_PEAK_GBS, 4),
+    }
+
+
 def traffic_probe():
     """Workload for the rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs: a plain 256 MiB device copy (the
     calibration: 268435456 bytes read and written), then the three GEMM shapes of the benchmark step and the
@@ -347,6 +384,8 @@ def main():
             "gemm_share_of_step": round(sum(gemm_ms) / ns.steps / ms_per_step, 4),
         },
     }
+    del mlp, x, go
+    result["cast"] = cast_rates()
     if not ns.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline()
     print(json.dumps(result), flush=True)
