@@ -102,6 +102,19 @@ int mi8_cast_tensorwise(const void* x, int hp_dtype, int64_t rows, int64_t cols,
                         int32_t n_slots, const float* scale_in, int fp8_dtype, uint32_t flags, void* out,
                         int64_t ld_out, void* out_t, int64_t ld_t, float* scale_out, void* stream);
 
+/* The dynamic tensorwise cast in one call for callers that cannot allocate device memory or hand over a
+ * workspace (code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc): amax pass +
+ * cast pass as mi8_amax_partials followed by mi8_cast_tensorwise(slots), with the partial maxima kept in an 8 KiB
+ * array that is part of the library's device image (one copy per GPU, held until the process ends) instead of a
+ * caller-owned workspace.  No counterpart in the reference.  Same outputs, bytes and scale as the two-call
+ * route.  Limits: rows, cols <= MI8_STATIC_CAST_MAX_DIM and rows * cols <= MI8_STATIC_CAST_MAX_ELEMS, larger
+ * inputs are refused with MI8_ERR_UNSUPPORTED.  All calls on one GPU share that GPU's array: calls that may
+ * overlap on one GPU (different streams, different threads) race; calls ordered on one stream do not. */
+#define MI8_STATIC_CAST_MAX_DIM ((int64_t)1 << 22)
+#define MI8_STATIC_CAST_MAX_ELEMS ((int64_t)1 << 32)
+int mi8_cast_tensorwise_static(const void* x, int hp_dtype, int64_t rows, int64_t cols, int fp8_dtype, uint32_t flags,
+                               void* out, int64_t ld_out, void* out_t, int64_t ld_t, float* scale_out, void* stream);
+
 
 /* ---------------------------------------------------------------------------------------------
  * Axiswise ("rowwise" recipe) dynamic casts: AXISWISE cast configs of the rowwise recipes

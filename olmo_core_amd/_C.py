@@ -42,6 +42,10 @@ _SIGNATURES = {
         [c_void_p, c_int, c_int64, c_int64, c_void_p, c_int32, c_void_p, c_int, c_uint32, c_void_p, c_int64,
          c_void_p, c_int64, c_void_p, c_void_p],
     ),
+    "mi8_cast_tensorwise_static": (
+        c_int,
+        [c_void_p, c_int, c_int64, c_int64, c_int, c_uint32, c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_void_p],
+    ),
     "mi8_cast_rowwise": (
         c_int,
         [c_void_p, c_int, c_int64, c_int64, c_int, c_uint32, c_void_p, c_int64, c_void_p, c_void_p],

@@ -1,6 +1,8 @@
 // amax reductions and saturating float8 casts (tensorwise, per-row, per-column with transposed output).
 // All kernels are HBM-bound streaming kernels: 16-byte loads per lane, wave-shuffle reductions, an
 // LDS-staged byte transpose for the transposed copy.
+#include <mutex>
+
 #include "mi8_groups.h"
 #include "mi8_swiglu.h"
 
@@ -1044,6 +1046,73 @@ extern "C" int mi8_cast_tensorwise(const void* x, int hp_dtype, int64_t rows, in
     dispatch_tile_cast(hp_dtype, fp8_dtype, (flags & MI8_FLAG_SW_CVT) != 0, slots ? kScalarFromSlots : kScalarFromPtr,
                        a, (hipStream_t)stream);
     return launch_status("mi8_cast_tensorwise");
+}
+
+// ------------------------------------------------------------------------------------------------
+// Tensorwise dynamic cast for callers that cannot allocate: the partial maxima live in a file-scope device
+// array instead of a caller-owned workspace.
+// ------------------------------------------------------------------------------------------------
+
+static __device__ __align__(256) uint32_t scratch[MI8_AMAX_SLOTS];
+
+namespace mi8 {
+namespace {
+
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mutex;
+uint32_t* g_scratch_ptr[kMaxDevices] = {};  // device address of `scratch` on each device, looked up once
+
+// The device address of this device's copy of `scratch` (every GPU holds its own copy at its own address; the
+// array's name is only a host-side handle for the lookup).
+int scratch_for_current_device(uint32_t** out)
+{
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess || dev < 0 || dev >= kMaxDevices) {
+        set_error("mi8_cast_tensorwise_static: cannot identify the current device (%s, device %d)",
+                  hipGetErrorString(e), dev);
+        return MI8_ERR_LAUNCH;
+    }
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (!g_scratch_ptr[dev]) {
+        void* p = nullptr;
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || !p) {
+            set_error("mi8_cast_tensorwise_static: hipGetSymbolAddress failed on device %d: %s", dev,
+                      hipGetErrorString(e));
+            return MI8_ERR_LAUNCH;
+        }
+        g_scratch_ptr[dev] = static_cast<uint32_t*>(p);
+    }
+    *out = g_scratch_ptr[dev];
+    return MI8_OK;
+}
+
+}  // namespace
+}  // namespace mi8
+
+extern "C" int mi8_cast_tensorwise_static(const void* x, int hp_dtype, int64_t rows, int64_t cols, int fp8_dtype,
+                                          uint32_t flags, void* out, int64_t ld_out, void* out_t, int64_t ld_t,
+                                          float* scale_out, void* stream)
+{
+    MI8_REQUIRE(x, MI8_ERR_ARG, "mi8_cast_tensorwise_static: x is null");
+    MI8_REQUIRE(valid_hp(hp_dtype), MI8_ERR_ARG, "mi8_cast_tensorwise_static: unknown hp dtype %d", hp_dtype);
+    MI8_REQUIRE(rows > 0 && cols > 0, MI8_ERR_ARG, "mi8_cast_tensorwise_static: empty input (%lld x %lld)",
+                (long long)rows, (long long)cols);
+    MI8_REQUIRE(rows <= MI8_STATIC_CAST_MAX_DIM && cols <= MI8_STATIC_CAST_MAX_DIM &&
+                    rows * cols <= MI8_STATIC_CAST_MAX_ELEMS,
+                MI8_ERR_UNSUPPORTED,
+                "mi8_cast_tensorwise_static: %lld x %lld is beyond the limit of this entry point (each dimension at "
+                "most %lld, at most %lld elements); use mi8_amax_partials + mi8_cast_tensorwise with a workspace",
+                (long long)rows, (long long)cols, (long long)MI8_STATIC_CAST_MAX_DIM,
+                (long long)MI8_STATIC_CAST_MAX_ELEMS);
+    uint32_t* slots = nullptr;
+    if (int rc = scratch_for_current_device(&slots)) return rc;
+    int32_t n_slots = 0;
+    // every slot the cast reads is written by this amax pass: nothing has to start at zero
+    if (int rc = mi8_amax_partials(x, hp_dtype, rows * cols, slots, &n_slots, stream)) return rc;
+    return mi8_cast_tensorwise(x, hp_dtype, rows, cols, slots, n_slots, nullptr, fp8_dtype, flags, out, ld_out, out_t,
+                               ld_t, scale_out, stream);
 }
 
 extern "C" int mi8_swiglu_bwd_cast(const void* x1, const void* x3, const void* gh, int64_t rows, int64_t cols,
