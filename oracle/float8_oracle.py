@@ -29,6 +29,12 @@ How each function is pinned (a check that a plausible mistake would fail), see t
   * ``swap/filter``   - known answers re-derived from src/olmo_core/float8/__init__.py:86-98,152-162.
   * ``grouped``       - per-expert loop (src/olmo_core/nn/moe/mlp.py:264-270) with the dense oracle
                         per slice, incl. empty groups.
+  * ``mlp_fwd_bwd``   - all five results against float32 autograd of w2(silu(w1 x) * w3 x) with w1, w3
+                        of different magnitude (cosine and norm ratio per tensor), and stage by stage,
+                        bit for bit, against the single-linear oracle plus the closed-form SwiGLU gradient.
+  * ``dropless_mlp_fwd_bwd`` - per expert against the float32 loop of mlp.py:264-292 (experts of
+                        different magnitude, an empty and a one-row expert), and exactly on
+                        small-integer inputs where the whole expert MLP is representable.
 Parity unpinned (no reference-held vector exists; only an import of torchao could confirm): the
 float64 upcast inside ``amax_to_scale``, the recipe defaults of ``from_recipe_name`` ("rowwise":
 e4m3 for grad_output, power-of-2 scales) and e5m2 as the default grad_output dtype.  Each of them is

@@ -306,3 +306,160 @@ def test_routing_bins():
     assert int(sizes.sum()) == 128 and bins[-1] == 128
     assert torch.equal(bins.long(), torch.cumsum(sizes, 0))
     assert bool((bin_ids[1:] >= bin_ids[:-1]).all())
+
+
+# ---- compositions: SwiGLU MLP and dropless-MoE MLP against float32 autograd ---------------------------
+
+
+def _cos(a, b):
+    a, b = a.double().reshape(-1), b.double().reshape(-1)
+    return float(torch.dot(a, b) / (a.norm() * b.norm()))
+
+
+def _norm_ratio(a, b):
+    return float(a.double().norm() / b.double().norm())
+
+
+# float8 noise bounds for the cosine: one e4m3 x e4m3 product is ~0.9993, the product of two such results
+# (h) ~0.9985; a gradient that passes through two e5m2 re-quantisations is ~0.9955.  A mis-wired composition
+# (g1/g3 swapped, an operand transposed, one grad_x term dropped, w2 used like w1) scores <= 0.95 on at least
+# one tensor with these inputs (asserted below), far outside these bounds.
+_COS_FWD, _COS_BWD = 0.998, 0.994
+
+
+@pytest.mark.parametrize("recipe", ["tensorwise", "rowwise"])
+def test_mlp_composition_tracks_autograd(recipe):
+    """All five results of mlp_fwd_bwd against float32 autograd of w2(silu(w1 x) * w3 x)
+    (src/olmo_core/nn/feed_forward.py:161-171).  w3 is three times larger than w1, so grad_w1 and grad_w3 (and the
+    two terms of grad_x) differ in magnitude as well as direction: a swap or a dropped term fails both the cosine
+    and the norm-ratio bound."""
+    M, D, H = 192, 128, 256
+    x = seeded((M, D), 1)
+    w1, w3 = seeded((H, D), 2, std=0.08), seeded((H, D), 3, std=0.24)
+    w2 = seeded((D, H), 4, std=0.05)
+    go = seeded((M, D), 5, std=1e-3)
+    tr = O.mlp_fwd_bwd(x, w1, w2, w3, go, O.recipe(recipe))
+
+    xr = x.float().requires_grad_()
+    p1, p2, p3 = (w.float().requires_grad_() for w in (w1, w2, w3))
+    F = torch.nn.functional
+    h = F.silu(F.linear(xr, p1)) * F.linear(xr, p3)
+    y = F.linear(h, p2)
+    y.backward(go.float())
+
+    assert tr.y.shape == (M, D) and tr.grad_x.shape == x.shape
+    assert tr.grad_w1.shape == w1.shape and tr.grad_w2.shape == w2.shape and tr.grad_w3.shape == w3.shape
+    assert _cos(tr.h, h.detach()) > _COS_FWD
+    assert _cos(tr.y, y.detach()) > 0.997
+    for name, got, want in (("grad_x", tr.grad_x, xr.grad), ("grad_w1", tr.grad_w1, p1.grad),
+                            ("grad_w2", tr.grad_w2, p2.grad), ("grad_w3", tr.grad_w3, p3.grad)):
+        assert _cos(got, want) > _COS_BWD, (name, _cos(got, want))
+        assert 0.97 < _norm_ratio(got, want) < 1.03, (name, _norm_ratio(got, want))
+    # the inputs do separate the mistakes this test is for
+    assert abs(_cos(p1.grad, p3.grad)) < 0.5 and not 0.8 < _norm_ratio(p1.grad, p3.grad) < 1.25
+    gx1 = torch.autograd.grad(F.linear(F.silu(F.linear(xr, p1)) * F.linear(xr, p3).detach(), p2), xr, go.float())[0]
+    assert _cos(gx1, xr.grad) < 0.95  # one term of grad_x alone is not grad_x
+
+
+def test_mlp_composition_feeds_each_stage_the_previous_stage():
+    """Wiring of the stages, bit for bit: w2 consumes the cast of h, w1/w3's backward consume the casts of the SwiGLU
+    gradients of w2's grad_input, and every stage equals the single-linear oracle on those tensors."""
+    M, D, H = 64, 64, 96
+    x, go = seeded((M, D), 1), seeded((M, D), 5, std=1e-3)
+    w1, w3, w2 = seeded((H, D), 2, std=0.1), seeded((H, D), 3, std=0.2), seeded((D, H), 4, std=0.1)
+    spec = O.recipe("tensorwise")
+    tr = O.mlp_fwd_bwd(x, w1, w2, w3, go, spec)
+    x1 = O.linear_forward(x, w1, None, spec).out
+    x3 = O.linear_forward(x, w3, None, spec).out
+    h = torch.nn.functional.silu(x1) * x3
+    assert torch.equal(tr.h, h)
+    t2 = O.linear_fwd_bwd(h, w2, None, go, spec)
+    assert torch.equal(tr.y, t2.out) and torch.equal(tr.grad_w2, t2.grad_weight)
+    # SwiGLU gradient in closed form (float64), compared after the bf16 roundings torch applies
+    gh = t2.grad_input.double()
+    s = torch.sigmoid(x1.double())
+    g1_ref = gh * x3.double() * (s * (1 + x1.double() * (1 - s)))
+    g3_ref = gh * (x1.double() * s)
+    g1, g3 = O.swiglu_backward(x1, x3, t2.grad_input)
+    assert _cos(g1, g1_ref) > 0.99995 and _cos(g3, g3_ref) > 0.99995
+    assert torch.equal(tr.grad_w1, O.linear_backward(x, w1, g1, spec).grad_weight)
+    assert torch.equal(tr.grad_w3, O.linear_backward(x, w3, g3, spec).grad_weight)
+    want_gx = O.linear_backward(x, w1, g1, spec).grad_input + O.linear_backward(x, w3, g3, spec).grad_input
+    assert torch.equal(tr.grad_x, want_gx)
+
+
+def _dropless_autograd(x, w1, w2, w3, sizes, go):
+    """The reference's per-expert loop in float32 (src/olmo_core/nn/moe/mlp.py:264-292): w1, w3 [E,H,D] used
+    transposed, w2 [E,H,D] used as stored."""
+    xr = x.float().requires_grad_()
+    p1, p2, p3 = (w.float().requires_grad_() for w in (w1, w2, w3))
+    outs, start = [], 0
+    for e, n in enumerate(sizes):
+        xe = xr[start:start + n]
+        he = torch.nn.functional.silu(xe @ p1[e].t()) * (xe @ p3[e].t())
+        outs.append(he @ p2[e])
+        start += n
+    y = torch.cat(outs)
+    y.backward(go.float())
+    return y.detach(), xr.grad, p1.grad, p2.grad, p3.grad
+
+
+def test_dropless_mlp_composition_tracks_autograd():
+    """dropless_mlp_fwd_bwd against the float32 per-expert loop: experts and the three weight tensors have distinct
+    magnitudes, one expert is empty, one has a single row; checked per expert so that a weight taken from the wrong
+    expert, w2 used transposed, or w1/w3 swapped shows."""
+    E, D, H = 5, 64, 96
+    sizes = [40, 0, 1, 23, 64]
+    T = sum(sizes)
+    x, go = seeded((T, D), 1), seeded((T, D), 5, std=1e-3)
+    mag = (2.0 ** torch.arange(E)).reshape(E, 1, 1)
+    w1 = (seeded((E, H, D), 2, std=0.05).float() * mag).bfloat16()
+    w3 = (seeded((E, H, D), 3, std=0.15).float() * mag.flip(0)).bfloat16()
+    w2 = seeded((E, H, D), 4, std=0.1)
+    res = O.dropless_mlp_fwd_bwd(x, w1, w2, w3, sizes, go, O.recipe("rowwise"))
+    y, gx, g1, g2, g3 = _dropless_autograd(x, w1, w2, w3, sizes, go)
+
+    assert res["y"].shape == (T, D) and res["grad_x"].shape == (T, D)
+    for k in ("grad_w1", "grad_w2", "grad_w3"):
+        assert res[k].shape == (E, H, D)
+        assert torch.count_nonzero(res[k][1]) == 0, "the empty expert's weight gradient is zero"
+    start = 0
+    for e, n in enumerate(sizes):
+        if n:
+            rows = slice(start, start + n)
+            assert _cos(res["y"][rows], y[rows]) > 0.996, (e, "y", _cos(res["y"][rows], y[rows]))
+            assert _cos(res["grad_x"][rows], gx[rows]) > _COS_BWD, (e, "grad_x", _cos(res["grad_x"][rows], gx[rows]))
+            assert 0.96 < _norm_ratio(res["grad_x"][rows], gx[rows]) < 1.04
+            for name, got, want in (("grad_w1", res["grad_w1"][e], g1[e]), ("grad_w2", res["grad_w2"][e], g2[e]),
+                                    ("grad_w3", res["grad_w3"][e], g3[e])):
+                assert _cos(got, want) > _COS_BWD, (e, name, _cos(got, want))
+                assert 0.96 < _norm_ratio(got, want) < 1.04, (e, name)
+        start += n
+    # the construction separates the mistakes: other experts' and the transposed w2's results are far away
+    assert abs(_cos(g1[0], g3[0])) < 0.5 and abs(_cos(g1[0], g1[4])) < 0.5
+
+
+def test_dropless_mlp_exact_on_representable_inputs():
+    """With silu's argument driven far positive (silu(v) = v to bf16 precision for v >= 32) and small-integer data
+    the whole expert MLP is exact in float8 under power-of-two scales: y = ((x w1^T) * (x w3^T)) w2 per expert.
+    Any indexing slip between experts changes an integer."""
+    E, D, H = 3, 16, 16
+    sizes = [3, 0, 5]
+    T = sum(sizes)
+    g = torch.Generator().manual_seed(0)
+    x = torch.zeros(T, D); x[:, 0] = 1.0
+    x[:, 1:4] = torch.randint(0, 2, (T, 3), generator=g).float()
+    w1 = torch.zeros(E, H, D); w1[:, :, 0] = 32.0            # x1 = 32 for every row and hidden unit
+    w3 = torch.randint(-2, 3, (E, H, D), generator=g).float() * torch.tensor([1.0, 2.0, 4.0]).reshape(E, 1, 1)
+    w2 = torch.randint(-1, 2, (E, H, D), generator=g).float()
+    res = O.dropless_mlp_fwd_bwd(x.bfloat16(), w1.bfloat16(), w2.bfloat16(), w3.bfloat16(), sizes, None, O.recipe("rowwise"))
+    start, outs = 0, []
+    for e, n in enumerate(sizes):
+        xe = x[start:start + n]
+        x1 = xe @ w1[e].t()
+        assert torch.equal(torch.nn.functional.silu(x1.bfloat16()).float(), x1)  # silu is the identity here
+        outs.append((x1 * (xe @ w3[e].t())) @ w2[e])
+        start += n
+    want = torch.cat(outs)
+    assert float(want.abs().max()) <= 2.0**15
+    assert torch.equal(res["y"].float(), want.bfloat16().float())
