@@ -21,6 +21,10 @@ from ..float8.linear import Float8Linear, _is_tensorwise, _shared_tensorwise
 
 __all__ = ["FeedForward", "swiglu"]
 
+# Test hook: when set to a dict, the fused function stores clones of its bf16 intermediates (x1, x3, h, gh) there,
+# so that a checker can feed each stage's actual input to a reference of that stage.
+STAGE_SINK = None
+
 
 class _SwiGLU(torch.autograd.Function):
     @staticmethod
@@ -65,6 +69,8 @@ class _Float8SwiGLUMLP(torch.autograd.Function):
         x1 = ops.gemm_fp8(xq, sx, w1q, s1, out_dtype=x.dtype)
         x3 = ops.gemm_fp8(xq, sx, w3q, s3, out_dtype=x.dtype)
         h, h_slots = ops.swiglu_fwd(x1, x3, want_amax=True)
+        if STAGE_SINK is not None:
+            STAGE_SINK.update(x1=x1.clone(), x3=x3.clone(), h=h.clone())
         hq, hq_t, sh = ops.cast_tensorwise(h, in_dt, pow2=pow2, want_transposed=need[2], slots=h_slots)
         y = ops.gemm_fp8(hq, sh, w2q, s2, out_dtype=x.dtype)
         ctx.config = c
@@ -95,6 +101,8 @@ class _Float8SwiGLUMLP(torch.autograd.Function):
         gx = gw1 = gw3 = None
         if need_gh:
             gh = ops.gemm_fp8(gyq, sgy, w2q_t, s2, k=D, out_dtype=x_dt)
+            if STAGE_SINK is not None:
+                STAGE_SINK.update(gh=gh.clone())
             need_t = need_w1 or need_w3
             # g1 and g3 are needed in fp8 only: amax pass, then recompute-and-cast pass (no bf16 round trip)
             g1q, g1q_t, sg1, g3q, g3q_t, sg3 = ops.swiglu_bwd_cast(

@@ -24,6 +24,10 @@ __all__ = ["DroplessMoEMLP", "float8_dropless_mlp"]
 
 _E4M3 = torch.float8_e4m3fn
 
+# Test hook: when set to a dict, the expert MLP stores clones of its bf16 intermediates (x1, x2, h, gh, g1, g2)
+# there, so that a checker can feed each stage's actual input to a reference of that stage.
+STAGE_SINK = None
+
 
 class _Float8DroplessMLP(torch.autograd.Function):
     @staticmethod
@@ -33,6 +37,8 @@ class _Float8DroplessMLP(torch.autograd.Function):
         H = w1.shape[0] // E
         dev = x.device
         equal = torch.full((E,), H, dtype=torch.int64, device=dev)  # the experts' weights as equal-size groups
+        # in the transposed copies every expert's segment starts on a multiple of 128 columns
+        Hp = (H + 127) // 128 * 128
 
         need = ctx.needs_input_grad
         need_w13 = need[1] or need[3]
@@ -56,6 +62,8 @@ class _Float8DroplessMLP(torch.autograd.Function):
         if need[2]:
             # the pointwise kernel also takes the amax of h per row and per (expert, column): the cast is one pass
             h, h_amax = ops.grouped_swiglu_fwd(x1, x2, sizes)
+            if STAGE_SINK is not None:
+                STAGE_SINK.update(x1=x1.clone(), x2=x2.clone(), h=h.clone())
             hq, sh, ht, shc = ops.grouped_cast_rows_and_colwise_t(h, sizes, _E4M3, pow2=pow2, amax=h_amax)
         else:
             h, _ = ops.swiglu_fwd(x1, x2, want_amax=False)
@@ -67,18 +75,18 @@ class _Float8DroplessMLP(torch.autograd.Function):
             w2q, s2r, w2t, s2 = ops.grouped_cast_rows_and_colwise_t(w2, equal, _E4M3, pow2=pow2)
         else:
             w2t, s2 = ops.grouped_cast_colwise_t(w2, equal, _E4M3, pow2=pow2)
-        y = ops.grouped_gemm_fp8(hq, sh, w2t, s2, sizes, n=D, k=H, b_group_stride=H, sb_group_stride=D)
+        y = ops.grouped_gemm_fp8(hq, sh, w2t, s2, sizes, n=D, k=H, b_group_stride=Hp, sb_group_stride=D)
         none = x.new_empty(0)
         opt = lambda t: none if t is None else t  # noqa: E731
         ctx.save_for_backward(opt(xt), opt(sxc), x1, x2, opt(ht), opt(shc), opt(w1t), opt(s1c), opt(w3t), opt(s3c),
                               opt(w2q), opt(s2r), sizes)
-        ctx.meta = (E, T, D, H, pow2, (x.dtype, w1.dtype, w2.dtype, w3.dtype))
+        ctx.meta = (E, T, D, H, Hp, pow2, (x.dtype, w1.dtype, w2.dtype, w3.dtype))
         return y
 
     @staticmethod
     def backward(ctx, gy):
         xt, sxc, x1, x2, ht, shc, w1t, s1c, w3t, s3c, w2q, s2r, sizes = ctx.saved_tensors
-        E, T, D, H, pow2, (x_dt, w1_dt, w2_dt, w3_dt) = ctx.meta
+        E, T, D, H, Hp, pow2, (x_dt, w1_dt, w2_dt, w3_dt) = ctx.meta
         gy = gy.reshape(T, D).contiguous()
         if gy.dtype != x_dt:
             gy = gy.to(x_dt)
@@ -103,6 +111,8 @@ class _Float8DroplessMLP(torch.autograd.Function):
             else:
                 g1, g2, _, _ = ops.swiglu_bwd(x1, x2, gh, want_amax=False)
                 amax1 = amax2 = None
+            if STAGE_SINK is not None:
+                STAGE_SINK.update(gh=gh.clone(), g1=g1.clone(), g2=g2.clone())
             del gh
 
             def both(g, want_rows, want_cols, amax):
@@ -119,8 +129,8 @@ class _Float8DroplessMLP(torch.autograd.Function):
             del g1, g2
             if need_x:
                 # gx_e = g_e @ w[e] : contraction over H, the right operand is w[e]^T [D, H], one scale per input channel
-                gx = ops.grouped_gemm_fp8(g1q, sg1, w1t, s1c, sizes, n=D, k=H, b_group_stride=H, sb_group_stride=D)
-                gx = gx + ops.grouped_gemm_fp8(g2q, sg2, w3t, s3c, sizes, n=D, k=H, b_group_stride=H, sb_group_stride=D)
+                gx = ops.grouped_gemm_fp8(g1q, sg1, w1t, s1c, sizes, n=D, k=H, b_group_stride=Hp, sb_group_stride=D)
+                gx = gx + ops.grouped_gemm_fp8(g2q, sg2, w3t, s3c, sizes, n=D, k=H, b_group_stride=Hp, sb_group_stride=D)
             if need_w1:
                 gw1 = ops.grouped_wgrad_fp8(g1t, sg1c, xt, sxc, sizes, tokens=T, out_dtype=x_dt).reshape(E * H, D)
             if need_w3:

@@ -74,3 +74,20 @@ def assert_gemm_close(got, ref, what=""):
 
 def spec_for(recipe: str) -> O.LinearSpec:
     return O.recipe(recipe)
+
+
+def assert_bf16_pointwise_close(got, ref, what="", max_frac=1e-2, ulps=2):
+    """A pointwise bf16 result against the host's evaluation of the same formula on the same inputs: the device's
+    exp / reciprocal differ from the host's in the last place before a bf16 rounding, so a small fraction of
+    elements may differ, each by at most `ulps` bf16 steps of its own magnitude."""
+    g, r = got.detach().cpu(), ref.detach().cpu()
+    assert g.shape == r.shape and g.dtype == r.dtype == torch.bfloat16, what
+    diff = g != r
+    frac = float(diff.float().mean())
+    assert frac < max_frac, f"{what}: {frac:.4%} of the elements differ (limit {max_frac:.2%})"
+    if diff.any():
+        gi, ri = g.view(torch.int16).int(), r.view(torch.int16).int()
+        # same sign and adjacent bit patterns = adjacent bf16 values
+        step = (gi - ri).abs()[diff]
+        tiny = (r.float().abs()[diff] < 1e-30) & (g.float().abs()[diff] < 1e-30)
+        assert bool(((step <= ulps) | tiny).all()), f"{what}: an element differs by more than {ulps} bf16 steps"

@@ -1,0 +1,120 @@
+"""Stage-by-stage parity of the two composed blocks (SwiGLU feed-forward, dropless-MoE expert MLP).
+
+The blocks re-quantise bf16 intermediates, so an end-to-end comparison with the oracle's composition compounds
+last-place differences of the device's bf16 intermediates.  Here every stage is compared with the oracle of that
+stage on the device's own input of the stage (copied to the host): GEMM stages are then held to the single-GEMM bar
+(max relative error 1e-2, cosine 0.9999), casts to bit-exact bytes and scales, pointwise stages to a couple of bf16
+steps on a small fraction of the elements.  GPU tests only."""
+
+import torch
+
+from helpers import (E4M3, E5M2, assert_bf16_pointwise_close, assert_bytes_equal, assert_gemm_close,
+                     assert_scale_equal)
+from oracle import float8_oracle as O
+
+
+def check_mlp_stages(dev, ff, x, go, recipe="tensorwise"):
+    """ff: a converted olmo_core_amd.nn.FeedForward on `dev` (tensorwise recipe, fused); x, go: host bf16 tensors."""
+    from olmo_core_amd.float8 import ops
+    from olmo_core_amd.nn import feed_forward as ff_mod
+
+    spec = O.recipe(recipe)
+    M = x.shape[0]
+    w1, w2, w3 = (ff.w1.weight.detach().cpu(), ff.w2.weight.detach().cpu(), ff.w3.weight.detach().cpu())
+    xd = x.to(dev).requires_grad_(True)
+    ff_mod.STAGE_SINK = sink = {}
+    try:
+        y = ff(xd)
+        y.backward(go.to(dev))
+    finally:
+        ff_mod.STAGE_SINK = None
+    assert set(sink) == {"x1", "x3", "h", "gh"}, "the fused function did not run"
+    gx, gw1, gw2, gw3 = xd.grad, ff.w1.weight.grad, ff.w2.weight.grad, ff.w3.weight.grad
+    x1, x3, h, gh = (sink[k].cpu() for k in ("x1", "x3", "h", "gh"))
+
+    # stage 1: the two input projections from x
+    assert_gemm_close(x1, O.linear_forward(x, w1, None, spec).out, "x1 = x W1^T")
+    assert_gemm_close(x3, O.linear_forward(x, w3, None, spec).out, "x3 = x W3^T")
+    # stage 2: h from the device's x1, x3
+    assert_bf16_pointwise_close(h, O.swiglu(x1, x3), "h = silu(x1) * x3")
+    # stage 3: the cast of the device's h (bytes and scale bit-exact), then y and w2's backward from it
+    hq, hq_t, sh = ops.cast_tensorwise(sink["h"], E4M3, want_transposed=True)
+    ref_hq, ref_sh = O.cast(h, E4M3)
+    assert_scale_equal(sh, ref_sh, "scale of h")
+    assert_bytes_equal(hq, ref_hq, what="q(h)")
+    assert_bytes_equal(hq_t[:, :M], ref_hq.t(), what="q(h)^T")
+    t2 = O.linear_fwd_bwd(h, w2, None, go, spec)
+    assert_gemm_close(y, t2.out, "y = h W2^T")
+    assert_gemm_close(gw2, t2.grad_weight, "grad_w2 = go^T h")
+    assert_gemm_close(gh, t2.grad_input, "grad_h = go W2")
+    # stage 4: the gate gradients from the device's x1, x3, grad_h.  The fused block never writes them in bf16: the
+    # two-step kernels (bit-identical to the fused route, test_swiglu_backward_cast_equals_two_steps) are compared
+    # with the host's autograd, and the fused cast's bytes with the oracle's cast of the device's g1, g3
+    g1, g3, _, _ = ops.swiglu_bwd(sink["x1"], sink["x3"], sink["gh"])
+    r1, r3 = O.swiglu_backward(x1, x3, gh)
+    assert_bf16_pointwise_close(g1, r1, "g1", max_frac=2e-2)
+    assert_bf16_pointwise_close(g3, r3, "g3", max_frac=2e-2)
+    q1, q1t, s1, q3, q3t, s3 = ops.swiglu_bwd_cast(sink["x1"], sink["x3"], sink["gh"], E5M2, want_transposed=True)
+    g1, g3 = g1.cpu(), g3.cpu()
+    for name, g, q, qt, s in (("g1", g1, q1, q1t, s1), ("g3", g3, q3, q3t, s3)):
+        ref_q, ref_s = O.cast(g, E5M2)
+        assert_scale_equal(s, ref_s, f"scale of {name}")
+        assert_bytes_equal(q, ref_q, what=f"q({name})")
+        assert_bytes_equal(qt[:, :M], ref_q.t(), what=f"q({name})^T")
+    # stage 5: w1 / w3 backward from the device's g1, g3
+    b1 = O.linear_backward(x, w1, g1, spec)
+    b3 = O.linear_backward(x, w3, g3, spec)
+    assert_gemm_close(gw1, b1.grad_weight, "grad_w1 = g1^T x")
+    assert_gemm_close(gw3, b3.grad_weight, "grad_w3 = g3^T x")
+    assert_gemm_close(gx, b1.grad_input + b3.grad_input, "grad_x = g1 W1 + g3 W3")
+
+
+def check_dropless_stages(dev, mlp, x, go, sizes, experts):
+    """mlp: an olmo_core_amd.nn.DroplessMoEMLP still on the host; x, go: host bf16 [sum(sizes), d_model];
+    experts: the experts whose slices are compared (every stage is checked per expert: a weight or a scale taken
+    from a neighbouring expert would hide in a maximum over all rows)."""
+    from olmo_core_amd.nn import moe as moe_mod
+
+    spec = O.recipe("rowwise")
+    E, H, D = mlp.num_experts, mlp.hidden_size, mlp.d_model
+    w1, w2, w3 = (p.detach().clone().view(E, H, D) for p in (mlp.w1, mlp.w2, mlp.w3))
+    mlp = mlp.to(dev)
+    xd = x.to(dev).requires_grad_(True)
+    moe_mod.STAGE_SINK = sink = {}
+    try:
+        y = mlp(xd, torch.tensor(sizes).to(dev))
+        y.backward(go.to(dev))
+    finally:
+        moe_mod.STAGE_SINK = None
+    assert set(sink) == {"x1", "x2", "h", "gh", "g1", "g2"}
+    gw1, gw2, gw3 = (p.grad.view(E, H, D) for p in (mlp.w1, mlp.w2, mlp.w3))
+    starts = [0]
+    for n in sizes:
+        starts.append(starts[-1] + int(n))
+    for e in experts:
+        n = int(sizes[e])
+        tag = f"expert {e} ({n} rows)"
+        if n == 0:
+            for gw in (gw1, gw2, gw3):
+                assert torch.count_nonzero(gw[e]) == 0, f"{tag}: weight gradient of an empty expert must be zero"
+            continue
+        rows = slice(starts[e], starts[e] + n)
+        xe, goe = x[rows], go[rows]
+        x1, x2, h, gh, g1, g2 = (sink[k][rows].cpu() for k in ("x1", "x2", "h", "gh", "g1", "g2"))
+        one = [n]
+        assert_gemm_close(x1, O.grouped_linear_fwd_bwd(xe, w1[e:e + 1], one, None, spec, trans_b=True)[0], f"{tag}: x1")
+        assert_gemm_close(x2, O.grouped_linear_fwd_bwd(xe, w3[e:e + 1], one, None, spec, trans_b=True)[0], f"{tag}: x2")
+        assert_bf16_pointwise_close(h, O.swiglu(x1, x2), f"{tag}: h")
+        ry, rgh, rgw2, _ = O.grouped_linear_fwd_bwd(h, w2[e:e + 1], one, goe, spec, trans_b=False)
+        assert_gemm_close(y[rows], ry, f"{tag}: y")
+        assert_gemm_close(gh, rgh, f"{tag}: grad_h")
+        assert_gemm_close(gw2[e], rgw2[0], f"{tag}: grad_w2")
+        r1, r2 = O.swiglu_backward(x1, x2, gh)
+        assert_bf16_pointwise_close(g1, r1, f"{tag}: g1", max_frac=2e-2)
+        assert_bf16_pointwise_close(g2, r2, f"{tag}: g2", max_frac=2e-2)
+        _, gxa, rgw1, _ = O.grouped_linear_fwd_bwd(xe, w1[e:e + 1], one, g1, spec, trans_b=True)
+        _, gxb, rgw3, _ = O.grouped_linear_fwd_bwd(xe, w3[e:e + 1], one, g2, spec, trans_b=True)
+        assert_gemm_close(gw1[e], rgw1[0], f"{tag}: grad_w1")
+        assert_gemm_close(gw3[e], rgw3[0], f"{tag}: grad_w3")
+        assert_gemm_close(xd.grad[rows], gxa + gxb, f"{tag}: grad_x")
+    return sink

@@ -260,7 +260,7 @@ def test_dropless_mlp_shape_contract(dev):
 
 
 @pytest.mark.parametrize("sizes", [[3, 2], [40, 0, 90, 7], [300, 17, 0, 0, 411, 64]], ids=_case_id)
-@pytest.mark.parametrize("dims", [(128, 256), (256, 384)], ids=lambda d: f"{d[0]}x{d[1]}")
+@pytest.mark.parametrize("dims", [(128, 256), (256, 384), (128, 320)], ids=lambda d: f"{d[0]}x{d[1]}")
 def test_dropless_mlp_against_oracle(dev, sizes, dims):
     E, (D, H) = len(sizes), dims
     if D >= 256 and sum(sizes) < 256:
@@ -332,3 +332,21 @@ def test_routed_layer_against_oracle(dev, tokens, top_k):
     rel, cos = gemm_errors(wd.grad, want_gw)
     assert rel <= 3e-2 and cos >= 0.9995, ("grad_expert_weights", rel, cos)
     assert torch.count_nonzero(mlp.w1.grad.view(E, H, D)[5]) == 0
+
+
+@pytest.mark.parametrize("sizes,dims", [([40, 0, 90, 7], (128, 256)), ([300, 17, 0, 0, 411, 64], (256, 384)),
+                                        ([33, 150, 1], (128, 320))], ids=["4e-128x256", "6e-256x384", "3e-128x320"])
+def test_dropless_mlp_stage_by_stage_against_oracle(dev, sizes, dims):
+    """Every stage of the expert MLP against the oracle of that stage fed with the device's own bf16 input of the
+    stage (stage_checks.check_dropless_stages), expert by expert.  A hidden size that is not a multiple of 128 is
+    included: the transposed weight copies pad every expert to 128 columns."""
+    from stage_checks import check_dropless_stages
+
+    E, (D, H) = len(sizes), dims
+    T = sum(sizes)
+    mlp = DroplessMoEMLP(d_model=D, hidden_size=H, num_experts=E, dtype=torch.bfloat16)
+    g = torch.Generator().manual_seed(3)
+    with torch.no_grad():
+        for i, p in enumerate(mlp.parameters()):
+            p.copy_((torch.randn(p.shape, generator=g) * 0.02 * (1 + i)).bfloat16())
+    check_dropless_stages(dev, mlp, seeded((T, D), 1), seeded((T, D), 2, std=1e-3), sizes, experts=range(E))

@@ -107,3 +107,16 @@ def test_swiglu_backward_cast_equals_two_steps(dev, shape, layouts, fp8):
             assert torch.equal(qt.view(torch.uint8), wqt.view(torch.uint8))
         else:
             assert qt is None
+
+
+@pytest.mark.parametrize("mdh", [(640, 512, 1280), (1024, 768, 2048)], ids=lambda s: "x".join(map(str, s)))
+def test_mlp_stage_by_stage_against_oracle(dev, mdh):
+    """Every stage of the fused block against the oracle of THAT stage fed with the device's own bf16 input of the
+    stage (stage_checks.check_mlp_stages): GEMM stages at the single-GEMM bar (1e-2 / 0.9999), casts bit-exact,
+    SwiGLU stages within bf16 steps on < 1-2 % of the elements.  The end-to-end comparison in
+    test_mlp_against_oracle is then a secondary check."""
+    from stage_checks import check_mlp_stages
+
+    M, D, H = mdh
+    x, go = seeded((M, D), 1), seeded((M, D), 2, std=1e-3)
+    check_mlp_stages(dev, _make(dev, D, H, fuse=True, seed=3), x, go)
