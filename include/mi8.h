@@ -6,7 +6,10 @@
  *   - returns MI8_OK (0) or a negative mi8_status; mi8_last_error() gives the text for the calling
  *     thread's most recent failure;
  *   - only enqueues work on `stream` (a hipStream_t passed as void*; NULL = the default stream): it never
- *     synchronises, never allocates or frees device memory, and keeps no state between calls;
+ *     synchronises, never allocates or frees device memory, and keeps no state between calls that a caller could
+ *     observe (the only memory of the library is per-device one-time set-up: a kernel's dynamic-LDS attribute and
+ *     the compute-unit count, both latched with atomics, so first calls from several threads or on several
+ *     devices are safe);
  *   - requires every pointer to be 16-byte aligned device memory of at least the stated size.
  * All matrices are dense row-major with the row pitch given (or implied) in elements.
  *

@@ -4,6 +4,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <atomic>
+
 #include "../../include/mi8.h"
 
 namespace mi8 {
@@ -11,6 +13,11 @@ namespace mi8 {
 // ---- host side: error reporting --------------------------------------------------------------
 void set_error(const char* fmt, ...) __attribute__((format(printf, 1, 2)));
 int launch_status(const char* what);  // MI8_OK or MI8_ERR_LAUNCH after a kernel launch
+
+// One-time set-up per kernel and device, safe under concurrent first calls: `done` holds one bit per device
+// ordinal; setting the attribute twice is harmless, so two racing threads only repeat the call.
+int reserve_dynamic_lds(const void* kernel, int bytes, std::atomic<uint64_t>& done, const char* what);
+int num_compute_units();  // of the current device (cached per device)
 
 #define MI8_REQUIRE(cond, code, ...)     \
     do {                                 \

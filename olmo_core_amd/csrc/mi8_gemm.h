@@ -72,14 +72,8 @@ __device__ __forceinline__ bool tile_of_block(const GemmArgs& g, int& tm, int& t
     return true;
 }
 
-// persistent direct-to-LDS kernel (mi8_gemm_dma.hip); requires M, N >= 256, K % 64 == 0, N % 8 == 0, ldc % 8 == 0,
-// a 16-byte aligned bf16 output
-int launch_dma(GemmArgs& g, int a_dtype, int b_dtype, hipStream_t st);
-// same, 8 waves per workgroup and full 128-byte rows; additionally K % 128 == 0 (mi8_gemm_dma8.hip)
-int launch_dma8(GemmArgs& g, int a_dtype, int b_dtype, hipStream_t st);
-// the same kernel with four waves of 128 x 128 (one wave per SIMD)
-int launch_dma4(GemmArgs& g, int a_dtype, int b_dtype, hipStream_t st);
-// four waves of 128 x 128 on 16x16x128 MFMAs (mi8_gemm_m16.hip), same requirements
+// persistent direct-to-LDS kernel, four waves of 128 x 128 on 16x16x128 MFMAs (mi8_gemm_m16.hip); requires
+// M, N >= 256, K % 128 == 0, N % 8 == 0, ldc % 8 == 0, a 16-byte aligned bf16 output
 int launch_m16(GemmArgs& g, int a_dtype, int b_dtype, hipStream_t st);
 // a few rows of A (M <= kSkinnyMaxM) against all of B, bound by reading B once (mi8_gemm_skinny.hip): any N,
 // K % 16 == 0, any mix of single scales and scale vectors, bf16 or fp32 output

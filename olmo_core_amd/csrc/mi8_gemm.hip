@@ -10,8 +10,8 @@
 //
 // This file holds that general tile kernel (any M, N; K % 16 == 0; bf16 or fp32 output), its split-K form for
 // problems with few output tiles, and the entry points, which pick a kernel by shape: the persistent direct-to-LDS
-// kernels of mi8_gemm_m16.hip / mi8_gemm_dma8.hip / mi8_gemm_dma.hip for large problems, the weight-streaming
-// kernel of mi8_gemm_skinny.hip for a few rows of A.
+// kernel of mi8_gemm_m16.hip for large problems, the weight-streaming kernel of mi8_gemm_skinny.hip for a few
+// rows of A.
 #include "mi8_gemm_body.h"
 
 namespace mi8 {
@@ -105,16 +105,9 @@ int launch_splitk_typed(const SplitArgs& a, hipStream_t st)
 {
     auto kern = gemm_fp8_splitk_kernel<CBSZ, BLGP>;
     constexpr int lds_bytes = 2 * (kSplitTile + kSplitTile) * BK;
-    static bool configured = false;
-    if (!configured) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
-        if (e != hipSuccess) {
-            set_error("mi8_gemm_fp8_splitk: cannot reserve %d bytes of LDS: %s", lds_bytes, hipGetErrorString(e));
-            return MI8_ERR_LAUNCH;
-        }
-        configured = true;
-    }
+    static std::atomic<uint64_t> configured{0};
+    if (int rc = reserve_dynamic_lds(reinterpret_cast<const void*>(kern), lds_bytes, configured, "mi8_gemm_fp8_splitk"))
+        return rc;
     const int total = a.g.tiles_m * a.g.tiles_n;
     hipLaunchKernelGGL(kern, dim3(((total + 7) / 8) * 8, a.splits), dim3(256), lds_bytes, st, a);
     const int64_t quads = (int64_t)a.g.M * (a.ld_plane / 4);
@@ -149,13 +142,10 @@ constexpr Variant kVariants[] = {
     {"128x128_w2x2", 128, 128, 256},
     {"256x128_w2x2", 256, 128, 256},
     {"128x256_w2x2", 128, 256, 256},
-    {"256x256_dma_w4_k64x4", 256, 256, 256},
-    {"256x256_dma_w8_k128x2", 256, 256, 512},
-    {"256x256_dma_w4x128_k128x2", 256, 256, 256},
     {"256x256_dma_w4x128_m16x128", 256, 256, 256},
     {"rows64x16_k8_m16x128", 64, 16, 512},
 };
-constexpr int kSmallTile = 2, kDma = 5, kDma8 = 6, kDma4 = 7, kM16 = 8, kSkinny = 9;
+constexpr int kSmallTile = 2, kM16 = 5, kSkinny = 6;
 constexpr int kNumVariants = sizeof(kVariants) / sizeof(kVariants[0]);
 
 template <int BM, int BN, int WM, int WN, int CBSZ, int BLGP>
@@ -163,16 +153,9 @@ int launch_one(const GemmArgs& g, hipStream_t st)
 {
     auto kern = gemm_fp8_kernel<BM, BN, WM, WN, CBSZ, BLGP>;
     constexpr int lds_bytes = 2 * (BM + BN) * BK;
-    static bool configured = false;  // the attribute is per function; setting it twice is harmless
-    if (!configured) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
-        if (e != hipSuccess) {
-            set_error("mi8_gemm_fp8: cannot reserve %d bytes of LDS: %s", lds_bytes, hipGetErrorString(e));
-            return MI8_ERR_LAUNCH;
-        }
-        configured = true;
-    }
+    static std::atomic<uint64_t> configured{0};
+    if (int rc = reserve_dynamic_lds(reinterpret_cast<const void*>(kern), lds_bytes, configured, "mi8_gemm_fp8"))
+        return rc;
     const int total = g.tiles_m * g.tiles_n;
     const int blocks = ((total + 7) / 8) * 8;
     hipLaunchKernelGGL(kern, dim3(blocks), dim3(WM * WN * 64), lds_bytes, st, g);
@@ -231,7 +214,7 @@ extern "C" int mi8_gemm_fp8(const void* a, int a_dtype, int64_t lda, const void*
     GemmArgs g{(const uint8_t*)a, (const uint8_t*)b, out, out_dtype == MI8_F32 ? 1 : 0, lda, ldb, ldc, (int)M, (int)N, (int)K,
                sa, sb, sa_is_vector ? 1 : 0, sb_is_vector ? 1 : 0, 0, 0};
     hipStream_t st = (hipStream_t)stream;
-    const bool dma_ok = (K % 64 == 0) && M >= 256 && N >= 256 && N % 8 == 0 && ldc % 8 == 0 && aligned16(out) &&
+    const bool dma_ok = (K % 128 == 0) && M >= 256 && N >= 256 && N % 8 == 0 && ldc % 8 == 0 && aligned16(out) &&
                         out_dtype == MI8_BF16 && (!sb_is_vector || aligned16(sb)) &&
                         (sa_is_vector != 0) == (sb_is_vector != 0);
     // measured on MI355X on the benchmark configurations' shapes: the four-wave layout beats the eight-wave one
@@ -244,20 +227,17 @@ extern "C" int mi8_gemm_fp8(const void* a, int a_dtype, int64_t lda, const void*
         if (M <= kSkinnyMaxM)
             variant = kSkinny;
         else if (dma_ok)
-            variant = tiles256 <= 96 ? kSmallTile : (K % 128 == 0 ? kM16 : kDma);
+            variant = tiles256 <= 96 ? kSmallTile : kM16;
         else
             variant = tiles256 <= 384 ? kSmallTile : 1;
     }
     if (variant == kSkinny) return launch_skinny(g, a_dtype, b_dtype, st);
-    if (variant == kDma8 && dma_ok && K % 128 == 0) return launch_dma8(g, a_dtype, b_dtype, st);
-    if (variant == kDma4 && dma_ok && K % 128 == 0) return launch_dma4(g, a_dtype, b_dtype, st);
-    if (variant == kM16 && dma_ok && K % 128 == 0) return launch_m16(g, a_dtype, b_dtype, st);
-    if (variant == kDma || variant == kDma8 || variant == kDma4 || variant == kM16) {
-        MI8_REQUIRE(dma_ok && variant == kDma, MI8_ERR_UNSUPPORTED,
-                    "mi8_gemm_fp8: the direct-to-LDS variant needs M, N >= 256, K %% 64 == 0 (8 waves: 128), N %% 8 == 0, ldc %% 8 == 0, "
+    if (variant == kM16) {
+        MI8_REQUIRE(dma_ok, MI8_ERR_UNSUPPORTED,
+                    "mi8_gemm_fp8: the direct-to-LDS variant needs M, N >= 256, K %% 128 == 0, N %% 8 == 0, ldc %% 8 == 0, "
                     "scales that are both single values or both vectors, and a 16-byte aligned bf16 output (M=%lld N=%lld K=%lld ldc=%lld)",
                     (long long)M, (long long)N, (long long)K, (long long)ldc);
-        return launch_dma(g, a_dtype, b_dtype, st);
+        return launch_m16(g, a_dtype, b_dtype, st);
     }
     if (a_dtype == MI8_E4M3)
         return b_dtype == MI8_E4M3 ? launch_variant<0, 0>(variant, g, st) : launch_variant<0, 1>(variant, g, st);

@@ -1,6 +1,5 @@
 // Persistent fp8 GEMM on 16x16x128 MFMAs: four waves of 128 x 128 per 256 x 256 workgroup tile, direct
-// global->LDS loads of full 128-byte rows.  Same problems, tile order and LDS budget as the 32x32x64 kernel
-// (mi8_gemm_dma8.hip); for full 256 x 256 tiles, K % 128 == 0, bf16 output.
+// global->LDS loads of full 128-byte rows; for full 256 x 256 tiles, K % 128 == 0, bf16 output.
 //
 // Why this MFMA shape: an MI355X running fp8 MFMAs on random operands is power limited (it clocks down to
 // 1.7-1.9 GHz), so throughput follows energy per flop, and v_mfma_f32_16x16x128_f8f6f4 needs less of it than
@@ -136,8 +135,9 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_fp8_m16_kernel(Problem pb)
         ++ld_seq;
     };
 
-    // ---- this workgroup's tiles (see mi8_gemm_dma8.hip: XCD-contiguous ranges for tiles of equal cost, plain
-    // striding for tiles of unequal cost)
+    // ---- this workgroup's tiles.  Workgroup ids are dealt round-robin to the 8 XCDs, each with its own L2: for tiles
+    // of equal cost every XCD takes a contiguous range of the tile order (neighbouring tiles share operand panels),
+    // its workgroups striding through it; tiles of unequal cost are strided over the whole grid instead
     const typename Problem::Cache cache = pb.prepare();
     const int total = pb.total_tiles(cache);
     int first_tile, tile_stride, my_tiles;
@@ -419,39 +419,19 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_fp8_m16_kernel(Problem pb)
     __syncthreads();
 }
 
-int num_cus()
-{
-    static int cached = 0;
-    if (cached == 0) {
-        int dev = 0, n = 0;
-        if (hipGetDevice(&dev) != hipSuccess ||
-            hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0)
-            n = 256;
-        cached = n;
-    }
-    return cached;
-}
-
 // persistent: one workgroup per CU walks a static share of the tiles (right when all tiles cost the same);
 // otherwise one workgroup per tile, handed to free CUs by the hardware dispatcher (tiles of unequal cost).
 template <typename Problem, int CBSZ_A, int BLGP_B>
 int launch(const Problem& pb, int max_tiles, bool persistent, hipStream_t st)
 {
     auto kern = gemm_fp8_m16_kernel<Problem, CBSZ_A, BLGP_B>;
-    static bool configured = false;
-    if (!configured) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES);
-        if (e != hipSuccess) {
-            set_error("mi8 16x16x128 GEMM: cannot reserve %d bytes of LDS: %s", LDS_BYTES, hipGetErrorString(e));
-            return MI8_ERR_LAUNCH;
-        }
-        configured = true;
-    }
+    static std::atomic<uint64_t> configured{0};
+    if (int rc = reserve_dynamic_lds(reinterpret_cast<const void*>(kern), LDS_BYTES, configured, "mi8 16x16x128 GEMM"))
+        return rc;
     // Persistent: one workgroup per compute unit, or, for fewer tiles, as many as the tiles need - rounded up to
     // a multiple of 8, because every XCD takes an eighth of the tiles (rounded up) and needs that many
     // workgroups to finish in one round (43 tiles on 43 workgroups: XCDs with 5 workgroups for 6 tiles).
-    int blocks = persistent ? num_cus() : max_tiles;
+    int blocks = persistent ? num_compute_units() : max_tiles;
     const int wanted = persistent ? (max_tiles + 7) / 8 * 8 : max_tiles;
     if (blocks > wanted) blocks = wanted;
     hipLaunchKernelGGL(kern, dim3(blocks), dim3(kThreads), LDS_BYTES, st, pb);

@@ -136,28 +136,13 @@ __global__ __launch_bounds__(kGroupedThreads, 1) void grouped_wgrad_kernel(Group
     gemm_tile_body<GBM, GBN, GWM, GWN, CBSZ, BLGP>(g, tn * GBM, tk * GBN, lds);
 }
 
-template <typename K>
-int reserve_lds(K kern, const char* what)
-{
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                       kGroupedLds);
-    if (e != hipSuccess) {
-        set_error("%s: cannot reserve %d bytes of LDS: %s", what, kGroupedLds, hipGetErrorString(e));
-        return MI8_ERR_LAUNCH;
-    }
-    return MI8_OK;
-}
-
 template <int CBSZ, int BLGP>
 int launch_grouped(const GroupedArgs& a, int blocks, hipStream_t st)
 {
     auto kern = grouped_gemm_kernel<CBSZ, BLGP>;
-    static bool configured = false;
-    if (!configured) {
-        int rc = reserve_lds(kern, "mi8_grouped_gemm_fp8");
-        if (rc != MI8_OK) return rc;
-        configured = true;
-    }
+    static std::atomic<uint64_t> configured{0};
+    if (int rc = reserve_dynamic_lds(reinterpret_cast<const void*>(kern), kGroupedLds, configured, "mi8_grouped_gemm_fp8"))
+        return rc;
     hipLaunchKernelGGL(kern, dim3(blocks), dim3(kGroupedThreads), kGroupedLds, st, a);
     return launch_status("mi8_grouped_gemm_fp8");
 }
@@ -166,12 +151,9 @@ template <int CBSZ, int BLGP>
 int launch_wgrad(const GroupedWgradArgs& a, int blocks, hipStream_t st)
 {
     auto kern = grouped_wgrad_kernel<CBSZ, BLGP>;
-    static bool configured = false;
-    if (!configured) {
-        int rc = reserve_lds(kern, "mi8_grouped_wgrad_fp8");
-        if (rc != MI8_OK) return rc;
-        configured = true;
-    }
+    static std::atomic<uint64_t> configured{0};
+    if (int rc = reserve_dynamic_lds(reinterpret_cast<const void*>(kern), kGroupedLds, configured, "mi8_grouped_wgrad_fp8"))
+        return rc;
     hipLaunchKernelGGL(kern, dim3(blocks), dim3(kGroupedThreads), kGroupedLds, st, a);
     return launch_status("mi8_grouped_wgrad_fp8");
 }
