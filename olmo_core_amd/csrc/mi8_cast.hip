@@ -131,6 +131,16 @@ struct TileCastArgs {
     float* scale_out;  // scalar modes: [1]; per-column mode: [cols]; may be null
 };
 
+// Source row of logical row r when the casts read their input through a token permutation (the rows of a
+// dropless-MoE expert batch: row r is the token that owns slot gather[r], top_k slots per token); -1 for a slot
+// index outside [0, src_rows * top_k) - a dropped token, which reads as a row of zeros.
+__device__ __forceinline__ int64_t gathered_row(const int32_t* gather, int top_k, int64_t src_rows, int64_t r, bool ok)
+{
+    if (!ok) return -1;
+    const int64_t slot = gather[r];
+    return (slot < 0 || slot >= src_rows * top_k) ? -1 : slot / top_k;
+}
+
 // LDS holds the transposed tile as 128 columns x 128 row-bytes.  Two columns share a 256-byte line; the
 // 16-byte chunk index inside the line is XORed with a function of the column's group of eight so that
 // both the dword writes (lanes spread over 16 column groups x 4 row groups) and the 16-byte reads
@@ -151,7 +161,8 @@ __device__ __forceinline__ void tile_cast_body(const void* x, int64_t row_end, i
                                                const float (&sc)[8], uint8_t* out, int64_t ld_out, uint8_t* out_t, int64_t ld_t,
                                                int64_t dst0, int64_t dst_end, uint32_t* lds_t,
                                                uint8_t* out_r = nullptr, int64_t ld_r = 0, const float* row_scale = nullptr,
-                                               int64_t row_scale_row0 = 0)
+                                               int64_t row_scale_row0 = 0, const int32_t* gather = nullptr, int top_k = 1,
+                                               int64_t src_rows = 0)
 {
     const int tid = threadIdx.x;
     const int wave = tid >> 6, lane = tid & 63;
@@ -166,8 +177,13 @@ __device__ __forceinline__ void tile_cast_body(const void* x, int64_t row_end, i
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
             const int64_t r = row0 + 32 * wave + 16 * it + 4 * g + j;
-            const bool ok = col_ok && r < row_end;
-            HpVec<HP>::load8(xb + (r * cols + c8) * HpVec<HP>::kBytes, ok, f[it][j]);
+            bool ok = col_ok && r < row_end;
+            int64_t src = r;
+            if (gather) {  // row r of the expert-sorted side is row gather[r] / top_k of x (uniform branch)
+                src = gathered_row(gather, top_k, src_rows, r, r < row_end);
+                ok = ok && src >= 0;
+            }
+            HpVec<HP>::load8(xb + (src * cols + c8) * HpVec<HP>::kBytes, ok, f[it][j]);
         }
 
     // the rows' own scales, read ahead of the stores below (a read placed between them would wait for them)
@@ -413,6 +429,11 @@ struct GroupedCastArgs {
     uint8_t* out_r;      // [T, ld_r] or null
     int64_t ld_r;
     float* row_scale;    // [T]
+    // optional token permutation in front of the cast (mi8_moe_gather_cast): row r of the [T, cols] input is row
+    // gather[r] / top_k of x [src_rows, cols]
+    const int32_t* gather;
+    int top_k;
+    int64_t src_rows;
 };
 
 // Tile p of the padded row space (128 rows each; group e owns ceil(m_e / 128) consecutive tiles) -> its group,
@@ -472,10 +493,11 @@ __global__ __launch_bounds__(kThreads) void grouped_colamax_kernel(GroupedCastAr
     for (int i = 0; i < kTile / 16; ++i) {
         const int64_t r = row0 + rg + 16 * i;
         uint32_t rowacc[4] = {0, 0, 0, 0};
-        if (c8 < a.cols && r < row_end) {
+        const int64_t src = a.gather ? gathered_row(a.gather, a.top_k, a.src_rows, r, r < row_end) : r;
+        if (c8 < a.cols && r < row_end && src >= 0) {
 #pragma unroll
             for (int k = 0; k < NV; ++k) {
-                const uint4 v = reinterpret_cast<const uint4*>(xb + (r * a.cols + c8) * HpVec<HP>::kBytes)[k];
+                const uint4 v = reinterpret_cast<const uint4*>(xb + (src * a.cols + c8) * HpVec<HP>::kBytes)[k];
                 absmax_accumulate<HP>(v, acc[k]);
                 if (a.row_amax) absmax_accumulate<HP>(v, rowacc);
             }
@@ -751,7 +773,7 @@ __global__ __launch_bounds__(kThreads) void grouped_tile_cast_kernel(GroupedCast
     for (int i = 0; i < 8; ++i) sc[i] = s_scale[8 * cl + i];
     const int64_t dst0 = (int64_t)kTile * blockIdx.y;
     tile_cast_body<HP, FP8, SW>(a.x, row_end, a.cols, row0, col0, sc, nullptr, 0, a.out_t, a.ld_t, dst0, a.ld_t, lds_t,
-                                a.out_r, a.ld_r, s_row_scale, row0);
+                                a.out_r, a.ld_r, s_row_scale, row0, a.gather, a.top_k, a.src_rows);
 }
 
 // ---- dispatch helpers ------------------------------------------------------------------------------
@@ -1229,9 +1251,11 @@ namespace {
 int grouped_cast_launch(const char* what, const void* x, int hp_dtype, int64_t T, int64_t cols, const int64_t* group_sizes,
                         int32_t num_groups, int fp8_dtype, uint32_t flags, uint32_t* amax_ws, void* out_t, int64_t ld_t,
                         float* scale_out, uint32_t* row_amax_ws, void* out_rows, int64_t ld_rows, float* row_scale_out,
-                        void* stream)
+                        void* stream, const int32_t* gather = nullptr, int32_t top_k = 1, int64_t src_rows = 0)
 {
     MI8_REQUIRE(x && group_sizes && amax_ws && out_t && scale_out, MI8_ERR_ARG, "%s: null pointer", what);
+    MI8_REQUIRE(!gather || (top_k > 0 && src_rows > 0 && src_rows * top_k < ((int64_t)1 << 31)), MI8_ERR_ARG,
+                "%s: a gathered input needs top_k > 0 and fewer than 2^31 token slots", what);
     MI8_REQUIRE(valid_hp(hp_dtype) && valid_fp8(fp8_dtype), MI8_ERR_ARG, "%s: unknown dtype", what);
     MI8_REQUIRE(T > 0 && cols > 0 && num_groups > 0, MI8_ERR_ARG, "%s: empty input", what);
     MI8_REQUIRE(cols % 16 == 0, MI8_ERR_UNSUPPORTED, "%s: cols (%lld) must be a multiple of 16", what, (long long)cols);
@@ -1247,7 +1271,7 @@ int grouped_cast_launch(const char* what, const void* x, int hp_dtype, int64_t T
     MI8_REQUIRE(ptiles <= 65535, MI8_ERR_UNSUPPORTED, "%s: too many row tiles (%lld)", what, (long long)ptiles);
     const bool pow2 = (flags & MI8_FLAG_POW2_SCALE) != 0;
     GroupedCastArgs a{x, T, cols, group_sizes, num_groups, pow2, amax_ws, (uint8_t*)out_t, ld_t, scale_out,
-                      out_rows ? row_amax_ws : nullptr, (uint8_t*)out_rows, ld_rows, row_scale_out};
+                      out_rows ? row_amax_ws : nullptr, (uint8_t*)out_rows, ld_rows, row_scale_out, gather, top_k, src_rows};
     hipStream_t st = (hipStream_t)stream;
     dim3 grid((unsigned)ceil_div(cols, kTile), (unsigned)ptiles);
     int rc = MI8_OK;
@@ -1338,4 +1362,20 @@ extern "C" int mi8_grouped_swiglu_bwd(const void* x1, const void* x2, const void
     GroupedSwigluArgs a{(const uint4*)x1, (const uint4*)x2, (const uint4*)gh, (uint4*)g1, (uint4*)g2, T, cols, group_sizes,
                         num_groups, amax_ws1, row_amax_ws1, amax_ws2, row_amax_ws2};
     return grouped_swiglu_launch("mi8_grouped_swiglu_bwd", a, true, stream);
+}
+
+extern "C" int mi8_moe_gather_cast_rows_and_colwise_t(const void* x, int hp_dtype, int64_t tokens, int64_t cols,
+                                                      const int32_t* indices, int32_t top_k, const int64_t* group_sizes,
+                                                      int32_t num_groups, int fp8_dtype, uint32_t flags,
+                                                      uint32_t* amax_ws, void* out_t, int64_t ld_t, float* scale_out,
+                                                      uint32_t* row_amax_ws, void* out_rows, int64_t ld_rows,
+                                                      float* row_scale_out, void* stream)
+{
+    MI8_REQUIRE(indices && out_rows, MI8_ERR_ARG, "mi8_moe_gather_cast_rows_and_colwise_t: null pointer");
+    MI8_REQUIRE(tokens > 0 && top_k > 0, MI8_ERR_ARG, "mi8_moe_gather_cast_rows_and_colwise_t: empty input");
+    MI8_REQUIRE(!(flags & MI8_FLAG_AMAX_READY), MI8_ERR_ARG,
+                "mi8_moe_gather_cast_rows_and_colwise_t: the amax pass is part of this call");
+    return grouped_cast_launch("mi8_moe_gather_cast_rows_and_colwise_t", x, hp_dtype, tokens * top_k, cols, group_sizes,
+                               num_groups, fp8_dtype, flags, amax_ws, out_t, ld_t, scale_out, row_amax_ws, out_rows,
+                               ld_rows, row_scale_out, stream, indices, top_k, tokens);
 }

@@ -498,6 +498,42 @@ def grouped_cast_rows_and_colwise_t(
     return q, row_scale, q_t, scale
 
 
+def gather_cast_rows_and_colwise_t(
+    x: torch.Tensor, indices: torch.Tensor, top_k: int, group_sizes: torch.Tensor, fp8_dtype: torch.dtype, *,
+    pow2: bool = False,
+) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]:
+    """
+    The unweighted token gather of a dropless-MoE layer (row ``i`` of the expert-sorted side is token
+    ``indices[i] // top_k`` of ``x [tokens, cols]``) fused with :func:`grouped_cast_rows_and_colwise_t`: the gathered
+    bf16 tensor is never written.  Returns ``(q [tokens * top_k, cols], row_scale, q_t [cols, ld_t], col_scale [E, cols])``
+    with the bytes and scales of the two-step route.
+    """
+    x = _hp2d(x, "gather_cast_rows_and_colwise_t")
+    tokens, cols = x.shape
+    T = tokens * top_k
+    if indices.dim() != 1 or indices.shape[0] != T or indices.device != x.device:
+        raise ValueError(f"gather_cast_rows_and_colwise_t: expected {T} indices on {x.device}")
+    if indices.dtype != torch.int32 or not indices.is_contiguous():
+        indices = indices.to(torch.int32).contiguous()
+    sizes = _sizes_i64(group_sizes, x.device)
+    E = sizes.numel()
+    ld_t = grouped_padded_rows(T, E)
+    q_t = torch.empty((cols, ld_t), dtype=fp8_dtype, device=x.device)
+    scale = torch.empty((E, cols), dtype=torch.float32, device=x.device)
+    q = torch.empty((T, cols), dtype=fp8_dtype, device=x.device)
+    row_scale = torch.empty(T, dtype=torch.float32, device=x.device)
+    ws = _grouped_amax_workspace(T, cols, E, x.device)
+    _C.check(
+        _C.lib().mi8_moe_gather_cast_rows_and_colwise_t(
+            x.data_ptr(), _HP_CODE[x.dtype], tokens, cols, indices.data_ptr(), top_k, sizes.data_ptr(), E,
+            _FP8_CODE[fp8_dtype], _flags(pow2), ws.data_ptr(), q_t.data_ptr(), ld_t, scale.data_ptr(),
+            ws.data_ptr() + 4 * E * cols, q.data_ptr(), cols, row_scale.data_ptr(), _stream(x),
+        ),
+        "mi8_moe_gather_cast_rows_and_colwise_t",
+    )
+    return q, row_scale, q_t, scale
+
+
 _ONE_GROUP: dict = {}
 
 

@@ -31,9 +31,12 @@ STAGE_SINK = None
 
 class _Float8DroplessMLP(torch.autograd.Function):
     @staticmethod
-    def forward(ctx, x, w1, w2, w3, sizes, num_experts, pow2):
+    def forward(ctx, x, w1, w2, w3, sizes, num_experts, pow2, indices=None, top_k=1):
+        # indices: None - the rows of x are already sorted by expert; else x is [tokens, D] in token order and row i
+        # of the expert-sorted side is token indices[i] // top_k: the gather is fused into the casts of x
         E = num_experts
-        T, D = x.shape
+        D = x.shape[1]
+        T = x.shape[0] if indices is None else x.shape[0] * top_k
         H = w1.shape[0] // E
         dev = x.device
         equal = torch.full((E,), H, dtype=torch.int64, device=dev)  # the experts' weights as equal-size groups
@@ -46,7 +49,9 @@ class _Float8DroplessMLP(torch.autograd.Function):
         # operands that are needed in both layouts (by rows for the forward / grad-input GEMMs, by the group's
         # columns for the weight-gradient GEMMs) come out of one pair of passes
         xt = sxc = ht = shc = w1t = s1c = w3t = s3c = w2q = s2r = None
-        if need_w13:
+        if indices is not None:
+            xq, sx, xt, sxc = ops.gather_cast_rows_and_colwise_t(x, indices, top_k, sizes, _E4M3, pow2=pow2)
+        elif need_w13:
             xq, sx, xt, sxc = ops.grouped_cast_rows_and_colwise_t(x, sizes, _E4M3, pow2=pow2)
         else:
             xq, sx = ops.cast_rowwise(x, _E4M3, pow2=pow2)
@@ -79,13 +84,14 @@ class _Float8DroplessMLP(torch.autograd.Function):
         none = x.new_empty(0)
         opt = lambda t: none if t is None else t  # noqa: E731
         ctx.save_for_backward(opt(xt), opt(sxc), x1, x2, opt(ht), opt(shc), opt(w1t), opt(s1c), opt(w3t), opt(s3c),
-                              opt(w2q), opt(s2r), sizes)
+                              opt(w2q), opt(s2r), sizes, opt(indices))
+        ctx.top_k = top_k if indices is not None else 0
         ctx.meta = (E, T, D, H, Hp, pow2, (x.dtype, w1.dtype, w2.dtype, w3.dtype))
         return y
 
     @staticmethod
     def backward(ctx, gy):
-        xt, sxc, x1, x2, ht, shc, w1t, s1c, w3t, s3c, w2q, s2r, sizes = ctx.saved_tensors
+        xt, sxc, x1, x2, ht, shc, w1t, s1c, w3t, s3c, w2q, s2r, sizes, indices = ctx.saved_tensors
         E, T, D, H, Hp, pow2, (x_dt, w1_dt, w2_dt, w3_dt) = ctx.meta
         gy = gy.reshape(T, D).contiguous()
         if gy.dtype != x_dt:
@@ -139,13 +145,22 @@ class _Float8DroplessMLP(torch.autograd.Function):
         def as_param(g, dt):
             return g if g is None or g.dtype == dt else g.to(dt)
 
-        return gx, as_param(gw1, w1_dt), as_param(gw2, w2_dt), as_param(gw3, w3_dt), None, None, None
+        if gx is not None and ctx.top_k:
+            # the gather's backward: every token sums the gradients of its top_k slots (the scatter kernel, unweighted)
+            from ..ops import moe as moe_ops
+
+            gx = moe_ops._scatter(gx, indices, None, ctx.top_k)
+        return gx, as_param(gw1, w1_dt), as_param(gw2, w2_dt), as_param(gw3, w3_dt), None, None, None, None, None
 
 
 @torch.compiler.disable
-def float8_dropless_mlp(x, w1, w2, w3, batch_size_per_expert, num_experts: int, pow2: bool = True):
-    """``gmm(silu(gmm(x, w1^T)) * gmm(x, w3^T), w2)`` with float8 grouped GEMMs; ``x`` is ``[T, d_model]`` bf16."""
-    return _Float8DroplessMLP.apply(x, w1, w2, w3, batch_size_per_expert, num_experts, pow2)
+def float8_dropless_mlp(x, w1, w2, w3, batch_size_per_expert, num_experts: int, pow2: bool = True, indices=None,
+                        top_k: int = 1):
+    """``gmm(silu(gmm(x, w1^T)) * gmm(x, w3^T), w2)`` with float8 grouped GEMMs; ``x`` is ``[T, d_model]`` bf16 with
+    rows sorted by expert, or, with ``indices`` (int32 ``[tokens * top_k]``, the slot held by each sorted row),
+    ``[tokens, d_model]`` in token order: the result is then the expert output of the gathered rows,
+    ``[tokens * top_k, d_model]``, and the gather never writes its bf16 result."""
+    return _Float8DroplessMLP.apply(x, w1, w2, w3, batch_size_per_expert, num_experts, pow2, indices, top_k)
 
 
 class DroplessMoEMLP(nn.Module):
@@ -189,6 +204,18 @@ class DroplessMoEMLP(nn.Module):
         y = float8_dropless_mlp(x2, self.w1, self.w2, self.w3, batch_size_per_expert, self.num_experts)
         return y.reshape(*lead, self.d_model).to(x.dtype)
 
+    def forward_gathered(self, x: torch.Tensor, indices: torch.Tensor, top_k: int,
+                         batch_size_per_expert: torch.Tensor) -> torch.Tensor:
+        """``forward(gather(x, indices, ..., top_k), batch_size_per_expert)`` (``olmo_core_amd.ops.moe.gather``) with
+        the gather fused into the quantisation of the expert inputs: ``x`` is ``(tokens, d_model)`` in token order,
+        the result ``(tokens * top_k, d_model)`` in expert order."""
+        x2 = x.reshape(-1, self.d_model)
+        if x2.dtype != torch.bfloat16:
+            x2 = x2.to(torch.bfloat16)
+        y = float8_dropless_mlp(x2, self.w1, self.w2, self.w3, batch_size_per_expert, self.num_experts,
+                                indices=indices, top_k=top_k)
+        return y.to(x.dtype)
+
 
 class ParallelDroplessMLP(nn.Module):
     """
@@ -198,10 +225,12 @@ class ParallelDroplessMLP(nn.Module):
     Single-device path only: expert parallelism needs more than one GPU.
     """
 
-    def __init__(self, *, mlp: DroplessMoEMLP, top_k: int):
+    def __init__(self, *, mlp: DroplessMoEMLP, top_k: int, fuse_gather: bool = True):
         super().__init__()
         self.mlp = mlp
         self.top_k = top_k
+        # gather -> quantise in one pass (the gathered bf16 rows are never written); False: the separate gather op
+        self.fuse_gather = fuse_gather
 
     @property
     def d_model(self) -> int:
@@ -248,6 +277,9 @@ class ParallelDroplessMLP(nn.Module):
         from ..ops import moe as moe_ops
 
         x = x.view(-1, x.shape[-1])
-        x = moe_ops.gather(x, indices, bin_ids, bins, top_k)
-        x = self.mlp(x, batch_size_per_expert)
+        if self.fuse_gather and x.is_cuda:
+            x = self.mlp.forward_gathered(x, indices, top_k, batch_size_per_expert)
+        else:
+            x = moe_ops.gather(x, indices, bin_ids, bins, top_k)
+            x = self.mlp(x, batch_size_per_expert)
         return moe_ops.scatter(x, indices, bin_ids, expert_weights, bins, top_k)

@@ -350,3 +350,34 @@ def test_dropless_mlp_stage_by_stage_against_oracle(dev, sizes, dims):
         for i, p in enumerate(mlp.parameters()):
             p.copy_((torch.randn(p.shape, generator=g) * 0.02 * (1 + i)).bfloat16())
     check_dropless_stages(dev, mlp, seeded((T, D), 1), seeded((T, D), 2, std=1e-3), sizes, experts=range(E))
+
+
+@pytest.mark.parametrize("tokens,top_k", [(96, 2), (700, 4)])
+def test_routed_layer_fused_gather_equals_separate_gather(dev, tokens, top_k):
+    """ParallelDroplessMLP with the gather fused into the quantisation of the expert inputs gives the bits of the
+    layer that gathers first (outputs, grad_x, the router-weight gradient and every expert weight gradient)."""
+    E, D, H = 8, 256, 384
+    g = torch.Generator().manual_seed(21)
+    x = seeded((tokens, D), 22)
+    logits = torch.randn(tokens, E, generator=g)
+    logits[:, 3] = -1e9
+    expert_weights, expert_indices = torch.topk(logits.softmax(-1), top_k, dim=-1)
+    sizes = O.batched_histc(expert_indices.reshape(1, -1), E)[0]
+    go = seeded((tokens, D), 23, std=1e-2)
+    mlp = DroplessMoEMLP(d_model=D, hidden_size=H, num_experts=E, dtype=torch.bfloat16)
+    with torch.no_grad():
+        for p_ in mlp.parameters():
+            p_.copy_((torch.randn(p_.shape, generator=g) * 0.02).bfloat16())
+    mlp = mlp.to(dev)
+    results = []
+    for fuse in (True, False):
+        layer = ParallelDroplessMLP(mlp=mlp, top_k=top_k, fuse_gather=fuse)
+        for p_ in mlp.parameters():
+            p_.grad = None
+        xd = x.to(dev).requires_grad_(True)
+        wd = expert_weights.bfloat16().to(dev).requires_grad_(True)
+        out = layer(xd, wd, expert_indices.to(dev), sizes.to(dev))
+        out.backward(go.to(dev))
+        results.append([out.detach(), xd.grad, wd.grad] + [p_.grad.clone() for p_ in mlp.parameters()])
+    for name, a, b in zip(("out", "grad_x", "grad_expert_weights", "grad_w1", "grad_w2", "grad_w3"), *results):
+        assert torch.equal(a, b), name

@@ -124,3 +124,54 @@ def test_errors(dev):
     bad = torch.tensor([0, 1, 99, -5], dtype=torch.int32, device=dev)
     out = ops._gather(torch.ones(4, 8, device=dev), bad, None, 1)
     assert out.cpu().sum(1).tolist() == [8.0, 8.0, 0.0, 0.0]
+
+
+@pytest.mark.parametrize("sl,hs,ne,top_k", [(100, 32, 7, 3), (257, 144, 5, 2), (700, 256, 8, 4), (2048, 512, 64, 8)],
+                         ids=lambda v: str(v))
+@pytest.mark.parametrize("pow2", [True, False], ids=["pow2", ""])
+def test_gather_fused_with_the_grouped_cast(dev, sl, hs, ne, top_k, pow2):
+    """gather -> quantise in one call: bytes and scales equal the two-call route (gather, then the grouped
+    two-product cast) and the oracle (NumPy-loop gather, then the per-expert casts), the gathered bf16 tensor is never
+    written.  An expert without tokens and an out-of-range slot index (a dropped token: a row of zeros) included."""
+    from helpers import E4M3, assert_bytes_equal, assert_scale_equal, u8
+    from olmo_core_amd.float8 import ops as f8
+    from oracle import float8_oracle as O
+
+    x, indices, _, bins, _ = _case(sl, hs, ne, top_k, torch.bfloat16, seed=3)
+    if ne >= 5:  # route everything away from expert 2
+        g = torch.Generator().manual_seed(9)
+        top_expert = torch.randint(0, ne - 1, (sl, top_k), generator=g)
+        top_expert[top_expert >= 2] += 1
+        indices, _, bins = M.indices_and_bins(top_expert, ne)
+    sizes = torch.diff(bins.long(), prepend=torch.zeros(1, dtype=torch.long))
+    d = lambda t: t.to(dev)  # noqa: E731
+    q, srow, q_t, scol = f8.gather_cast_rows_and_colwise_t(d(x), d(indices), top_k, d(sizes), E4M3, pow2=pow2)
+
+    xs_dev = ops._gather(d(x), d(indices), None, top_k)
+    q2, srow2, q_t2, scol2 = f8.grouped_cast_rows_and_colwise_t(xs_dev, d(sizes), E4M3, pow2=pow2)
+    assert torch.equal(u8(q), u8(q2)) and torch.equal(srow.cpu(), srow2.cpu())
+
+    xs = M.gather(x, indices, None, top_k)
+    start = seg = 0
+    for e, n in enumerate(sizes.tolist()):
+        if n:
+            xe = xs[start:start + n]
+            ref_r, ref_sr = O.cast(xe, E4M3, O.AXISWISE, -1, pow2)
+            ref_c, ref_sc = O.cast(xe, E4M3, O.AXISWISE, 0, pow2)
+            assert_scale_equal(srow[start:start + n], ref_sr, f"expert {e}: row scales")
+            assert_scale_equal(scol[e], ref_sc, f"expert {e}: column scales")
+            assert_scale_equal(scol[e], scol2[e], f"expert {e}: column scales vs two-call route")
+            assert_bytes_equal(q[start:start + n], ref_r, what=f"expert {e}: per-row bytes")
+            assert_bytes_equal(q_t[:, seg:seg + n], ref_c.t(), what=f"expert {e}: per-column bytes")
+            pad = (n + 127) // 128 * 128
+            assert torch.equal(u8(q_t[:, seg:seg + pad]), u8(q_t2[:, seg:seg + pad])), f"expert {e}: transposed copy"
+            seg += pad
+        start += n
+
+    # a slot index that points nowhere reads as a row of zeros (zero bytes; scale of an all-zero row)
+    bad = indices.clone()
+    bad[0] = sl * top_k + 5
+    qb, srb, _, _ = f8.gather_cast_rows_and_colwise_t(d(x), d(bad), top_k, d(sizes), E4M3, pow2=pow2)
+    assert int(u8(qb[0]).max()) == 0
+    assert_scale_equal(srb[0:1], O.amax_to_scale(torch.zeros(1, 1, dtype=torch.bfloat16), E4M3, pow2))
+    assert torch.equal(u8(qb[1:]), u8(q[1:]))
