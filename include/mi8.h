@@ -153,6 +153,16 @@ int mi8_gemm_fp8(const void* a, int a_dtype, int64_t lda, const void* b, int b_d
                  int64_t N, int64_t K, const float* sa, int sa_is_vector, const float* sb, int sb_is_vector,
                  void* out, int out_dtype, int64_t ldc, int variant, void* stream);
 
+/* out[M, N] += the product mi8_gemm_fp8 would write: the new term is rounded to out_dtype first and the sum of the
+ * two is formed in float32 and rounded once, i.e. exactly what `out = out + gemm(...)` gives when both terms are
+ * tensors of out_dtype.  This is how the grad_input of a block whose input feeds two linears (w1 and w3 of the
+ * feed-forward block, src/olmo_core/nn/feed_forward.py:171) is summed by autograd; here the second GEMM adds into the
+ * first one's output and the separate elementwise pass over [M, N] disappears.  Arguments as mi8_gemm_fp8 (the kernel
+ * is chosen by shape). */
+int mi8_gemm_fp8_accumulate(const void* a, int a_dtype, int64_t lda, const void* b, int b_dtype, int64_t ldb, int64_t M,
+                            int64_t N, int64_t K, const float* sa, int sa_is_vector, const float* sb, int sb_is_vector,
+                            void* out, int out_dtype, int64_t ldc, void* stream);
+
 /* The same product with K cut into `splits` slices, for problems whose few output tiles would leave most of the
  * GPU idle (a few hundred rows of A against a weight matrix): every slice is summed by its own workgroups into
  * an fp32 plane of `workspace`, a second kernel adds the planes in slice order (results do not depend on
@@ -224,6 +234,13 @@ int mi8_grouped_gemm_fp8(const void* a, int a_dtype, int64_t lda, const void* b,
                          int64_t b_group_stride, const int64_t* group_sizes, int32_t num_groups, int64_t T, int64_t N,
                          int64_t K, const float* sa, const float* sb, int64_t sb_group_stride, void* out,
                          int out_dtype, int64_t ldc, void* stream);
+
+/* out[R_e, :N] += that product, summed as mi8_gemm_fp8_accumulate does (the two grad_input terms of the expert
+ * layer, src/olmo_core/nn/moe/mlp.py:286-291). */
+int mi8_grouped_gemm_fp8_accumulate(const void* a, int a_dtype, int64_t lda, const void* b, int b_dtype, int64_t ldb,
+                                    int64_t b_group_stride, const int64_t* group_sizes, int32_t num_groups, int64_t T,
+                                    int64_t N, int64_t K, const float* sa, const float* sb, int64_t sb_group_stride,
+                                    void* out, int out_dtype, int64_t ldc, void* stream);
 
 /* out[e, :N, :Kl] = (A_t[:N, S_e] . B_t[:Kl, S_e]^T) / sa[e, n] / sb[e, k]: the contraction runs over group e's
  * 128-aligned segment S_e of the padded token axis (layout written by mi8_grouped_cast_colwise_t; both operands

@@ -60,6 +60,11 @@ _SIGNATURES = {
         [c_void_p, c_int, c_int64, c_void_p, c_int, c_int64, c_int64, c_int64, c_int64, c_void_p, c_int, c_void_p,
          c_int, c_void_p, c_int, c_int64, c_int, c_void_p],
     ),
+    "mi8_gemm_fp8_accumulate": (
+        c_int,
+        [c_void_p, c_int, c_int64, c_void_p, c_int, c_int64, c_int64, c_int64, c_int64, c_void_p, c_int, c_void_p,
+         c_int, c_void_p, c_int, c_int64, c_void_p],
+    ),
     "mi8_gemm_fp8_splitk": (
         c_int,
         [c_void_p, c_int, c_int64, c_void_p, c_int, c_int64, c_int64, c_int64, c_int64, c_void_p, c_int, c_void_p,
@@ -131,6 +136,11 @@ _SIGNATURES = {
          c_int64, c_void_p, c_void_p, c_void_p, c_int64, c_void_p, c_void_p],
     ),
     "mi8_grouped_gemm_fp8": (
+        c_int,
+        [c_void_p, c_int, c_int64, c_void_p, c_int, c_int64, c_int64, c_void_p, c_int32, c_int64, c_int64, c_int64,
+         c_void_p, c_void_p, c_int64, c_void_p, c_int, c_int64, c_void_p],
+    ),
+    "mi8_grouped_gemm_fp8_accumulate": (
         c_int,
         [c_void_p, c_int, c_int64, c_void_p, c_int, c_int64, c_int64, c_void_p, c_int32, c_int64, c_int64, c_int64,
          c_void_p, c_void_p, c_int64, c_void_p, c_int, c_int64, c_void_p],

@@ -22,7 +22,9 @@ struct GemmArgs {
     const float* sb;
     int sa_vec, sb_vec;
     int tiles_m, tiles_n;
+    int accumulate;  // add the rounded product to what C holds (the sum of two grad_input halves) instead of overwriting
 };
+
 
 __device__ __forceinline__ int swz(int r) { return (r ^ (r >> 3)) & 7; }
 
@@ -39,6 +41,21 @@ __device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi)
 {
     const f32x2_t f = {lo, hi};
     return __builtin_bit_cast(uint32_t, __builtin_convertvector(f, bf16x2_t));
+}
+
+// bf16(a) + bf16(b) for eight packed values, each sum formed in float32 and rounded once (what an elementwise add of
+// two bf16 tensors computes)
+__device__ __forceinline__ v4i add_bf16x8(v4i a, v4i b)
+{
+    v4i r;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const uint32_t x = (uint32_t)a[i], y = (uint32_t)b[i];
+        const float lo = bits_to_f32(x << 16) + bits_to_f32(y << 16);
+        const float hi = bits_to_f32(x & 0xFFFF0000u) + bits_to_f32(y & 0xFFFF0000u);
+        r[i] = (int)pack_bf16x2(lo, hi);
+    }
+    return r;
 }
 
 // Linear tile index -> tile coordinates: tiles are walked in groups of 8 tile-rows (all columns of the group
@@ -74,7 +91,7 @@ __device__ __forceinline__ bool tile_of_block(const GemmArgs& g, int& tm, int& t
 
 // persistent direct-to-LDS kernel, four waves of 128 x 128 on 16x16x128 MFMAs (mi8_gemm_m16.hip); requires
 // M, N >= 256, K % 128 == 0, N % 8 == 0, ldc % 8 == 0, a 16-byte aligned bf16 output
-int launch_m16(GemmArgs& g, int a_dtype, int b_dtype, hipStream_t st);
+int launch_m16(GemmArgs& g, int a_dtype, int b_dtype, hipStream_t st);  // (honours g.accumulate)
 // a few rows of A (M <= kSkinnyMaxM) against all of B, bound by reading B once (mi8_gemm_skinny.hip): any N,
 // K % 16 == 0, any mix of single scales and scale vectors, bf16 or fp32 output
 constexpr int kSkinnyMaxM = 64;
@@ -83,7 +100,8 @@ int launch_skinny(GemmArgs& g, int a_dtype, int b_dtype, hipStream_t st);
 // forward / grad_input (T, N >= 256, K % 128 == 0) and grad_weight (N, Kl >= 256)
 int launch_m16_grouped(const uint8_t* a, int a_dtype, int64_t lda, const uint8_t* b, int b_dtype, int64_t ldb,
                        int64_t b_group_stride, const int64_t* sizes, int E, int64_t T, int N, int K, const float* sa,
-                       const float* sb, int64_t sb_group_stride, uint16_t* out, int64_t ldc, hipStream_t st);
+                       const float* sb, int64_t sb_group_stride, uint16_t* out, int64_t ldc, bool accumulate,
+                       hipStream_t st);
 int launch_m16_grouped_wgrad(const uint8_t* a_t, int a_dtype, const uint8_t* b_t, int b_dtype, int64_t ld_t,
                              const int64_t* sizes, int E, int64_t T, int N, int Kl, const float* sa, const float* sb,
                              uint16_t* out, hipStream_t st);

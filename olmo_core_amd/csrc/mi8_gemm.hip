@@ -191,9 +191,10 @@ extern "C" const char* mi8_gemm_variant_name(int variant)
     return (variant >= 0 && variant < kNumVariants) ? kVariants[variant].name : nullptr;
 }
 
-extern "C" int mi8_gemm_fp8(const void* a, int a_dtype, int64_t lda, const void* b, int b_dtype, int64_t ldb,
-                            int64_t M, int64_t N, int64_t K, const float* sa, int sa_is_vector, const float* sb,
-                            int sb_is_vector, void* out, int out_dtype, int64_t ldc, int variant, void* stream)
+namespace {
+int gemm_fp8_entry(const void* a, int a_dtype, int64_t lda, const void* b, int b_dtype, int64_t ldb, int64_t M, int64_t N,
+                   int64_t K, const float* sa, int sa_is_vector, const float* sb, int sb_is_vector, void* out,
+                   int out_dtype, int64_t ldc, int variant, bool accumulate, void* stream)
 {
     MI8_REQUIRE(a && b && sa && sb && out, MI8_ERR_ARG, "mi8_gemm_fp8: null pointer");
     MI8_REQUIRE((a_dtype == MI8_E4M3 || a_dtype == MI8_E5M2) && (b_dtype == MI8_E4M3 || b_dtype == MI8_E5M2),
@@ -212,11 +213,13 @@ extern "C" int mi8_gemm_fp8(const void* a, int a_dtype, int64_t lda, const void*
     MI8_REQUIRE(out_dtype == MI8_BF16 || out_dtype == MI8_F32, MI8_ERR_ARG, "mi8_gemm_fp8: unknown output dtype %d",
                 out_dtype);
     GemmArgs g{(const uint8_t*)a, (const uint8_t*)b, out, out_dtype == MI8_F32 ? 1 : 0, lda, ldb, ldc, (int)M, (int)N, (int)K,
-               sa, sb, sa_is_vector ? 1 : 0, sb_is_vector ? 1 : 0, 0, 0};
+               sa, sb, sa_is_vector ? 1 : 0, sb_is_vector ? 1 : 0, 0, 0, accumulate ? 1 : 0};
     hipStream_t st = (hipStream_t)stream;
+    // (the persistent kernel shifts its last tile row / column back over the previous one when M or N is not a
+    // multiple of 256 and rewrites the overlap with identical values: not possible when accumulating)
     const bool dma_ok = (K % 128 == 0) && M >= 256 && N >= 256 && N % 8 == 0 && ldc % 8 == 0 && aligned16(out) &&
                         out_dtype == MI8_BF16 && (!sb_is_vector || aligned16(sb)) &&
-                        (sa_is_vector != 0) == (sb_is_vector != 0);
+                        (sa_is_vector != 0) == (sb_is_vector != 0) && (!accumulate || (M % 256 == 0 && N % 256 == 0));
     // measured on MI355X on the benchmark configurations' shapes: the four-wave layout beats the eight-wave one
     // by 0-14 %, and its 16x16x128 form beats its 32x32x64 form by 3-9 % (random operands, power-limited clocks).
     // Problems with few 256 x 256 tiles leave most compute units idle and pay one memory latency per K step:
@@ -224,13 +227,15 @@ extern "C" int mi8_gemm_fp8(const void* a, int a_dtype, int64_t lda, const void*
     // rows of A go to the kernel that streams B once.
     if (variant < 0) {
         const int64_t tiles256 = ((M + 255) / 256) * ((N + 255) / 256);
-        if (M <= kSkinnyMaxM)
+        if (M <= kSkinnyMaxM && !accumulate)
             variant = kSkinny;
         else if (dma_ok)
             variant = tiles256 <= 96 ? kSmallTile : kM16;
         else
             variant = tiles256 <= 384 ? kSmallTile : 1;
     }
+    MI8_REQUIRE(!(accumulate && variant == kSkinny), MI8_ERR_UNSUPPORTED,
+                "mi8_gemm_fp8_accumulate: the few-rows variant does not accumulate");
     if (variant == kSkinny) return launch_skinny(g, a_dtype, b_dtype, st);
     if (variant == kM16) {
         MI8_REQUIRE(dma_ok, MI8_ERR_UNSUPPORTED,
@@ -242,6 +247,24 @@ extern "C" int mi8_gemm_fp8(const void* a, int a_dtype, int64_t lda, const void*
     if (a_dtype == MI8_E4M3)
         return b_dtype == MI8_E4M3 ? launch_variant<0, 0>(variant, g, st) : launch_variant<0, 1>(variant, g, st);
     return b_dtype == MI8_E4M3 ? launch_variant<1, 0>(variant, g, st) : launch_variant<1, 1>(variant, g, st);
+}
+}  // namespace
+
+extern "C" int mi8_gemm_fp8(const void* a, int a_dtype, int64_t lda, const void* b, int b_dtype, int64_t ldb,
+                            int64_t M, int64_t N, int64_t K, const float* sa, int sa_is_vector, const float* sb,
+                            int sb_is_vector, void* out, int out_dtype, int64_t ldc, int variant, void* stream)
+{
+    return gemm_fp8_entry(a, a_dtype, lda, b, b_dtype, ldb, M, N, K, sa, sa_is_vector, sb, sb_is_vector, out, out_dtype,
+                          ldc, variant, false, stream);
+}
+
+extern "C" int mi8_gemm_fp8_accumulate(const void* a, int a_dtype, int64_t lda, const void* b, int b_dtype, int64_t ldb,
+                                       int64_t M, int64_t N, int64_t K, const float* sa, int sa_is_vector,
+                                       const float* sb, int sb_is_vector, void* out, int out_dtype, int64_t ldc,
+                                       void* stream)
+{
+    return gemm_fp8_entry(a, a_dtype, lda, b, b_dtype, ldb, M, N, K, sa, sa_is_vector, sb, sb_is_vector, out, out_dtype,
+                          ldc, -1, true, stream);
 }
 
 extern "C" int mi8_gemm_splitk_suggest(int64_t M, int64_t N, int64_t K)

@@ -157,10 +157,16 @@ __device__ __forceinline__ void gemm_tile_body(const GemmArgs& g, const int m0, 
                 if (!col_ok[j]) continue;
                 const int col = n0 + wn * WTN + j * 32 + l32;
                 const float v = acc[i][j][e] * isa * isb[j];
-                if (g.c_f32)
-                    reinterpret_cast<float*>(g.C)[(int64_t)row * g.ldc + col] = v;
-                else
-                    reinterpret_cast<uint16_t*>(g.C)[(int64_t)row * g.ldc + col] = f32_to_bf16_bits(v);
+                if (g.c_f32) {
+                    float* c = reinterpret_cast<float*>(g.C) + (int64_t)row * g.ldc + col;
+                    *c = g.accumulate ? *c + v : v;
+                } else {
+                    uint16_t* c = reinterpret_cast<uint16_t*>(g.C) + (int64_t)row * g.ldc + col;
+                    uint16_t r = f32_to_bf16_bits(v);
+                    if (g.accumulate)  // both terms are bf16 values, summed in float32 and rounded once
+                        r = f32_to_bf16_bits(bits_to_f32((uint32_t)*c << 16) + bits_to_f32((uint32_t)r << 16));
+                    *c = r;
+                }
             }
         }
     }

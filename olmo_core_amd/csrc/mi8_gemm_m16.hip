@@ -310,6 +310,31 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_fp8_m16_kernel(Problem pb)
         // memory only after the arithmetic of the next pass, so that each pass exposes one LDS round trip instead
         // of two.
         v4i staged[4];  // (an ext-vector type: arrays of HIP's uint4 struct end up in scratch)
+        // Accumulating problems (C += product): what C holds at the addresses of a pass is fetched one pass ahead
+        // of the stores that replace it, with the same coalesced 16-byte accesses, and added to the staged rows as
+        // an elementwise bf16 add would (float32 sum of the two bf16 values, one rounding).
+        v4i held[4];
+        auto load_held = [&](int jq, int ih) __attribute__((always_inline)) {
+            const int rt = wm * WT + ih * 32;
+            if constexpr (Problem::kMaskRows) {
+                const int voff = (rt + (lane >> 3) - td.row_lo) * ldc_bytes + (wn * WT + jq * 64 + (lane & 7) * 8) * 2;
+#pragma unroll
+                for (int it = 0; it < 4; ++it)  // (rows outside the group read as zeros and are not stored)
+                    held[it] = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(c_rows, voff + it * 8 * ldc_bytes, 0, 0));
+            } else {
+#pragma unroll
+                for (int it = 0; it < 4; ++it) {
+                    const uint8_t* base = reinterpret_cast<const uint8_t*>(td.c + (int64_t)(rt + it * 8) * pb.ldc + wn * WT + jq * 64);
+                    uint32_t o = c_lane_off;
+                    asm volatile("" : "+v"(o));
+                    held[it] = *reinterpret_cast<const v4i*>(base + o);
+                }
+            }
+        };
+        auto add_held = [&]() __attribute__((always_inline)) {
+#pragma unroll
+            for (int it = 0; it < 4; ++it) staged[it] = add_bf16x8(staged[it], held[it]);
+        };
         auto store_staged = [&](int jq, int ih) __attribute__((always_inline)) {
             const int rt = wm * WT + ih * 32;  // first tile row of the pass
             if constexpr (Problem::kMaskRows) {
@@ -381,8 +406,12 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_fp8_m16_kernel(Problem pb)
                 if (jq + ih > 0) {
                     // the previous pass's rows have arrived in registers (so its staging area is free again)
                     __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0)
-                    store_staged(ih == 0 ? jq - 1 : jq, ih == 0 ? 3 : ih - 1);
+                    if constexpr (Problem::kAccumulate) add_held();
                 }
+                // (this pass's old C values are requested before the previous pass's stores are issued: the wait for
+                // them, one pass later, then leaves those stores outstanding)
+                if constexpr (Problem::kAccumulate) load_held(jq, ih);
+                if (jq + ih > 0) store_staged(ih == 0 ? jq - 1 : jq, ih == 0 ? 3 : ih - 1);
 #pragma unroll
                 for (int t = 0; t < 2; ++t)
 #pragma unroll
@@ -407,6 +436,7 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_fp8_m16_kernel(Problem pb)
             }
         }
         __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0)
+        if constexpr (Problem::kAccumulate) add_held();
         store_staged(1, 3);
         // The last step's phase B has read the next tile's first fragments like any other step; reading them
         // again here makes those 96 registers free during the epilogue, which otherwise spills (and every
@@ -454,22 +484,29 @@ int launch_m16(GemmArgs& g, int a_dtype, int b_dtype, hipStream_t st)
 {
     g.tiles_m = (g.M + BM - 1) / BM;
     g.tiles_n = (g.N + BN - 1) / BN;
+    const int tiles = g.tiles_m * g.tiles_n;
     if (g.sa_vec) {
-        DenseProblem<true> pb{g, g.lda, g.ldb, g.ldc};
-        return launch_typed(pb, g.tiles_m * g.tiles_n, true, a_dtype, b_dtype, st);
+        if (g.accumulate) return launch_typed(DenseProblem<true, true>{g, g.lda, g.ldb, g.ldc}, tiles, true, a_dtype, b_dtype, st);
+        return launch_typed(DenseProblem<true>{g, g.lda, g.ldb, g.ldc}, tiles, true, a_dtype, b_dtype, st);
     }
-    DenseProblem<false> pb{g, g.lda, g.ldb, g.ldc};
-    return launch_typed(pb, g.tiles_m * g.tiles_n, true, a_dtype, b_dtype, st);
+    if (g.accumulate) return launch_typed(DenseProblem<false, true>{g, g.lda, g.ldb, g.ldc}, tiles, true, a_dtype, b_dtype, st);
+    return launch_typed(DenseProblem<false>{g, g.lda, g.ldb, g.ldc}, tiles, true, a_dtype, b_dtype, st);
 }
 
 int launch_m16_grouped(const uint8_t* a, int a_dtype, int64_t lda, const uint8_t* b, int b_dtype, int64_t ldb,
                        int64_t b_group_stride, const int64_t* sizes, int E, int64_t T, int N, int K, const float* sa,
-                       const float* sb, int64_t sb_group_stride, uint16_t* out, int64_t ldc, hipStream_t st)
+                       const float* sb, int64_t sb_group_stride, uint16_t* out, int64_t ldc, bool accumulate,
+                       hipStream_t st)
 {
     const int tiles_n = (N + BN - 1) / BN;
-    GroupedProblem pb{a, b, out, lda, ldb, ldc, b_group_stride, sb_group_stride, sizes, E, T, N, K, tiles_n, sa, sb};
-    const int64_t max_tiles = ((T + BM - 1) / BM + E) * tiles_n;
-    return launch_typed(pb, max_tiles > (1 << 30) ? (1 << 30) : (int)max_tiles, true, a_dtype, b_dtype, st);
+    const int64_t max_tiles64 = ((T + BM - 1) / BM + E) * tiles_n;
+    const int max_tiles = max_tiles64 > (1 << 30) ? (1 << 30) : (int)max_tiles64;
+    if (accumulate) {
+        GroupedProblem<true> pb{a, b, out, lda, ldb, ldc, b_group_stride, sb_group_stride, sizes, E, T, N, K, tiles_n, sa, sb};
+        return launch_typed(pb, max_tiles, true, a_dtype, b_dtype, st);
+    }
+    GroupedProblem<false> pb{a, b, out, lda, ldb, ldc, b_group_stride, sb_group_stride, sizes, E, T, N, K, tiles_n, sa, sb};
+    return launch_typed(pb, max_tiles, true, a_dtype, b_dtype, st);
 }
 
 int launch_m16_grouped_wgrad(const uint8_t* a_t, int a_dtype, const uint8_t* b_t, int b_dtype, int64_t ld_t,

@@ -26,11 +26,12 @@ struct NoCache {};
 
 // Dense problem: C[M, N] = A[M, K] . B[N, K]^T.  The last tile row / column is shifted back so that every tile
 // is full (M, N >= 256): the overlap is recomputed with the same K order and rewritten with identical values.
-template <bool VEC>
+template <bool VEC, bool ACC = false>
 struct DenseProblem {
     GemmArgs g;
     int64_t lda, ldb, ldc;
     static constexpr bool kVecScales = VEC;  // both scales are vectors (per row / per column) or both single
+    static constexpr bool kAccumulate = ACC;  // C += the rounded product
     static constexpr bool kMaskRows = false, kXcdRanges = true, kPeelFirstStep = true;
     using Cache = NoCache;
     __device__ __forceinline__ Cache prepare() const { return Cache{}; }
@@ -110,7 +111,9 @@ __device__ __forceinline__ GroupSpan locate_group_cached(const GroupCache& c, co
 // Ragged-M grouped problem (dropless-MoE forward / grad_input): rows of A form consecutive groups, group e
 // multiplies B_e = B + e * b_group_stride.  A tile covers up to 256 rows of ONE group; it always loads a full
 // 256-row window (shifted back at the end of the matrix, T >= 256) and stores only its group's rows.
+template <bool ACC = false>
 struct GroupedProblem {
+    static constexpr bool kAccumulate = ACC;
     const uint8_t* A;
     const uint8_t* B;
     uint16_t* C;
@@ -167,6 +170,7 @@ struct GroupedWgradProblem {
     const float* sa;  // [E, N]
     const float* sb;  // [E, Kl]
     static constexpr bool kVecScales = true, kMaskRows = false, kXcdRanges = false, kPeelFirstStep = true;
+    static constexpr bool kAccumulate = false;
     using Cache = GroupCache;
     __device__ __forceinline__ Cache prepare() const { return build_group_cache<128>(sizes, E, T); }
     __device__ __forceinline__ int total_tiles(const Cache&) const { return E * tiles_n * tiles_k; }

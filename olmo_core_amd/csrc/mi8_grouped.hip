@@ -31,6 +31,7 @@ struct GroupedArgs {
     const float* sa;  // [T]
     const float* sb;  // group e: sb + e * sb_group_stride, N values
     int tiles_n;
+    int accumulate;   // C += the rounded product
 };
 
 template <int CBSZ, int BLGP>
@@ -72,6 +73,7 @@ __global__ __launch_bounds__(kGroupedThreads, 1) void grouped_gemm_kernel(Groupe
     g.sb_vec = 1;
     g.tiles_m = 0;
     g.tiles_n = a.tiles_n;
+    g.accumulate = a.accumulate;
     gemm_tile_body<GBM, GBN, GWM, GWN, CBSZ, BLGP>(g, (mt - tiles_before) * GBM, nt * GBN, lds);
 }
 
@@ -133,6 +135,7 @@ __global__ __launch_bounds__(kGroupedThreads, 1) void grouped_wgrad_kernel(Group
     g.sb_vec = seg ? 1 : 0;
     g.tiles_m = 0;
     g.tiles_n = a.tiles_k;
+    g.accumulate = 0;
     gemm_tile_body<GBM, GBN, GWM, GWN, CBSZ, BLGP>(g, tn * GBM, tk * GBN, lds);
 }
 
@@ -165,10 +168,11 @@ bool fp8_code(int v) { return v == MI8_E4M3 || v == MI8_E5M2; }
 
 using namespace mi8;
 
-extern "C" int mi8_grouped_gemm_fp8(const void* a, int a_dtype, int64_t lda, const void* b, int b_dtype, int64_t ldb,
-                                    int64_t b_group_stride, const int64_t* group_sizes, int32_t num_groups, int64_t T,
-                                    int64_t N, int64_t K, const float* sa, const float* sb, int64_t sb_group_stride,
-                                    void* out, int out_dtype, int64_t ldc, void* stream)
+namespace {
+int grouped_gemm_entry(const void* a, int a_dtype, int64_t lda, const void* b, int b_dtype, int64_t ldb,
+                       int64_t b_group_stride, const int64_t* group_sizes, int32_t num_groups, int64_t T, int64_t N,
+                       int64_t K, const float* sa, const float* sb, int64_t sb_group_stride, void* out, int out_dtype,
+                       int64_t ldc, bool accumulate, void* stream)
 {
     MI8_REQUIRE(a && b && group_sizes && sa && sb && out, MI8_ERR_ARG, "mi8_grouped_gemm_fp8: null pointer");
     MI8_REQUIRE(fp8_code(a_dtype) && fp8_code(b_dtype), MI8_ERR_ARG, "mi8_grouped_gemm_fp8: unknown fp8 dtype");
@@ -184,18 +188,41 @@ extern "C" int mi8_grouped_gemm_fp8(const void* a, int a_dtype, int64_t lda, con
     const int64_t m_tiles = ceil_div(T, GBM) + num_groups;  // every group adds at most one partial tile
     MI8_REQUIRE(m_tiles * tiles_n < ((int64_t)1 << 31), MI8_ERR_UNSUPPORTED, "mi8_grouped_gemm_fp8: grid too large");
     GroupedArgs g{(const uint8_t*)a, (const uint8_t*)b, out, out_dtype == MI8_F32 ? 1 : 0, lda, ldb, ldc,
-                  b_group_stride, sb_group_stride, group_sizes, num_groups, T, (int)N, (int)K, sa, sb, tiles_n};
+                  b_group_stride, sb_group_stride, group_sizes, num_groups, T, (int)N, (int)K, sa, sb, tiles_n,
+                  accumulate ? 1 : 0};
     const int blocks = (int)(m_tiles * tiles_n);
     hipStream_t st = (hipStream_t)stream;
-    // full-tile shapes with bf16 output run on the persistent direct-to-LDS kernel
+    // full-tile shapes with bf16 output run on the persistent direct-to-LDS kernel (which rewrites the overlap of its
+    // shifted last tile column when N is not a multiple of 256: not possible when accumulating)
     if (out_dtype == MI8_BF16 && T >= 256 && N >= 256 && K % 128 == 0 && N % 8 == 0 && ldc % 8 == 0 && aligned16(out) &&
-        sb_group_stride % 4 == 0 && aligned16(sb) && lda < (1 << 23) && ldb < (1 << 23) && ldc < (1 << 22))
+        sb_group_stride % 4 == 0 && aligned16(sb) && lda < (1 << 23) && ldb < (1 << 23) && ldc < (1 << 22) &&
+        (!accumulate || N % 256 == 0))
         return launch_m16_grouped((const uint8_t*)a, a_dtype, lda, (const uint8_t*)b, b_dtype, ldb, b_group_stride,
                                    group_sizes, num_groups, T, (int)N, (int)K, sa, sb, sb_group_stride, (uint16_t*)out,
-                                   ldc, st);
+                                   ldc, accumulate, st);
     if (a_dtype == MI8_E4M3)
         return b_dtype == MI8_E4M3 ? launch_grouped<0, 0>(g, blocks, st) : launch_grouped<0, 1>(g, blocks, st);
     return b_dtype == MI8_E4M3 ? launch_grouped<1, 0>(g, blocks, st) : launch_grouped<1, 1>(g, blocks, st);
+}
+}  // namespace
+
+extern "C" int mi8_grouped_gemm_fp8(const void* a, int a_dtype, int64_t lda, const void* b, int b_dtype, int64_t ldb,
+                                    int64_t b_group_stride, const int64_t* group_sizes, int32_t num_groups, int64_t T,
+                                    int64_t N, int64_t K, const float* sa, const float* sb, int64_t sb_group_stride,
+                                    void* out, int out_dtype, int64_t ldc, void* stream)
+{
+    return grouped_gemm_entry(a, a_dtype, lda, b, b_dtype, ldb, b_group_stride, group_sizes, num_groups, T, N, K, sa, sb,
+                              sb_group_stride, out, out_dtype, ldc, false, stream);
+}
+
+extern "C" int mi8_grouped_gemm_fp8_accumulate(const void* a, int a_dtype, int64_t lda, const void* b, int b_dtype,
+                                               int64_t ldb, int64_t b_group_stride, const int64_t* group_sizes,
+                                               int32_t num_groups, int64_t T, int64_t N, int64_t K, const float* sa,
+                                               const float* sb, int64_t sb_group_stride, void* out, int out_dtype,
+                                               int64_t ldc, void* stream)
+{
+    return grouped_gemm_entry(a, a_dtype, lda, b, b_dtype, ldb, b_group_stride, group_sizes, num_groups, T, N, K, sa, sb,
+                              sb_group_stride, out, out_dtype, ldc, true, stream);
 }
 
 extern "C" int mi8_grouped_wgrad_fp8(const void* a_t, int a_dtype, const void* b_t, int b_dtype, int64_t ld_t,

@@ -227,9 +227,11 @@ def gemm_fp8(
     variant: int = -1,
     out: Optional[torch.Tensor] = None,
     splits: int = -1,
+    accumulate: bool = False,
 ) -> torch.Tensor:
     """
     ``out[M, N] = (a[M, :k] @ b[N, :k].T) / sa / sb`` with fp32 accumulation on the fp8 matrix cores.
+    ``accumulate`` (needs ``out``): ``out += product`` with the bits of ``out + gemm_fp8(...)`` on ``out_dtype`` tensors.
     ``a`` and ``b`` are fp8 tensors whose rows are K-contiguous; ``sa`` / ``sb`` hold one scale or one per row.
     ``out``: an ``[M, N]`` tensor of ``out_dtype`` with contiguous rows (any row pitch) to write into.
     ``splits``: slices of K summed separately and added afterwards (for problems with few output tiles);
@@ -246,6 +248,8 @@ def gemm_fp8(
     K = min(a.shape[1], b.shape[1]) if k is None else k
     if sa.numel() not in (1, M) or sb.numel() not in (1, N):
         raise ValueError(f"gemm_fp8: scale sizes {sa.numel()}, {sb.numel()} do not match M={M}, N={N}")
+    if accumulate and out is None:
+        raise ValueError("gemm_fp8: accumulate needs the tensor to add into (out=)")
     if out is None:
         out = torch.empty((M, N), dtype=out_dtype, device=a.device)
     elif tuple(out.shape) != (M, N) or out.dtype != out_dtype or out.stride(1) != 1 or out.device != a.device:
@@ -255,6 +259,19 @@ def gemm_fp8(
         ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         ev0.record()
     L = _C.lib()
+    if accumulate:
+        _C.check(
+            L.mi8_gemm_fp8_accumulate(
+                a.data_ptr(), _FP8_CODE[a.dtype], a.stride(0), b.data_ptr(), _FP8_CODE[b.dtype], b.stride(0), M, N, K,
+                sa.data_ptr(), int(sa.numel() != 1), sb.data_ptr(), int(sb.numel() != 1),
+                out.data_ptr(), _HP_CODE[out_dtype], out.stride(0), _stream(a),
+            ),
+            "mi8_gemm_fp8_accumulate",
+        )
+        if sink is not None:
+            ev1.record()
+            sink.append((ev0, ev1, (M, N, K)))
+        return out
     if variant >= 0:
         splits = 1
     elif splits < 0:
@@ -567,23 +584,32 @@ def grouped_gemm_fp8(
     b_group_stride: int,
     sb_group_stride: int,
     out_dtype: torch.dtype = torch.bfloat16,
+    accumulate_into: Optional[torch.Tensor] = None,
 ) -> torch.Tensor:
     """
     ``out[rows of group e] = a[rows of group e, :k] @ B_e[:n, :k].T / sa / sb_e`` where ``B_e`` starts
     ``e * b_group_stride`` bytes into ``b`` (row pitch ``b.stride(0)``) and its scales ``e * sb_group_stride``
-    floats into ``sb``.
+    floats into ``sb``.  ``accumulate_into``: a ``[T, n]`` tensor of ``out_dtype`` that the product is added to (the
+    bits of ``accumulate_into + grouped_gemm_fp8(...)``) and that is returned.
     """
     _require_gpu(a, "grouped_gemm_fp8")
     T = a.shape[0]
     sizes = _sizes_i64(group_sizes, a.device)
-    out = torch.empty((T, n), dtype=out_dtype, device=a.device)
+    if accumulate_into is not None:
+        out = accumulate_into
+        if tuple(out.shape) != (T, n) or out.dtype != out_dtype or out.stride(1) != 1 or out.device != a.device:
+            raise ValueError(f"grouped_gemm_fp8: accumulate_into must be a [{T}, {n}] {out_dtype} tensor on {a.device}")
+        fn, what = _C.lib().mi8_grouped_gemm_fp8_accumulate, "mi8_grouped_gemm_fp8_accumulate"
+    else:
+        out = torch.empty((T, n), dtype=out_dtype, device=a.device)
+        fn, what = _C.lib().mi8_grouped_gemm_fp8, "mi8_grouped_gemm_fp8"
     _C.check(
-        _C.lib().mi8_grouped_gemm_fp8(
+        fn(
             a.data_ptr(), _FP8_CODE[a.dtype], a.stride(0), b.data_ptr(), _FP8_CODE[b.dtype], b.stride(0),
             b_group_stride, sizes.data_ptr(), sizes.numel(), T, n, k, sa.data_ptr(), sb.data_ptr(), sb_group_stride,
             out.data_ptr(), _HP_CODE[out_dtype], out.stride(0), _stream(a),
         ),
-        "mi8_grouped_gemm_fp8",
+        what,
     )
     return out
 

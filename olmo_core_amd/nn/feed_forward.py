@@ -109,8 +109,9 @@ class _Float8SwiGLUMLP(torch.autograd.Function):
                 x1, x3, gh, go_dt, pow2=pow2, want_rowmajor=need_x, want_transposed=need_t)
             del gh
             if need_x:
+                # the sum of the two halves as autograd forms it (two bf16 tensors added), by the second GEMM's epilogue
                 gx = ops.gemm_fp8(g1q, sg1, w1q_t, s1, k=H, out_dtype=x_dt)
-                gx = gx + ops.gemm_fp8(g3q, sg3, w3q_t, s3, k=H, out_dtype=x_dt)
+                ops.gemm_fp8(g3q, sg3, w3q_t, s3, k=H, out_dtype=x_dt, out=gx, accumulate=True)
             if need_w1:
                 gw1 = ops.gemm_fp8(g1q_t, sg1, xq_t, sx, out_dtype=x_dt)
             if need_w3:

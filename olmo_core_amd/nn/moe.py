@@ -136,7 +136,8 @@ class _Float8DroplessMLP(torch.autograd.Function):
             if need_x:
                 # gx_e = g_e @ w[e] : contraction over H, the right operand is w[e]^T [D, H], one scale per input channel
                 gx = ops.grouped_gemm_fp8(g1q, sg1, w1t, s1c, sizes, n=D, k=H, b_group_stride=Hp, sb_group_stride=D)
-                gx = gx + ops.grouped_gemm_fp8(g2q, sg2, w3t, s3c, sizes, n=D, k=H, b_group_stride=Hp, sb_group_stride=D)
+                ops.grouped_gemm_fp8(g2q, sg2, w3t, s3c, sizes, n=D, k=H, b_group_stride=Hp, sb_group_stride=D,
+                                     accumulate_into=gx)
             if need_w1:
                 gw1 = ops.grouped_wgrad_fp8(g1t, sg1c, xt, sxc, sizes, tokens=T, out_dtype=x_dt).reshape(E * H, D)
             if need_w3:

@@ -295,3 +295,38 @@ def test_argument_errors(dev):
     rc = L.mi8_gemm_fp8_splitk(b.data_ptr(), 0, 256, b.data_ptr(), 0, 256, 16, 16, 256, one.data_ptr(), 0, one.data_ptr(), 0,
                                out.data_ptr(), 0, 16, 2, small.data_ptr(), small.numel(), 0)
     assert rc != 0 and b"workspace" in L.mi8_last_error()
+
+
+@pytest.mark.parametrize("shape", [(512, 768, 256), (1024, 512, 1152), (300, 272, 144), (64, 512, 256), (2048, 2048, 128)],
+                         ids=lambda s: "x".join(map(str, s)))
+@pytest.mark.parametrize("vec", [False, True], ids=["single-scales", "scale-vectors"])
+@pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float32], ids=["bf16", "f32"])
+def test_accumulating_gemm_equals_gemm_plus_add(dev, shape, vec, out_dtype):
+    """out += product: the bits of `out + gemm(...)` on tensors of the output type (the new term rounded first, the
+    sum formed in float32 and rounded once), on the persistent kernel (full 256-tiles) and on the general one."""
+    M, N, K = shape
+    a, b = seeded((M, K), 31, std=1e-3), seeded((N, K), 32)
+    if vec:
+        aq, sa = ops.cast_rowwise(a.to(dev), E4M3, pow2=True)
+        bq, sb = ops.cast_rowwise(b.to(dev), E4M3, pow2=True)
+    else:
+        aq, _, sa = ops.cast_tensorwise(a.to(dev), E5M2)
+        bq, _, sb = ops.cast_tensorwise(b.to(dev), E4M3)
+    first = (seeded((M, N), 33, std=1e-3 * K ** 0.5).float()).to(out_dtype).to(dev)
+    first[0, 0] = float("inf")
+    first[1, 1] = -0.0
+    term = ops.gemm_fp8(aq, sa, bq, sb, out_dtype=out_dtype)
+    want = first + term
+    got = first.clone()
+    res = ops.gemm_fp8(aq, sa, bq, sb, out_dtype=out_dtype, out=got, accumulate=True)
+    assert res.data_ptr() == got.data_ptr()
+    assert torch.equal(got.view(torch.int16 if out_dtype == torch.bfloat16 else torch.int32),
+                       want.view(torch.int16 if out_dtype == torch.bfloat16 else torch.int32))
+    # a view with a row pitch: only the addressed columns change
+    if out_dtype == torch.bfloat16:
+        wide = torch.full((M, N + 64), 7.0, dtype=out_dtype, device=dev)
+        wide[:, :N] = first
+        ops.gemm_fp8(aq, sa, bq, sb, out_dtype=out_dtype, out=wide[:, :N], accumulate=True)
+        assert torch.equal(wide[:, :N], want) and bool((wide[:, N:] == 7.0).all())
+    with pytest.raises(ValueError):
+        ops.gemm_fp8(aq, sa, bq, sb, out_dtype=out_dtype, accumulate=True)

@@ -381,3 +381,20 @@ def test_routed_layer_fused_gather_equals_separate_gather(dev, tokens, top_k):
         results.append([out.detach(), xd.grad, wd.grad] + [p_.grad.clone() for p_ in mlp.parameters()])
     for name, a, b in zip(("out", "grad_x", "grad_expert_weights", "grad_w1", "grad_w2", "grad_w3"), *results):
         assert torch.equal(a, b), name
+
+
+@pytest.mark.parametrize("sizes,n,k", [([300, 17, 0, 411, 64], 512, 256), ([5, 0, 9, 2], 48, 64), ([700, 1, 0, 323], 256, 1024),
+                                       ([256, 256], 320, 128)], ids=["full-tiles", "small", "full-tiles-k1024", "n320"])
+def test_accumulating_grouped_gemm_equals_gemm_plus_add(dev, sizes, n, k):
+    T, E = sum(sizes), len(sizes)
+    x = seeded((T, k), 41, std=1e-3)
+    w = seeded((E * n, k), 42, std=0.05)
+    sz = torch.tensor(sizes).to(dev)
+    xq, sx = ops.cast_rowwise(x.to(dev), E4M3, pow2=True)
+    wq, sw = ops.cast_rowwise(w.to(dev), E4M3, pow2=True)
+    kw = dict(n=n, k=k, b_group_stride=n * wq.stride(0), sb_group_stride=n)
+    term = ops.grouped_gemm_fp8(xq, sx, wq, sw, sz, **kw)
+    first = seeded((T, n), 43, std=1e-3).to(dev)
+    want = first + term
+    got = ops.grouped_gemm_fp8(xq, sx, wq, sw, sz, accumulate_into=first.clone(), **kw)
+    assert torch.equal(got.view(torch.int16), want.view(torch.int16))
