@@ -49,10 +49,14 @@ def build_mlp(dev):
 # ---- the other benchmark configurations (parity-test shapes; measured with --config N) ----
 
 
-def build_config(n, dev):
-    """Returns (step_fn, flops_per_step, gemms_per_step, flops_per_gemm_launch or None, description)."""
+def build_config(n, dev, keep_float8_weights=False, routed=False):
+    """Returns (step_fn, flops_per_step, gemms_per_step, flops_per_gemm_launch or None, description).
+    Configuration 5 only: `keep_float8_weights` keeps the experts' float8 weight copies from step to step (the
+    steady state of gradient-accumulation micro-batches; by default every step quantises the weights again, as a
+    step that follows an optimizer update must); `routed` times the whole routed layer (token gather fused into
+    the quantisation, experts, weighted scatter back to token order) instead of the experts alone."""
     from olmo_core_amd.float8 import AOFloat8LinearRecipe, Float8Config
-    from olmo_core_amd.nn import DroplessMoEMLP, FeedForward
+    from olmo_core_amd.nn import DroplessMoEMLP, FeedForward, ParallelDroplessMLP
 
     def rand(shape, g, std=1.0):
         return (torch.randn(shape, generator=g) * std).to(torch.bfloat16)
@@ -117,16 +121,37 @@ def build_config(n, dev):
         pmf = rank ** -1.1
         pmf = pmf / pmf.sum()
         logits = torch.randn(T, E, generator=g) + (1.75 * torch.log(pmf)).float()  # Zipf(s=1.1) bias: 7 of 64 experts get no token
-        idx = logits.float().softmax(-1).topk(top_k, dim=-1).indices.reshape(-1)
+        weights, experts = logits.float().softmax(-1).topk(top_k, dim=-1)
+        idx = experts.reshape(-1)
         sizes = torch.bincount(idx, minlength=E)
-        mlp = DroplessMoEMLP(d_model=d, hidden_size=h, num_experts=E, dtype=torch.bfloat16)
+        mlp = DroplessMoEMLP(d_model=d, hidden_size=h, num_experts=E, dtype=torch.bfloat16,
+                             keep_float8_weights=keep_float8_weights)
         with torch.no_grad():
             for p in mlp.parameters():
                 p.copy_(rand(p.shape, g, 0.02))
         mlp = mlp.to(dev)
+        sizes_d = sizes.to(dev)
+        f = float(T * top_k) * 18 * d * h
+        desc = (f"config 5: dropless MoE experts fwd+bwd, 64 experts, {T * top_k} rows, group sizes min {int(sizes.min())} "
+                f"max {int(sizes.max())} empty {int((sizes == 0).sum())}, grouped rowwise")
+        if keep_float8_weights:
+            desc += ", float8 expert weights kept across steps"
+        if routed:
+            layer = ParallelDroplessMLP(mlp=mlp, top_k=top_k)
+            x = rand((T, d), g).to(dev).requires_grad_(True)
+            go = rand((T, d), g, 1e-3).to(dev)
+            w_d = weights.to(torch.bfloat16).to(dev).requires_grad_(True)
+            experts_d = experts.to(dev)
+
+            def fn_routed():
+                x.grad = w_d.grad = None
+                for p in mlp.parameters():
+                    p.grad = None
+                layer(x, w_d, experts_d, sizes_d).backward(go)
+
+            return fn_routed, f, 9, None, desc + f"; whole routed layer from {T} tokens (sort, fused gather, experts, weighted scatter)"
         x = rand((T * top_k, d), g).to(dev).requires_grad_(True)
         go = rand((T * top_k, d), g, 1e-3).to(dev)
-        sizes_d = sizes.to(dev)
 
         def fn():
             x.grad = None
@@ -134,16 +159,13 @@ def build_config(n, dev):
                 p.grad = None
             mlp(x, sizes_d).backward(go)
 
-        f = float(T * top_k) * 18 * d * h
-        desc = (f"config 5: dropless MoE experts fwd+bwd, 64 experts, {T * top_k} rows, group sizes min {int(sizes.min())} "
-                f"max {int(sizes.max())} empty {int((sizes == 0).sum())}, grouped rowwise")
         return fn, f, 9, None, desc
     raise ValueError(n)
 
 
-def run_other_config(n, steps, warmup):
+def run_other_config(n, steps, warmup, keep_float8_weights=False, routed=False):
     dev = torch.device("cuda:0")
-    fn, flops, _, _, desc = build_config(n, dev)
+    fn, flops, _, _, desc = build_config(n, dev, keep_float8_weights, routed)
     for _ in range(warmup):
         fn()
     torch.cuda.synchronize()
@@ -301,6 +323,10 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--config", type=int, default=2, help="benchmark configuration 1..5 (2 is the headline line)")
+    ap.add_argument("--keep-float8-weights", action="store_true",
+                    help="config 5: keep the experts' float8 weight copies across steps (micro-batch steady state)")
+    ap.add_argument("--routed", action="store_true",
+                    help="config 5: time the whole routed layer (fused gather, experts, weighted scatter)")
     ap.add_argument("--traffic-probe", action="store_true", help="workload for the FETCH_SIZE/WRITE_SIZE counter runs")
     ap.add_argument("--gemm", type=str, default=None, metavar="M,N,K[;M,N,K...]",
                     help="time single scaled GEMMs of these shapes (library's choice of kernel) instead of a step")
@@ -321,7 +347,7 @@ def main():
         gemm_shapes([tuple(int(v) for v in part.split(",")) for part in ns.gemm.split(";")], ns.steps, ns.warmup)
         return
     if ns.config != 2:
-        run_other_config(ns.config, ns.steps, ns.warmup)
+        run_other_config(ns.config, ns.steps, ns.warmup, ns.keep_float8_weights, ns.routed)
         return
 
     dev = torch.device("cuda:0")

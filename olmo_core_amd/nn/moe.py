@@ -31,7 +31,7 @@ STAGE_SINK = None
 
 class _Float8DroplessMLP(torch.autograd.Function):
     @staticmethod
-    def forward(ctx, x, w1, w2, w3, sizes, num_experts, pow2, indices=None, top_k=1):
+    def forward(ctx, x, w1, w2, w3, sizes, num_experts, pow2, indices=None, top_k=1, kept=None):
         # indices: None - the rows of x are already sorted by expert; else x is [tokens, D] in token order and row i
         # of the expert-sorted side is token indices[i] // top_k: the gather is fused into the casts of x
         E = num_experts
@@ -56,7 +56,10 @@ class _Float8DroplessMLP(torch.autograd.Function):
         else:
             xq, sx = ops.cast_rowwise(x, _E4M3, pow2=pow2)
         # w1/w3: one scale per output channel (row of w[e]) forward, per input channel of w[e] for grad_input
-        if need[0]:
+        # (kept: the float8 copies of the three weights made by an earlier call and still valid)
+        if kept is not None:
+            (w1q, s1, w1t, s1c), (w3q, s3, w3t, s3c), _ = kept
+        elif need[0]:
             w1q, s1, w1t, s1c = ops.grouped_cast_rows_and_colwise_t(w1, equal, _E4M3, pow2=pow2)
             w3q, s3, w3t, s3c = ops.grouped_cast_rows_and_colwise_t(w3, equal, _E4M3, pow2=pow2)
         else:
@@ -76,7 +79,9 @@ class _Float8DroplessMLP(torch.autograd.Function):
         del h
         # w2[e] is [H, D] and is used as-is (h_e @ w2[e]): its output channel is the column -> transposed copy
         # [D, E*H] with one scale per (expert, column); the by-rows copy is the grad_h GEMM's right operand
-        if any_grad:
+        if kept is not None:
+            w2q, s2r, w2t, s2 = kept[2]
+        elif any_grad:
             w2q, s2r, w2t, s2 = ops.grouped_cast_rows_and_colwise_t(w2, equal, _E4M3, pow2=pow2)
         else:
             w2t, s2 = ops.grouped_cast_colwise_t(w2, equal, _E4M3, pow2=pow2)
@@ -151,17 +156,17 @@ class _Float8DroplessMLP(torch.autograd.Function):
             from ..ops import moe as moe_ops
 
             gx = moe_ops._scatter(gx, indices, None, ctx.top_k)
-        return gx, as_param(gw1, w1_dt), as_param(gw2, w2_dt), as_param(gw3, w3_dt), None, None, None, None, None
+        return gx, as_param(gw1, w1_dt), as_param(gw2, w2_dt), as_param(gw3, w3_dt), None, None, None, None, None, None
 
 
 @torch.compiler.disable
 def float8_dropless_mlp(x, w1, w2, w3, batch_size_per_expert, num_experts: int, pow2: bool = True, indices=None,
-                        top_k: int = 1):
+                        top_k: int = 1, kept=None):
     """``gmm(silu(gmm(x, w1^T)) * gmm(x, w3^T), w2)`` with float8 grouped GEMMs; ``x`` is ``[T, d_model]`` bf16 with
     rows sorted by expert, or, with ``indices`` (int32 ``[tokens * top_k]``, the slot held by each sorted row),
     ``[tokens, d_model]`` in token order: the result is then the expert output of the gathered rows,
     ``[tokens * top_k, d_model]``, and the gather never writes its bf16 result."""
-    return _Float8DroplessMLP.apply(x, w1, w2, w3, batch_size_per_expert, num_experts, pow2, indices, top_k)
+    return _Float8DroplessMLP.apply(x, w1, w2, w3, batch_size_per_expert, num_experts, pow2, indices, top_k, kept)
 
 
 class DroplessMoEMLP(nn.Module):
@@ -175,6 +180,7 @@ class DroplessMoEMLP(nn.Module):
         num_experts: int,
         dtype: torch.dtype = torch.float32,
         init_device: str = "cpu",
+        keep_float8_weights: bool = False,
     ):
         super().__init__()
         if d_model % 16 or hidden_size % 16:
@@ -182,6 +188,11 @@ class DroplessMoEMLP(nn.Module):
         self.d_model = d_model
         self.hidden_size = hidden_size
         self.num_experts = num_experts
+        # Keep the float8 copies of the expert weights (two layouts, 2 bytes per parameter) from one call to the
+        # next for as long as the weights are not modified: the micro-batches of one optimizer step then quantise
+        # the experts once (what enable_fsdp_float8_all_gather does for a Float8Linear).  Off: every call quantises.
+        self.keep_float8_weights = keep_float8_weights
+        self._kept = None
         shape = (num_experts * hidden_size, d_model)
         self.w1 = nn.Parameter(torch.empty(*shape, device=init_device, dtype=dtype))
         self.w2 = nn.Parameter(torch.empty(*shape, device=init_device, dtype=dtype))
@@ -193,6 +204,24 @@ class DroplessMoEMLP(nn.Module):
             if not w.is_meta:
                 nn.init.kaiming_uniform_(w, a=math.sqrt(5))
 
+    def weight_operands(self):
+        """The float8 operands of the three expert weights, ``((w1q, s1, w1t, s1c), (w3q, ...), (w2q, s2r, w2t, s2))``
+        as the expert function makes them itself, kept until a weight is modified or replaced (address and version
+        counter; a write through ``.data`` goes unnoticed).  ``None`` unless ``keep_float8_weights``."""
+        if not self.keep_float8_weights:
+            return None
+        ws = (self.w1, self.w3, self.w2)
+        if not all(w.is_cuda and w.is_contiguous() and w.dtype in (torch.bfloat16, torch.float32) for w in ws):
+            return None
+        key = tuple((w.data_ptr(), w._version, w.dtype) for w in ws)
+        if self._kept is not None and self._kept[0] == key:
+            return self._kept[1]
+        equal = torch.full((self.num_experts,), self.hidden_size, dtype=torch.int64, device=self.w1.device)
+        with torch.no_grad():
+            made = tuple(ops.grouped_cast_rows_and_colwise_t(w.detach(), equal, _E4M3, pow2=True) for w in ws)
+        self._kept = (key, made)
+        return made
+
     def forward(self, x: torch.Tensor, batch_size_per_expert: torch.Tensor) -> torch.Tensor:
         """
         :param x: the expert inputs of shape ``(*, d_model)``, rows ordered by expert.
@@ -202,7 +231,8 @@ class DroplessMoEMLP(nn.Module):
         x2 = x.reshape(-1, self.d_model)
         if x2.dtype != torch.bfloat16:
             x2 = x2.to(torch.bfloat16)
-        y = float8_dropless_mlp(x2, self.w1, self.w2, self.w3, batch_size_per_expert, self.num_experts)
+        y = float8_dropless_mlp(x2, self.w1, self.w2, self.w3, batch_size_per_expert, self.num_experts,
+                                kept=self.weight_operands())
         return y.reshape(*lead, self.d_model).to(x.dtype)
 
     def forward_gathered(self, x: torch.Tensor, indices: torch.Tensor, top_k: int,
@@ -214,7 +244,7 @@ class DroplessMoEMLP(nn.Module):
         if x2.dtype != torch.bfloat16:
             x2 = x2.to(torch.bfloat16)
         y = float8_dropless_mlp(x2, self.w1, self.w2, self.w3, batch_size_per_expert, self.num_experts,
-                                indices=indices, top_k=top_k)
+                                indices=indices, top_k=top_k, kept=self.weight_operands())
         return y.to(x.dtype)
 
 

@@ -398,3 +398,45 @@ def test_accumulating_grouped_gemm_equals_gemm_plus_add(dev, sizes, n, k):
     want = first + term
     got = ops.grouped_gemm_fp8(xq, sx, wq, sw, sz, accumulate_into=first.clone(), **kw)
     assert torch.equal(got.view(torch.int16), want.view(torch.int16))
+
+
+def test_kept_expert_weight_operands(dev):
+    """keep_float8_weights: the float8 copies of the expert weights are made once and reused until a weight changes;
+    results are the bits of a module that quantises on every call."""
+    E, D, H, sizes = 4, 256, 384, [300, 0, 170, 42]
+    T = sum(sizes)
+    x, go = seeded((T, D), 51).to(dev), seeded((T, D), 52, std=1e-3).to(dev)
+    sz = torch.tensor(sizes).to(dev)
+    g = torch.Generator().manual_seed(53)
+    mods = []
+    for keep in (False, True):
+        m = DroplessMoEMLP(d_model=D, hidden_size=H, num_experts=E, dtype=torch.bfloat16, keep_float8_weights=keep)
+        g.manual_seed(53)
+        with torch.no_grad():
+            for p_ in m.parameters():
+                p_.copy_((torch.randn(p_.shape, generator=g) * 0.02).bfloat16())
+        mods.append(m.to(dev))
+    plain, kept = mods
+    assert plain.weight_operands() is None
+
+    def run(m):
+        for p_ in m.parameters():
+            p_.grad = None
+        xd = x.clone().requires_grad_(True)
+        y = m(xd, sz)
+        y.backward(go)
+        return [y.detach(), xd.grad] + [p_.grad.clone() for p_ in m.parameters()]
+
+    for a, b in zip(run(plain), run(kept)):
+        assert torch.equal(a, b)
+    first = kept.weight_operands()
+    assert first is kept.weight_operands(), "unchanged weights: the same copies are handed out"
+    for a, b in zip(run(plain), run(kept)):  # second call on kept copies
+        assert torch.equal(a, b)
+    with torch.no_grad():  # an optimizer step: in-place updates move the version counters
+        for m in mods:
+            m.w1.mul_(1.5)
+            m.w2.add_(0.01)
+    assert kept.weight_operands() is not first
+    for a, b in zip(run(plain), run(kept)):
+        assert torch.equal(a, b)
