@@ -169,7 +169,7 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_fp8_m16_kernel(Problem pb)
         while (ld_tile + 1 < my_tiles) {
             ++ld_tile;
             const TileDesc d = my_tile(ld_tile);
-            if (d.nk > 0) {
+            if (d.nk > 0 && d.c != nullptr) {
                 ld_a = d.a;
                 ld_b = d.b;
                 ld_nk = d.nk;
@@ -233,6 +233,7 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_fp8_m16_kernel(Problem pb)
     int step = 0;
     for (int cp_tile = 0; cp_tile < my_tiles; ++cp_tile) {
         const TileDesc td = my_tile(cp_tile);
+        if (td.c == nullptr) continue;  // (uniform) a grid slot without a tile
         // One 128-byte K step.  `fresh`: the tile's first step; phase A touches the accumulators of A tiles 0-3,
         // phase B those of A tiles 4-7, so both start from 0 then.  The first step is written out separately
         // from the loop, not as a branch inside it.
@@ -449,8 +450,8 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_fp8_m16_kernel(Problem pb)
     __syncthreads();
 }
 
-// persistent: one workgroup per CU walks a static share of the tiles (right when all tiles cost the same);
-// otherwise one workgroup per tile, handed to free CUs by the hardware dispatcher (tiles of unequal cost).
+// persistent: one workgroup per CU walks a static share of the tiles; otherwise one workgroup per tile, handed to
+// free CUs by the hardware dispatcher.
 template <typename Problem, int CBSZ_A, int BLGP_B>
 int launch(const Problem& pb, int max_tiles, bool persistent, hipStream_t st)
 {
@@ -515,7 +516,9 @@ int launch_m16_grouped_wgrad(const uint8_t* a_t, int a_dtype, const uint8_t* b_t
 {
     const int tiles_n = (N + BM - 1) / BM, tiles_k = (Kl + BN - 1) / BN;
     GroupedWgradProblem pb{a_t, b_t, out, ld_t, ld_t, Kl, sizes, E, T, N, Kl, tiles_n, tiles_k, sa, sb};
-    return launch_typed(pb, E * tiles_n * tiles_k, false, a_dtype, b_dtype, st);
+    // persistent: workgroup b walks slots b, b + grid, ... - on its XCD (b % 8 is kept by a stride that is a multiple
+    // of 8) these are the same tile position of one group after the other, so the XCD's workgroups stay in step
+    return launch_typed(pb, GroupedWgradProblem::grid_tiles(E, tiles_n * tiles_k), true, a_dtype, b_dtype, st);
 }
 
 }  // namespace gemm

@@ -18,7 +18,7 @@ struct TileDesc {
     int nk;            // 128-byte K steps (0: the tile is all zeros)
     const float* sa;   // scale of the tile's first row (or the single scale)
     const float* sb;   // scale of the tile's first column (or the single scale)
-    uint16_t* c;       // C element (first row, first column) of the tile
+    uint16_t* c;       // C element (first row, first column) of the tile; null: the slot holds no tile
     int row_lo, row_hi;  // rows [row_lo, row_hi) of the 256 are stored
 };
 
@@ -158,6 +158,20 @@ struct GroupedProblem {
 // Ragged-K grouped problem (dropless-MoE grad_weight): out[e] = A_t[:, S_e] . B_t[:, S_e]^T over group e's
 // 128-aligned segment S_e of the padded token axis; N, Kl >= 256.  An empty group gives nk = 0: its tiles are
 // written as zeros and its scales (never produced) are ignored.
+//
+// Tile order.  The tiles of one group share its operand panels (tiles_n of A_t, tiles_k of B_t) and cost the same;
+// tiles of different groups share nothing and differ in cost by orders of magnitude.  Slot t of the tile order
+// belongs to XCD t % 8 (workgroup b runs on XCD b % 8 and walks slots b, b + grid, ...): all tiles of a group are
+// given to ONE XCD, whose workgroups run them side by side (its L2 serves every panel to all of them) and move on to
+// the XCD's next group together, so a static walk is balanced inside an XCD.  Groups are dealt to the XCDs largest
+// first in boustrophedon order (ranks 0..7 to XCDs 0..7, ranks 8..15 to XCDs 7..0, ...), which evens out the XCDs'
+// loads for skewed sizes.  The ranks are computed by every wave from the sizes in its registers (E <= 64; more
+// groups: in index order).
+struct WgradCache {
+    GroupCache g;
+    int group_at_rank;  // lane p: the group whose size has rank p (ties broken by index)
+};
+
 struct GroupedWgradProblem {
     const uint8_t* At;
     const uint8_t* Bt;
@@ -171,21 +185,43 @@ struct GroupedWgradProblem {
     const float* sb;  // [E, Kl]
     static constexpr bool kVecScales = true, kMaskRows = false, kXcdRanges = false, kPeelFirstStep = true;
     static constexpr bool kAccumulate = false;
-    using Cache = GroupCache;
-    __device__ __forceinline__ Cache prepare() const { return build_group_cache<128>(sizes, E, T); }
-    __device__ __forceinline__ int total_tiles(const Cache&) const { return E * tiles_n * tiles_k; }
+    using Cache = WgradCache;
+    __device__ __forceinline__ Cache prepare() const
+    {
+        Cache c{build_group_cache<128>(sizes, E, T), 0};
+        const int lane = (int)threadIdx.x & 63;
+        c.group_at_rank = lane;
+        if (c.g.valid) {
+            const int m = lane < E ? c.g.m : -1;
+            int rank = 0;
+            for (int j = 0; j < E; ++j) {
+                const int mj = __builtin_amdgcn_readlane(c.g.m, j);
+                rank += (mj > m || (mj == m && j < lane)) ? 1 : 0;
+            }
+            for (int j = 0; j < E; ++j)
+                if (__builtin_amdgcn_readlane(rank, j) == lane) c.group_at_rank = j;
+        }
+        return c;
+    }
+    // slots of the launch grid: 8 XCDs x ceil(E / 8) groups x tiles per group (slots past the last group do nothing)
+    __host__ __device__ __forceinline__ static int grid_tiles(int E, int per_group) { return 8 * ((E + 7) / 8) * per_group; }
+    __device__ __forceinline__ int total_tiles(const Cache&) const { return grid_tiles(E, tiles_n * tiles_k); }
     __device__ __forceinline__ TileDesc tile(int t, const Cache& c) const
     {
         const int per_group = tiles_n * tiles_k;
-        const int e = t / per_group, rem = t % per_group;
+        const int xcd = t & 7, slot = t >> 3;
+        const int k = slot / per_group, rem = slot % per_group;  // the XCD's k-th group, tile rem of it
+        const int rank = (k & 1) ? 8 * k + 7 - xcd : 8 * k + xcd;
+        TileDesc d{};
+        if (rank >= E) return d;  // d.c == nullptr: nothing to do
+        const int e = c.g.valid ? __builtin_amdgcn_readlane(c.group_at_rank, rank) : rank;
         const int tn = rem / tiles_k, tk = rem % tiles_k;
-        const GroupSpan s = locate_group_cached<128, false>(c, sizes, E, T, e);
+        const GroupSpan s = locate_group_cached<128, false>(c.g, sizes, E, T, e);
         const int64_t seg0 = 128 * s.units_before;
         int64_t seg = 128 * ((s.m + 127) / 128);
         if (seg0 + seg > lda) seg = 0;
         const int n0 = (tn * BM + BM <= N) ? tn * BM : N - BM;
         const int k0 = (tk * BN + BN <= Kl) ? tk * BN : Kl - BN;
-        TileDesc d;
         d.a = At + (int64_t)n0 * lda + seg0;
         d.b = Bt + (int64_t)k0 * ldb + seg0;
         d.nk = (int)(seg / BK);
