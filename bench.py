@@ -371,10 +371,12 @@ def main():
     flops_per_step = GEMMS_PER_STEP * 2.0 * TOKENS * D_MODEL * HIDDEN
     tflops = flops_per_step / (ms_per_step * 1e-3) / 1e12
 
+    # one event pair per GEMM launch; the fused launch of the two input projections counts as the two GEMMs it is
     gemm_ms = [s.elapsed_time(e) for s, e, _ in events]
-    assert len(gemm_ms) == GEMMS_PER_STEP * ns.steps, (len(gemm_ms), ns.steps)
-    avg_gemm_s = sum(gemm_ms) / len(gemm_ms) * 1e-3
+    gemm_flops = sum(2.0 * m * n * k for _, _, (m, n, k) in events)
     flops_per_launch = 2.0 * TOKENS * D_MODEL * HIDDEN
+    assert abs(gemm_flops - GEMMS_PER_STEP * ns.steps * flops_per_launch) < 1e-6 * gemm_flops, (gemm_flops, ns.steps)
+    avg_gemm_s = sum(gemm_ms) / (GEMMS_PER_STEP * ns.steps) * 1e-3  # per 2*M*N*K unit of work
     achieved = flops_per_launch / avg_gemm_s / 1e12
 
     result = {

@@ -163,6 +163,21 @@ int mi8_gemm_fp8_accumulate(const void* a, int a_dtype, int64_t lda, const void*
                             int64_t N, int64_t K, const float* sa, int sa_is_vector, const float* sb, int sb_is_vector,
                             void* out, int out_dtype, int64_t ldc, void* stream);
 
+/* The two input projections of a SwiGLU feed-forward block and the activation between them and the output projection
+ * in one launch (reference: src/olmo_core/nn/feed_forward.py:171, `self.w2(F.silu(self.w1(x)) * self.w3(x))`):
+ *   x1[M, H] = bf16((A . B1^T) / sa / sb1),  x3[M, H] = bf16((A . B3^T) / sa / sb3)   (what mi8_gemm_fp8 writes, bit for bit)
+ *   h[M, H]  = silu(x1) * x3                                                          (what mi8_swiglu_fwd writes, bit for bit)
+ *   slots_h[0 .. *n_slots_used) = partial maxima of |h| as mi8_swiglu_fwd produces them for the cast of h that follows.
+ * Every workgroup computes matching 128-column tiles of x1 and x3 and forms h in its epilogue, so x1 and x3 are written
+ * once and never read back.  A fp8 [M, lda]; B1, B3 fp8 [H, ldb] of one type; single scales (float32 [1] each);
+ * x1, x3, h bf16 [M, ldc]; slots_h must hold MI8_AMAX_SLOTS uint32.  Needs M >= 256, H >= 128, H % 8 == 0,
+ * K % 128 == 0 (MI8_ERR_UNSUPPORTED otherwise: run the three calls it stands for). */
+int mi8_gemm_fp8_swiglu_matches_separate(int64_t M, int64_t H, int64_t K); /* host only: 1 if the fused launch takes
+    the shape and mi8_gemm_fp8 would run both projections on the same tile kernel, so that the bits agree as well */
+int mi8_gemm_fp8_swiglu(const void* a, int a_dtype, int64_t lda, const void* b1, const void* b3, int b_dtype, int64_t ldb,
+                        int64_t M, int64_t H, int64_t K, const float* sa, const float* sb1, const float* sb3, void* x1,
+                        void* x3, void* h, int64_t ldc, uint32_t* slots_h, int32_t* n_slots_used, void* stream);
+
 /* The same product with K cut into `splits` slices, for problems whose few output tiles would leave most of the
  * GPU idle (a few hundred rows of A against a weight matrix): every slice is summed by its own workgroups into
  * an fp32 plane of `workspace`, a second kernel adds the planes in slice order (results do not depend on

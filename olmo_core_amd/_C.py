@@ -65,6 +65,12 @@ _SIGNATURES = {
         [c_void_p, c_int, c_int64, c_void_p, c_int, c_int64, c_int64, c_int64, c_int64, c_void_p, c_int, c_void_p,
          c_int, c_void_p, c_int, c_int64, c_void_p],
     ),
+    "mi8_gemm_fp8_swiglu_matches_separate": (c_int, [c_int64, c_int64, c_int64]),
+    "mi8_gemm_fp8_swiglu": (
+        c_int,
+        [c_void_p, c_int, c_int64, c_void_p, c_void_p, c_int, c_int64, c_int64, c_int64, c_int64, c_void_p, c_void_p,
+         c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_void_p, POINTER(c_int32), c_void_p],
+    ),
     "mi8_gemm_fp8_splitk": (
         c_int,
         [c_void_p, c_int, c_int64, c_void_p, c_int, c_int64, c_int64, c_int64, c_int64, c_void_p, c_int, c_void_p,

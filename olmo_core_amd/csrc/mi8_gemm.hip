@@ -230,7 +230,7 @@ int gemm_fp8_entry(const void* a, int a_dtype, int64_t lda, const void* b, int b
         if (M <= kSkinnyMaxM && !accumulate)
             variant = kSkinny;
         else if (dma_ok)
-            variant = tiles256 <= 96 ? kSmallTile : kM16;
+            variant = tiles256 <= 96 ? kSmallTile : kM16;  // (mi8_gemm_fp8_swiglu_matches_separate mirrors this)
         else
             variant = tiles256 <= 384 ? kSmallTile : 1;
     }
@@ -265,6 +265,43 @@ extern "C" int mi8_gemm_fp8_accumulate(const void* a, int a_dtype, int64_t lda, 
 {
     return gemm_fp8_entry(a, a_dtype, lda, b, b_dtype, ldb, M, N, K, sa, sa_is_vector, sb, sb_is_vector, out, out_dtype,
                           ldc, -1, true, stream);
+}
+
+// 1 if mi8_gemm_fp8_swiglu takes the shape AND mi8_gemm_fp8 would run both projections on the same persistent
+// kernel (then the fused launch reproduces the three-call route bit for bit; other tile kernels sum in another order)
+extern "C" int mi8_gemm_fp8_swiglu_matches_separate(int64_t M, int64_t H, int64_t K)
+{
+    if (M < 256 || H < 256 || K <= 0 || K % 128 || H % 8) return 0;
+    const int64_t tiles256 = ((M + 255) / 256) * ((H + 255) / 256);
+    return tiles256 > 96 ? 1 : 0;
+}
+
+extern "C" int mi8_gemm_fp8_swiglu(const void* a, int a_dtype, int64_t lda, const void* b1, const void* b3, int b_dtype,
+                                   int64_t ldb, int64_t M, int64_t H, int64_t K, const float* sa, const float* sb1,
+                                   const float* sb3, void* x1, void* x3, void* h, int64_t ldc, uint32_t* slots_h,
+                                   int32_t* n_slots_used, void* stream)
+{
+    MI8_REQUIRE(a && b1 && b3 && sa && sb1 && sb3 && x1 && x3 && h && slots_h && n_slots_used, MI8_ERR_ARG,
+                "mi8_gemm_fp8_swiglu: null pointer");
+    MI8_REQUIRE((a_dtype == MI8_E4M3 || a_dtype == MI8_E5M2) && (b_dtype == MI8_E4M3 || b_dtype == MI8_E5M2),
+                MI8_ERR_ARG, "mi8_gemm_fp8_swiglu: unknown fp8 dtype");
+    MI8_REQUIRE(M >= 256 && H >= 128 && K > 0 && K % 128 == 0 && H % 8 == 0, MI8_ERR_UNSUPPORTED,
+                "mi8_gemm_fp8_swiglu: needs M >= 256, H >= 128, H %% 8 == 0, K %% 128 == 0 (got %lld x %lld x %lld); use "
+                "mi8_gemm_fp8 twice and mi8_swiglu_fwd",
+                (long long)M, (long long)H, (long long)K);
+    MI8_REQUIRE(lda % 16 == 0 && ldb % 16 == 0 && lda >= K && ldb >= K && ldc >= H && ldc % 8 == 0, MI8_ERR_UNSUPPORTED,
+                "mi8_gemm_fp8_swiglu: lda, ldb must be multiples of 16 and >= K, ldc a multiple of 8 and >= H");
+    MI8_REQUIRE(aligned16(a) && aligned16(b1) && aligned16(b3) && aligned16(x1) && aligned16(x3) && aligned16(h),
+                MI8_ERR_UNSUPPORTED, "mi8_gemm_fp8_swiglu: operands and outputs must be 16-byte aligned");
+    MI8_REQUIRE(M * lda < (int64_t)1 << 32 && H * ldb < (int64_t)1 << 32 && M < (1 << 30) && H < (1 << 30) &&
+                    K < (1 << 30),
+                MI8_ERR_UNSUPPORTED, "mi8_gemm_fp8_swiglu: operand larger than 4 GiB");
+    GemmArgs g{(const uint8_t*)a, (const uint8_t*)b1, x1, 0, lda, ldb, ldc, (int)M, (int)H, (int)K, sa, sb1, 0, 0, 0, 0, 0};
+    int used = 0;
+    const int rc = launch_m16_swiglu(g, (const uint8_t*)b3, sb3, (uint16_t*)x3, (uint16_t*)h, slots_h, &used, a_dtype,
+                                     b_dtype, (hipStream_t)stream);
+    *n_slots_used = used;
+    return rc;
 }
 
 extern "C" int mi8_gemm_splitk_suggest(int64_t M, int64_t N, int64_t K)

@@ -23,6 +23,7 @@
 // tile it belongs to, so two address registers per operand serve all eight tiles through the instruction's
 // offset field.
 #include "mi8_gemm_tiles.h"
+#include "mi8_swiglu.h"
 
 namespace mi8 {
 namespace gemm {
@@ -121,7 +122,16 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_fp8_m16_kernel(Problem pb)
     // counted over tiles that have K steps (the cursor skips the others, however many): the cursor is at most
     // two steps, hence two such tiles, ahead of the epilogue that reads a slot.
     float inv_single = 1.0f;
-    if constexpr (!Problem::kVecScales) {
+    if constexpr (Problem::kSwiglu) {
+        // The fused problem has two multipliers (x1, x3) and a running maximum of |h| per lane.  They live in the
+        // scale-slot area of LDS (unused with single scales), not in registers: the K loop has none to spare.
+        float* aux = reinterpret_cast<float*>(lds + 2 * STAGE + OUT_STAGING);
+        if (tid == 0) {
+            aux[0] = (1.0f / pb.single_sa()) * (1.0f / pb.single_sb());
+            aux[1] = (1.0f / pb.single_sa()) * (1.0f / pb.sb3[0]);
+        }
+        reinterpret_cast<uint32_t*>(aux)[64 + tid] = 0;
+    } else if constexpr (!Problem::kVecScales) {
         inv_single = (1.0f / pb.single_sa()) * (1.0f / pb.single_sb());
         asm volatile("" ::"v"(inv_single));  // the value is complete before the first direct load is issued
     }
@@ -157,9 +167,18 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_fp8_m16_kernel(Problem pb)
         tile_stride = (int)gridDim.x;
         my_tiles = (first_tile < total) ? (total - first_tile + tile_stride - 1) / tile_stride : 0;
     }
-    if (my_tiles == 0) return;
+    if (my_tiles == 0) {
+        if constexpr (Problem::kSwiglu)
+            if (lane == 0) pb.h_slots[(int)blockIdx.x * 4 + wave] = 0;
+        return;
+    }
     auto my_tile = [&](int idx) __attribute__((always_inline)) { return pb.tile(first_tile + idx * tile_stride, cache); };
 
+    // Fused SwiGLU problem: LDS B rows [64 w, 64 w + 64), the rows this wave fetches, are rows 64 (w / 2) .. of B1
+    // (even w) or of B3 (odd w); folded into the wave's B cursor once per tile.
+    int64_t b_wave_shift = 0;
+    if constexpr (Problem::kSwiglu)
+        b_wave_shift = (int64_t)(wave & 1) * pb.b3_offset + (int64_t)((wave >> 1) * 64 - wave * 64) * pb.ldb;
     // load cursor: the K step whose stage is fetched next (two steps ahead of the compute cursor); it skips
     // tiles without K steps and, past the last tile, keeps fetching valid data nobody reads
     int ld_tile = -1, ld_kt = 0, ld_nk = 0;
@@ -171,7 +190,7 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_fp8_m16_kernel(Problem pb)
             const TileDesc d = my_tile(ld_tile);
             if (d.nk > 0 && d.c != nullptr) {
                 ld_a = d.a;
-                ld_b = d.b;
+                ld_b = d.b + b_wave_shift;
                 ld_nk = d.nk;
                 ld_kt = 0;
                 scale_dma(d);
@@ -256,7 +275,7 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_fp8_m16_kernel(Problem pb)
             // A tile's first step follows the previous tile's epilogue, whose 32 stores are younger than the loads
             // waited for here (one in-order counter): they may stay outstanding as well.
             if (fresh)
-                __builtin_amdgcn_s_waitcnt(0x8F78);  // vmcnt(40)
+                __builtin_amdgcn_s_waitcnt(Problem::kSwiglu ? 0xCF78 : 0x8F78);  // vmcnt(56) / vmcnt(40)
             else
                 __builtin_amdgcn_s_waitcnt(0x0F78);  // vmcnt(8)
             asm volatile("s_barrier" ::: "memory");
@@ -358,6 +377,96 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_fp8_m16_kernel(Problem pb)
                 }
             }
         };
+        if constexpr (Problem::kSwiglu) {
+            // Fused SwiGLU epilogue: the wave holds x1 (B tiles 0-3) and x3 (B tiles 4-7) of the same 128 rows x 64
+            // columns.  Per 32 rows: x1 is scaled, rounded and staged; x3 likewise; h = silu(x1) * x3 is formed from
+            // the rounded values (the arithmetic of the stand-alone pointwise kernel) and staged; the three outputs
+            // leave through the same pipelined staging area as any other tile, twelve passes instead of eight.
+            const float* aux = reinterpret_cast<const float*>(lds + 2 * STAGE + OUT_STAGING);
+            uint32_t hmax = 0;
+            auto store_out = [&](int which, int ih) __attribute__((always_inline)) {
+                const int rt = wm * WT + ih * 32;
+                const int64_t shift = which == 0 ? 0 : (which == 1 ? pb.x3_offset : pb.h_offset);
+#pragma unroll
+                for (int it = 0; it < 4; ++it) {
+                    uint8_t* base = reinterpret_cast<uint8_t*>(td.c + shift + (int64_t)(rt + it * 8) * pb.ldc + wn * 64);
+                    uint32_t o = c_lane_off;
+                    asm volatile("" : "+v"(o));
+                    *reinterpret_cast<v4i*>(base + o) = staged[it];
+                }
+            };
+            // stage one pass (32 rows x 64 columns held as o[t][jj]); the pass before it goes to memory first
+            auto stage = [&](const uint2 (&o)[2][4], int prev_which, int prev_ih) __attribute__((always_inline)) {
+                asm volatile("" ::: "memory");
+                if (prev_which >= 0) {
+                    __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): the previous pass's rows are in registers
+                    store_out(prev_which, prev_ih);
+                }
+#pragma unroll
+                for (int t = 0; t < 2; ++t)
+#pragma unroll
+                    for (int jj = 0; jj < 4; ++jj) {
+                        const int row = 16 * t + r16;
+                        const int cw = 16 * jj + 4 * kb;
+                        const int chunk = (cw >> 3) ^ ((row >> 1) & 7);
+                        const uint32_t saddr = stg_lds + (uint32_t)(row * 128 + chunk * 16 + (cw & 4) * 2);
+                        asm volatile("ds_write_b64 %0, %1" ::"v"(saddr), "v"(o[t][jj]) : "memory");
+                    }
+                __builtin_amdgcn_s_waitcnt(0xc07f);
+                __builtin_amdgcn_wave_barrier();
+#pragma unroll
+                for (int it = 0; it < 4; ++it) {
+                    const int rw = it * 8 + (lane >> 3);
+                    staged[it] = *reinterpret_cast<const v4i*>(stg + rw * 128 + (((lane & 7) ^ ((rw >> 1) & 7)) << 4));
+                }
+                asm volatile("" ::: "memory");
+            };
+            auto scaled = [&](uint2 (&o)[2][4], int ih, int j0, float mult_in) __attribute__((always_inline)) {
+#pragma unroll
+                for (int t = 0; t < 2; ++t) {
+                    float mult = mult_in;
+                    asm volatile("" : "+v"(mult));  // (a loop-invariant multiplier makes the compiler hoist all products)
+#pragma unroll
+                    for (int jj = 0; jj < 4; ++jj) {
+                        float v[4];
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) {
+                            float a_;
+                            asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(a_) : "a"(acc[2 * ih + t][j0 + jj][e]));
+                            v[e] = a_ * mult;
+                        }
+                        o[t][jj].x = pack_bf16x2(v[0], v[1]);
+                        o[t][jj].y = pack_bf16x2(v[2], v[3]);
+                    }
+                }
+            };
+#pragma unroll
+            for (int ih = 0; ih < 4; ++ih) {
+                uint2 o1[2][4], o3[2][4], oh[2][4];
+                scaled(o1, ih, 0, aux[0]);
+                stage(o1, ih == 0 ? -1 : 2, ih - 1);
+                scaled(o3, ih, 4, aux[1]);
+#pragma unroll
+                for (int t = 0; t < 2; ++t)
+#pragma unroll
+                    for (int jj = 0; jj < 4; ++jj) {
+                        oh[t][jj] = swiglu_fwd4(o1[t][jj], o3[t][jj]);
+                        hmax = umax32(hmax, (oh[t][jj].x & 0x7FFFu) << 16);
+                        hmax = umax32(hmax, oh[t][jj].x & 0x7FFF0000u);
+                        hmax = umax32(hmax, (oh[t][jj].y & 0x7FFFu) << 16);
+                        hmax = umax32(hmax, oh[t][jj].y & 0x7FFF0000u);
+                    }
+                stage(o3, 0, ih);
+                stage(oh, 1, ih);
+            }
+            __builtin_amdgcn_s_waitcnt(0xc07f);
+            store_out(2, 3);
+            {   // fold this tile's maximum into the lane's slot (an LDS atomic the compiler need not order against
+                // the direct loads in flight)
+                const uint32_t maddr = (uint32_t)(uintptr_t)(lptr_t)(lds + 2 * STAGE + OUT_STAGING) + (64 + tid) * 4;
+                asm volatile("ds_max_u32 %0, %1" ::"v"(maddr), "v"(hmax) : "memory");
+            }
+        } else {
 #pragma unroll
         for (int jq = 0; jq < 2; ++jq) {
             float isb[4][4];
@@ -439,6 +548,7 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_fp8_m16_kernel(Problem pb)
         __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0)
         if constexpr (Problem::kAccumulate) add_held();
         store_staged(1, 3);
+        }
         // The last step's phase B has read the next tile's first fragments like any other step; reading them
         // again here makes those 96 registers free during the epilogue, which otherwise spills (and every
         // reload from scratch waits on the in-order vector memory counter, i.e. on the stores above).
@@ -448,6 +558,11 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_fp8_m16_kernel(Problem pb)
     // direct loads issued for steps past the end must have landed before the LDS allocation is released
     __builtin_amdgcn_s_waitcnt(0x0070);  // vmcnt(0) lgkmcnt(0)
     __syncthreads();
+    if constexpr (Problem::kSwiglu) {  // one partial maximum of |h| per wave
+        uint32_t m = reinterpret_cast<const uint32_t*>(lds + 2 * STAGE + OUT_STAGING)[64 + tid];
+        m = wave_umax(m);
+        if (lane == 0) pb.h_slots[(int)blockIdx.x * 4 + wave] = m;
+    }
 }
 
 // persistent: one workgroup per CU walks a static share of the tiles; otherwise one workgroup per tile, handed to
@@ -492,6 +607,21 @@ int launch_m16(GemmArgs& g, int a_dtype, int b_dtype, hipStream_t st)
     }
     if (g.accumulate) return launch_typed(DenseProblem<false, true>{g, g.lda, g.ldb, g.ldc}, tiles, true, a_dtype, b_dtype, st);
     return launch_typed(DenseProblem<false>{g, g.lda, g.ldb, g.ldc}, tiles, true, a_dtype, b_dtype, st);
+}
+
+int launch_m16_swiglu(GemmArgs& g, const uint8_t* b3, const float* sb3, uint16_t* x3, uint16_t* h, uint32_t* h_slots,
+                      int* n_slots, int a_dtype, int b_dtype, hipStream_t st)
+{
+    g.tiles_m = (g.M + BM - 1) / BM;
+    g.tiles_n = (g.N + 127) / 128;
+    SwigluProblem pb{g, g.lda, g.ldb, g.ldc, (int64_t)(b3 - g.B), (int64_t)(x3 - reinterpret_cast<uint16_t*>(g.C)),
+                     (int64_t)(h - reinterpret_cast<uint16_t*>(g.C)), sb3, h_slots};
+    const int tiles = g.tiles_m * g.tiles_n;
+    int blocks = num_compute_units();
+    const int wanted = (tiles + 7) / 8 * 8;
+    if (blocks > wanted) blocks = wanted;
+    *n_slots = 4 * blocks;
+    return launch_typed(pb, tiles, true, a_dtype, b_dtype, st);
 }
 
 int launch_m16_grouped(const uint8_t* a, int a_dtype, int64_t lda, const uint8_t* b, int b_dtype, int64_t ldb,

@@ -32,6 +32,7 @@ struct DenseProblem {
     int64_t lda, ldb, ldc;
     static constexpr bool kVecScales = VEC;  // both scales are vectors (per row / per column) or both single
     static constexpr bool kAccumulate = ACC;  // C += the rounded product
+    static constexpr bool kSwiglu = false;
     static constexpr bool kMaskRows = false, kXcdRanges = true, kPeelFirstStep = true;
     using Cache = NoCache;
     __device__ __forceinline__ Cache prepare() const { return Cache{}; }
@@ -51,6 +52,45 @@ struct DenseProblem {
         d.nk = g.K / BK;
         d.sa = g.sa + (VEC ? m0 : 0);
         d.sb = g.sb + (VEC ? n0 : 0);
+        d.c = reinterpret_cast<uint16_t*>(g.C) + (int64_t)m0 * g.ldc + n0;
+        d.row_lo = 0;
+        d.row_hi = BM;
+        return d;
+    }
+};
+
+// The two input projections of a SwiGLU feed-forward block in one problem: x1 = A . B1^T, x3 = A . B3^T and
+// h = silu(x1) * x3, all [M, H] bf16, single scales.  A 256 x 256 workgroup tile covers 128 columns of H: its B rows
+// are, per 128-row half (one half per wave column), 64 rows of B1 followed by the same 64 rows of B3, so that a wave's
+// accumulators for B tiles j and j + 4 hold x1 and x3 of the same elements and the epilogue can form h in registers.
+// Tiles are shifted back at the ends like the dense problem's (M >= 256, H >= 128).
+struct SwigluProblem {
+    GemmArgs g;             // A, B = B1, C = x1; N = H; tiles_n counts 128-column tiles; sa, sb = scale of A, of B1
+    int64_t lda, ldb, ldc;
+    int64_t b3_offset;      // bytes from B1 to B3
+    int64_t x3_offset;      // elements from x1 to x3 and to h (same pitch ldc)
+    int64_t h_offset;
+    const float* sb3;       // scale of B3
+    uint32_t* h_slots;      // [4 * workgroups] partial maxima of |h| (float32 bit patterns)
+    static constexpr bool kVecScales = false, kAccumulate = false, kSwiglu = true;
+    static constexpr bool kMaskRows = false, kXcdRanges = true, kPeelFirstStep = true;
+    using Cache = NoCache;
+    __device__ __forceinline__ Cache prepare() const { return Cache{}; }
+    __device__ __forceinline__ int total_tiles(const Cache&) const { return g.tiles_m * g.tiles_n; }
+    __device__ __forceinline__ float single_sa() const { return g.sa[0]; }
+    __device__ __forceinline__ float single_sb() const { return g.sb[0]; }
+    __device__ __forceinline__ TileDesc tile(int t, const Cache&) const
+    {
+        int tm, tn;
+        tile_coords(g, t, tm, tn);
+        const int m0 = (tm * BM + BM <= g.M) ? tm * BM : g.M - BM;
+        const int n0 = (tn * 128 + 128 <= g.N) ? tn * 128 : g.N - 128;
+        TileDesc d;
+        d.a = g.A + (int64_t)m0 * g.lda;
+        d.b = g.B + (int64_t)n0 * g.ldb;
+        d.nk = g.K / BK;
+        d.sa = g.sa;
+        d.sb = g.sb;
         d.c = reinterpret_cast<uint16_t*>(g.C) + (int64_t)m0 * g.ldc + n0;
         d.row_lo = 0;
         d.row_hi = BM;
@@ -114,6 +154,7 @@ __device__ __forceinline__ GroupSpan locate_group_cached(const GroupCache& c, co
 template <bool ACC = false>
 struct GroupedProblem {
     static constexpr bool kAccumulate = ACC;
+    static constexpr bool kSwiglu = false;
     const uint8_t* A;
     const uint8_t* B;
     uint16_t* C;
@@ -184,7 +225,7 @@ struct GroupedWgradProblem {
     const float* sa;  // [E, N]
     const float* sb;  // [E, Kl]
     static constexpr bool kVecScales = true, kMaskRows = false, kXcdRanges = false, kPeelFirstStep = true;
-    static constexpr bool kAccumulate = false;
+    static constexpr bool kAccumulate = false, kSwiglu = false;
     using Cache = WgradCache;
     __device__ __forceinline__ Cache prepare() const
     {

@@ -58,6 +58,22 @@ __device__ __forceinline__ uint4 swiglu_fwd8(uint4 x1, uint4 x3)
     return pack8(o);
 }
 
+// the same for four packed values (the fused epilogue of the two input projections holds four columns per lane)
+__device__ __forceinline__ uint2 swiglu_fwd4(uint2 x1, uint2 x3)
+{
+    const float a[4] = {bits_to_f32(x1.x << 16), bits_to_f32(x1.x & 0xFFFF0000u), bits_to_f32(x1.y << 16),
+                        bits_to_f32(x1.y & 0xFFFF0000u)};
+    const float b[4] = {bits_to_f32(x3.x << 16), bits_to_f32(x3.x & 0xFFFF0000u), bits_to_f32(x3.y << 16),
+                        bits_to_f32(x3.y & 0xFFFF0000u)};
+    float o[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+        const float s = bf16_round(a[k] * sigmoid_f32(a[k]));
+        o[k] = s * b[k];
+    }
+    return make_uint2(pack_bf16(o[0], o[1]), pack_bf16(o[2], o[3]));
+}
+
 // gradients of h = silu(x1) * x3 with respect to x1 and x3
 __device__ __forceinline__ void swiglu_bwd8(uint4 x1, uint4 x3, uint4 gh, uint4& g1, uint4& g3)
 {

@@ -305,6 +305,56 @@ def gemm_fp8(
     return out
 
 
+def swiglu_gemm_supported(M: int, H: int, K: int) -> bool:
+    """Shapes :func:`gemm_fp8_swiglu` takes (otherwise: two :func:`gemm_fp8` calls and :func:`swiglu_fwd`)."""
+    return M >= 256 and H >= 128 and H % 8 == 0 and K % 128 == 0
+
+
+def swiglu_gemm_matches_separate(M: int, H: int, K: int) -> bool:
+    """Shapes for which :func:`gemm_fp8_swiglu` gives the bits of the three separate launches as the library
+    dispatches them (large problems: both routes run the persistent tile kernel)."""
+    return bool(_C.lib().mi8_gemm_fp8_swiglu_matches_separate(M, H, K))
+
+
+def gemm_fp8_swiglu(a: torch.Tensor, sa: torch.Tensor, b1: torch.Tensor, sb1: torch.Tensor, b3: torch.Tensor,
+                    sb3: torch.Tensor, *, k: Optional[int] = None):
+    """
+    ``x1 = a @ b1.T``, ``x3 = a @ b3.T`` (scaled, bf16) and ``h = silu(x1) * x3`` from one launch, with the amax
+    partials of ``h``: ``(x1, x3, h, (slots, n_slots))``, each bit-identical to :func:`gemm_fp8` / :func:`swiglu_fwd`.
+    Single scales only (the tensorwise recipe).
+    """
+    _require_gpu(a, "gemm_fp8_swiglu")
+    if a.dim() != 2 or b1.dim() != 2 or b1.shape != b3.shape or b1.dtype != b3.dtype or b1.stride(0) != b3.stride(0):
+        raise ValueError("gemm_fp8_swiglu: b1 and b3 must be matrices of one shape, type and row pitch")
+    if a.stride(1) != 1 or b1.stride(1) != 1 or b3.stride(1) != 1:
+        raise ValueError("gemm_fp8_swiglu: operands must have contiguous rows")
+    if a.dtype not in _FP8_CODE or b1.dtype not in _FP8_CODE:
+        raise TypeError("gemm_fp8_swiglu: operands must be float8")
+    if sa.numel() != 1 or sb1.numel() != 1 or sb3.numel() != 1:
+        raise ValueError("gemm_fp8_swiglu: single scales only")
+    M, H = a.shape[0], b1.shape[0]
+    K = min(a.shape[1], b1.shape[1]) if k is None else k
+    x1, x3, h = (torch.empty((M, H), dtype=torch.bfloat16, device=a.device) for _ in range(3))
+    slots = torch.empty(_C.AMAX_SLOTS, dtype=torch.int32, device=a.device)
+    used = _C.c_int32(0)
+    sink = GEMM_EVENT_SINK
+    if sink is not None:
+        ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        ev0.record()
+    _C.check(
+        _C.lib().mi8_gemm_fp8_swiglu(
+            a.data_ptr(), _FP8_CODE[a.dtype], a.stride(0), b1.data_ptr(), b3.data_ptr(), _FP8_CODE[b1.dtype],
+            b1.stride(0), M, H, K, sa.data_ptr(), sb1.data_ptr(), sb3.data_ptr(), x1.data_ptr(), x3.data_ptr(),
+            h.data_ptr(), H, slots.data_ptr(), used, _stream(a),
+        ),
+        "mi8_gemm_fp8_swiglu",
+    )
+    if sink is not None:
+        ev1.record()
+        sink.append((ev0, ev1, (M, 2 * H, K)))
+    return x1, x3, h, (slots, used.value)
+
+
 def gemm_variants() -> list:
     L = _C.lib()
     return [L.mi8_gemm_variant_name(i).decode() for i in range(L.mi8_gemm_num_variants())]

@@ -25,6 +25,10 @@ __all__ = ["FeedForward", "swiglu"]
 # so that a checker can feed each stage's actual input to a reference of that stage.
 STAGE_SINK = None
 
+# Run the two input projections and the SwiGLU between them as one launch where the shape allows (same bits as the
+# three separate launches); a switch so that the two routes can be compared.
+FUSE_SWIGLU_EPILOGUE = True
+
 
 class _SwiGLU(torch.autograd.Function):
     @staticmethod
@@ -66,9 +70,13 @@ class _Float8SwiGLUMLP(torch.autograd.Function):
         w1q, w1q_t, s1 = wo1 or ops.cast_tensorwise(w1, w_dt, pow2=pow2, want_transposed=need[0], scale=ws1)
         w3q, w3q_t, s3 = wo3 or ops.cast_tensorwise(w3, w_dt, pow2=pow2, want_transposed=need[0], scale=ws3)
         w2q, w2q_t, s2 = wo2 or ops.cast_tensorwise(w2, w_dt, pow2=pow2, want_transposed=any_grad, scale=ws2)
-        x1 = ops.gemm_fp8(xq, sx, w1q, s1, out_dtype=x.dtype)
-        x3 = ops.gemm_fp8(xq, sx, w3q, s3, out_dtype=x.dtype)
-        h, h_slots = ops.swiglu_fwd(x1, x3, want_amax=True)
+        if FUSE_SWIGLU_EPILOGUE and x.dtype == torch.bfloat16 and ops.swiglu_gemm_matches_separate(x.shape[0], w1.shape[0], x.shape[1]):
+            # both input projections and the activation in one launch: x1 and x3 are never read back
+            x1, x3, h, h_slots = ops.gemm_fp8_swiglu(xq, sx, w1q, s1, w3q, s3)
+        else:
+            x1 = ops.gemm_fp8(xq, sx, w1q, s1, out_dtype=x.dtype)
+            x3 = ops.gemm_fp8(xq, sx, w3q, s3, out_dtype=x.dtype)
+            h, h_slots = ops.swiglu_fwd(x1, x3, want_amax=True)
         if STAGE_SINK is not None:
             STAGE_SINK.update(x1=x1.clone(), x3=x3.clone(), h=h.clone())
         hq, hq_t, sh = ops.cast_tensorwise(h, in_dt, pow2=pow2, want_transposed=need[2], slots=h_slots)

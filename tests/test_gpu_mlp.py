@@ -120,3 +120,55 @@ def test_mlp_stage_by_stage_against_oracle(dev, mdh):
     M, D, H = mdh
     x, go = seeded((M, D), 1), seeded((M, D), 2, std=1e-3)
     check_mlp_stages(dev, _make(dev, D, H, fuse=True, seed=3), x, go)
+
+
+@pytest.mark.parametrize("mhk", [(256, 128, 128), (512, 256, 256), (300, 272, 384), (1024, 1416, 512), (2560, 2816, 1024),
+                                 (4100, 1672, 256)], ids=lambda s: "x".join(map(str, s)))
+@pytest.mark.parametrize("a_fp8", [E4M3, E5M2], ids=["e4m3", "e5m2"])
+def test_swiglu_fused_into_the_projection_gemm(dev, mhk, a_fp8):
+    """x1, x3, h and the amax of h from the one-launch route are the bits of gemm_fp8 twice + swiglu_fwd (token and
+    hidden sizes that are not multiples of the tile included: the shifted-back edge tiles rewrite identical values)."""
+    M, H, K = mhk
+    x, w1, w3 = seeded((M, K), 61), seeded((H, K), 62, std=0.05), seeded((H, K), 63, std=0.02)
+    xq, _, sx = ops.cast_tensorwise(x.to(dev), a_fp8)
+    w1q, _, s1 = ops.cast_tensorwise(w1.to(dev), E4M3)
+    w3q, _, s3 = ops.cast_tensorwise(w3.to(dev), E4M3)
+    assert ops.swiglu_gemm_supported(M, H, K)
+    x1, x3, h, (slots, n) = ops.gemm_fp8_swiglu(xq, sx, w1q, s1, w3q, s3)
+    # the projections: bit-identical to the persistent tile kernel (the library's choice for large problems; forced
+    # here where the library would pick another tile kernel, which sums in another order)
+    m16 = ops.gemm_variants().index("256x256_dma_w4x128_m16x128")
+    same_kernel = ops.swiglu_gemm_matches_separate(M, H, K)
+    assert same_kernel == (-(-M // 256) * -(-H // 256) > 96 and H >= 256)
+    kw = {} if same_kernel else ({"variant": m16} if H >= 256 else None)
+    if kw is not None:
+        assert torch.equal(x1, ops.gemm_fp8(xq, sx, w1q, s1, **kw)), "x1"
+        assert torch.equal(x3, ops.gemm_fp8(xq, sx, w3q, s3, **kw)), "x3"
+    # h and its amax: the bits of the pointwise kernel on these x1, x3
+    rh, (rslots, rn) = ops.swiglu_fwd(x1, x3)
+    assert torch.equal(h.view(torch.int16), rh.view(torch.int16)), "h"
+    assert 0 < n <= 1024
+    got = slots[:n].view(torch.float32).max()
+    assert float(got) == float(rh.abs().max().float()) == float(rslots[:rn].view(torch.float32).max())
+    assert_gemm_close(x3, O.emulated_mm_f32(xq.cpu(), sx.cpu()[0], w3q.cpu().t(), s3.cpu()[0]), "x3 vs oracle")
+    # and against the oracle of each stage
+    assert_gemm_close(x1, O.emulated_mm_f32(xq.cpu(), sx.cpu()[0], w1q.cpu().t(), s1.cpu()[0]), "x1 vs oracle")
+    from helpers import assert_bf16_pointwise_close
+    assert_bf16_pointwise_close(h, O.swiglu(x1.cpu(), x3.cpu()), "h vs oracle")
+
+
+def test_fused_swiglu_epilogue_switch_gives_identical_block_results(dev):
+    from olmo_core_amd.nn import feed_forward as ff_mod
+
+    M, D, H = 4096, 512, 1792  # 16 x 7 tiles: the library runs the separate projections on the persistent kernel too
+    assert ops.swiglu_gemm_matches_separate(M, H, D)
+    x, go = seeded((M, D), 1).to(dev), seeded((M, D), 2, std=1e-3).to(dev)
+    res = []
+    for flag in (True, False):
+        ff_mod.FUSE_SWIGLU_EPILOGUE = flag
+        try:
+            res.append(_run(_make(dev, D, H, fuse=True), x, go))
+        finally:
+            ff_mod.FUSE_SWIGLU_EPILOGUE = True
+    for name, u, v in zip(("y", "gx", "gw1", "gw2", "gw3"), *res):
+        assert torch.equal(u, v), name
