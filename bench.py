@@ -25,9 +25,20 @@ import torch
 D_MODEL, HIDDEN, TOKENS = 4096, 11008, 16384
 FP8_MFMA_PEAK_TFLOPS = 5000.0  # MI355X dense fp8 matrix peak
 GEMMS_PER_STEP = 9
-# HBM-side bytes per GEMM launch (L2 fill reads + writes), mean over the 9 launches of a step, from the
-# FETCH_SIZE / WRITE_SIZE counter runs summarised in profiles/gemm_fp8_m16_kernel__mlp7b_traffic_pmc.txt
-GEMM_TRAFFIC_BYTES_PER_LAUNCH = 1.406e9
+TRAFFIC_PROFILE = os.path.join(os.path.dirname(os.path.abspath(__file__)), "profiles", "gemm_fp8_m16_kernel__mlp7b_traffic_pmc.txt")
+
+
+def gemm_traffic_bytes_per_launch():
+    """HBM-side bytes per GEMM launch (L2 fills + write-backs, mean over the GEMM work of a step), taken from the
+    line `traffic_bytes_per_launch: N` of the FETCH_SIZE / WRITE_SIZE counter summary under profiles/ (a figure from
+    rocprofv3 --pmc runs, not measured by this script); None when that file is missing."""
+    try:
+        for line in open(TRAFFIC_PROFILE):
+            if line.startswith("traffic_bytes_per_launch:"):
+                return float(line.split(":")[1].split()[0])
+    except OSError:
+        pass
+    return None
 
 
 def build_mlp(dev):
@@ -236,8 +247,154 @@ def cast_rates(iters: int = 10):
         "us": round(us, 1),
         "GB/s_algorithmic_4B_per_elem": round(4.0 * n / us / 1e3, 1),
         "GB/s_streamed_6B_per_elem": round(6.0 * n / us / 1e3, 1),
+        "frac_hbm_peak_algorithmic": round(4.0 * n / us / 1e3 / HBM_PEAK_GBS, 4),
         "frac_hbm_peak_streamed": round(6.0 * n / us / 1e3 / HBM_PEAK_GBS, 4),
     }
+
+
+def _time_us(fn, iters=10, warmup=3):
+    for _ in range(warmup):
+        fn()
+    start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    start.record()
+    for _ in range(iters):
+        fn()
+    end.record()
+    torch.cuda.synchronize()
+    return start.elapsed_time(end) / iters * 1e3
+
+
+def cast_table():
+    """The HBM-bound kernels of the path one by one at the benchmark's shapes: one JSON line each with the time, the
+    rate on the algorithmic bytes (what any implementation must move: inputs read once, outputs written once) and on
+    the bytes the kernel streams (a second read of the input where a global amax separates two passes), and the
+    fractions of the 8 TB/s HBM peak."""
+    from olmo_core_amd import _C
+    from olmo_core_amd.float8 import ops
+
+    dev = torch.device("cuda:0")
+    e4m3, e5m2 = torch.float8_e4m3fn, torch.float8_e5m2
+
+    def line(kernel, shape, us, alg_bytes, streamed_bytes):
+        print(json.dumps({
+            "kernel": kernel, "shape": "x".join(map(str, shape)), "us": round(us, 1),
+            "GB/s_algorithmic": round(alg_bytes / us / 1e3, 1), "frac_hbm_peak_algorithmic": round(alg_bytes / us / 1e3 / HBM_PEAK_GBS, 3),
+            "GB/s_streamed": round(streamed_bytes / us / 1e3, 1), "frac_hbm_peak_streamed": round(streamed_bytes / us / 1e3 / HBM_PEAK_GBS, 3),
+        }), flush=True)
+
+    for shape in ((TOKENS, D_MODEL), (HIDDEN, D_MODEL), (TOKENS, HIDDEN)):
+        n = shape[0] * shape[1]
+        x = torch.randn(*shape, device=dev).to(torch.bfloat16)
+        y = torch.empty_like(x)
+        line("device copy (torch), for scale", shape, _time_us(lambda: y.copy_(x)), 4 * n, 4 * n)
+        del y
+        line("amax_partials_kernel", shape, _time_us(lambda: ops.amax_partials(x)), 2 * n, 2 * n)
+        slots = ops.amax_partials(x)
+        line("tile_cast_kernel (scale known): row-major + transposed", shape,
+             _time_us(lambda: ops.cast_tensorwise(x, e4m3, want_transposed=True, slots=slots)), 4 * n, 4 * n)
+        line("tile_cast_kernel (scale known): row-major only", shape,
+             _time_us(lambda: ops.cast_tensorwise(x, e4m3, slots=slots)), 3 * n, 3 * n)
+        line("tensorwise cast, fused amax + cast passes: row-major + transposed", shape,
+             _time_us(lambda: ops.cast_tensorwise(x, e4m3, want_transposed=True)), 4 * n, 6 * n)
+        line("rowwise_cast_kernel (single pass)", shape, _time_us(lambda: ops.cast_rowwise(x, e4m3, pow2=True)), 3 * n, 3 * n)
+        line("colamax + per-column transposed cast", shape, _time_us(lambda: ops.cast_colwise_t(x, e4m3, pow2=True)), 3 * n, 5 * n)
+        line("two-product cast (per-row copy + per-column transposed copy)", shape,
+             _time_us(lambda: ops.cast_rows_and_colwise_t(x, e4m3, pow2=True)), 4 * n, 6 * n)
+        del x, slots
+    shape = (TOKENS, HIDDEN)
+    n = shape[0] * shape[1]
+    x1 = torch.randn(*shape, device=dev).to(torch.bfloat16)
+    x3 = torch.randn(*shape, device=dev).to(torch.bfloat16)
+    gh = (torch.randn(*shape, device=dev) * 1e-3).to(torch.bfloat16)
+    line("swiglu_fwd_kernel (+ amax of h)", shape, _time_us(lambda: ops.swiglu_fwd(x1, x3)), 6 * n, 6 * n)
+    s1 = torch.empty(_C.AMAX_SLOTS, dtype=torch.int32, device=dev)
+    s3 = torch.empty(_C.AMAX_SLOTS, dtype=torch.int32, device=dev)
+    st = torch.cuda.current_stream().cuda_stream
+    line("swiglu_bwd_kernel, amax-only pass", shape,
+         _time_us(lambda: _C.lib().mi8_swiglu_bwd(x1.data_ptr(), x3.data_ptr(), gh.data_ptr(), None, None, n, s1.data_ptr(),
+                                                  s3.data_ptr(), st)), 6 * n, 6 * n)
+    line("swiglu backward to float8 (amax pass + swiglu_bwd_cast_kernel): g1, g3 row-major + transposed", shape,
+         _time_us(lambda: ops.swiglu_bwd_cast(x1, x3, gh, e5m2, want_transposed=True)), 10 * n, 16 * n)
+    del x1, x3, gh
+    # grouped (configuration 5): 131072 routed rows of 2048, the benchmark's group sizes
+    _, _, _, _, desc = build_config(5, dev)
+    g = torch.Generator().manual_seed(1005)
+    E, T, top_k, d = 64, 16384, 8, 2048
+    rank = torch.arange(1, E + 1, dtype=torch.float64)
+    pmf = rank ** -1.1
+    pmf = pmf / pmf.sum()
+    logits = torch.randn(T, E, generator=g) + (1.75 * torch.log(pmf)).float()
+    experts = logits.float().softmax(-1).topk(top_k, dim=-1).indices
+    sizes = torch.bincount(experts.reshape(-1), minlength=E).to(dev)
+    indices = torch.sort(experts.reshape(-1).int(), stable=True)[1].int().to(dev)
+    xs = torch.randn(T * top_k, d, device=dev).to(torch.bfloat16)
+    n = xs.numel()
+    line("grouped two-product cast (grouped_colamax + grouped_tile_cast), 64 ragged groups", (T * top_k, d),
+         _time_us(lambda: ops.grouped_cast_rows_and_colwise_t(xs, sizes, e4m3, pow2=True)), 4 * n, 6 * n)
+    del xs
+    xt = torch.randn(T, d, device=dev).to(torch.bfloat16)
+    line("token gather fused into the grouped two-product cast (top-8 of 16384 tokens)", (T * top_k, d),
+         _time_us(lambda: ops.gather_cast_rows_and_colwise_t(xt, indices, top_k, sizes, e4m3, pow2=True)),
+         2 * xt.numel() + 2 * n, 2 * xt.numel() + 2 * n)
+
+
+def power_probe():
+    """What the power limit leaves of the matrix peak: back-to-back MFMAs with nothing else running, and the
+    benchmark's longest-K GEMM, each on all-zero and on random operands (under `rocprofv3 --pmc GRBM_GUI_ACTIVE` the
+    kernel durations and active cycles give the clock in each case)."""
+    from olmo_core_amd import _C
+    from olmo_core_amd.float8 import ops
+
+    dev = torch.device("cuda:0")
+    sink = torch.empty(256 * 256, dtype=torch.float32, device=dev)
+    st = torch.cuda.current_stream().cuda_stream
+    iters = 20000
+    flop = 256 * 4 * iters * 2.0 * 128 ** 3
+    for shape, name in ((1, "16x16x128"), (0, "32x32x64")):
+        for rnd in (0, 1):
+            us = _time_us(lambda: _C.check(_C.lib().mi8_probe_mfma_loop(shape, rnd, iters, 256, sink.data_ptr(), st)), iters=3, warmup=1)
+            print(json.dumps({"probe": f"bare v_mfma_f32_{name}_f8f6f4 loop, 256 workgroups x 4 waves",
+                              "operands": "random bytes" if rnd else "zeros", "ms": round(us / 1e3, 2),
+                              "TFLOP/s": round(flop / us / 1e6, 1), "frac_of_5.0_PFLOP/s": round(flop / us / 1e6 / FP8_MFMA_PEAK_TFLOPS, 3)}), flush=True)
+    one = torch.ones(1, device=dev)
+    for (m, n, k) in ((TOKENS, D_MODEL, HIDDEN), (TOKENS, HIDDEN, D_MODEL)):
+        for rnd in (0, 1):
+            if rnd:
+                a = torch.randn(m, k, device=dev).to(torch.float8_e4m3fn)
+                b = torch.randn(n, k, device=dev).to(torch.float8_e4m3fn)
+            else:
+                a = torch.zeros(m, k, device=dev, dtype=torch.float8_e4m3fn)
+                b = torch.zeros(n, k, device=dev, dtype=torch.float8_e4m3fn)
+            us = _time_us(lambda: ops.gemm_fp8(a, one, b, one), iters=20, warmup=5)
+            print(json.dumps({"probe": f"gemm_fp8_m16_kernel {m}x{n}x{k}", "operands": "N(0,1) cast to e4m3" if rnd else "zeros",
+                              "us": round(us, 1), "TFLOP/s": round(2.0 * m * n * k / us / 1e6, 1),
+                              "frac_of_5.0_PFLOP/s": round(2.0 * m * n * k / us / 1e6 / FP8_MFMA_PEAK_TFLOPS, 3)}), flush=True)
+            del a, b
+
+
+def profile_summary(path):
+    """Print the per-kernel table of a `rocprofv3 --kernel-trace --stats --output-format csv` run (its
+    *_kernel_stats.csv) in the compact form kept under profiles/."""
+    import csv
+    import glob
+
+    files = [path] if os.path.isfile(path) else sorted(glob.glob(os.path.join(path, "**", "*kernel_stats.csv"), recursive=True))
+    if not files:
+        print(f"no *kernel_stats.csv under {path}", file=sys.stderr)
+        sys.exit(2)
+    rows = list(csv.DictReader(open(files[0])))
+    total = sum(float(r["TotalDurationNs"]) for r in rows)
+    print(f"{'kernel':100s} {'calls':>6s} {'avg_us':>9s} {'min_us':>9s} {'max_us':>9s} {'total_ms':>9s} {'pct':>6s}")
+    for r in rows:
+        t = float(r["TotalDurationNs"])
+        if t < 0.001 * total:
+            continue
+        name = " ".join(r["Name"].split())
+        name = name.replace("(anonymous namespace)::", "").replace("mi8::gemm::", "").replace("mi8::", "")
+        print(f"{name[:100]:100s} {int(r['Calls']):6d} {float(r['AverageNs']) / 1e3:9.2f} {float(r['MinNs']) / 1e3:9.2f} "
+              f"{float(r['MaxNs']) / 1e3:9.2f} {t / 1e6:9.3f} {100 * t / total:6.2f}")
+    print(f"(kernels below 0.1 % of the {total / 1e6:.3f} ms of GPU time are left out)")
 
 
 def traffic_probe():
@@ -327,10 +484,17 @@ def main():
                     help="config 5: keep the experts' float8 weight copies across steps (micro-batch steady state)")
     ap.add_argument("--routed", action="store_true",
                     help="config 5: time the whole routed layer (fused gather, experts, weighted scatter)")
+    ap.add_argument("--cast-table", action="store_true", help="time every HBM-bound kernel of the path at the benchmark's shapes")
+    ap.add_argument("--power-probe", action="store_true", help="bare MFMA loops and the GEMM on zero / random operands")
+    ap.add_argument("--profile-summary", type=str, default=None, metavar="DIR_OR_CSV",
+                    help="print the per-kernel table of a rocprofv3 --stats --output-format csv run (no GPU needed)")
     ap.add_argument("--traffic-probe", action="store_true", help="workload for the FETCH_SIZE/WRITE_SIZE counter runs")
     ap.add_argument("--gemm", type=str, default=None, metavar="M,N,K[;M,N,K...]",
                     help="time single scaled GEMMs of these shapes (library's choice of kernel) instead of a step")
     ns = ap.parse_args()
+    if ns.profile_summary:
+        profile_summary(ns.profile_summary)
+        return
     if ns.gpus != 1:
         print("bench.py: this build measures the float8 linear path on ONE GPU; --gpus must be 1", file=sys.stderr)
         sys.exit(2)
@@ -342,6 +506,12 @@ def main():
 
     if ns.traffic_probe:
         traffic_probe()
+        return
+    if ns.cast_table:
+        cast_table()
+        return
+    if ns.power_probe:
+        power_probe()
         return
     if ns.gemm:
         gemm_shapes([tuple(int(v) for v in part.split(",")) for part in ns.gemm.split(";")], ns.steps, ns.warmup)
@@ -407,7 +577,8 @@ def main():
             "peak": FP8_MFMA_PEAK_TFLOPS,
             "unit": "TFLOP/s",
             "frac": round(achieved / FP8_MFMA_PEAK_TFLOPS, 4),
-            "traffic": GEMM_TRAFFIC_BYTES_PER_LAUNCH,
+            "traffic": gemm_traffic_bytes_per_launch(),
+            "traffic_source": "profiles/gemm_fp8_m16_kernel__mlp7b_traffic_pmc.txt (rocprofv3 --pmc FETCH_SIZE, WRITE_SIZE; not measured in this run)",
             "avg_launch_us": round(avg_gemm_s * 1e6, 2),
             "gemm_share_of_step": round(sum(gemm_ms) / ns.steps / ms_per_step, 4),
         },

@@ -348,6 +348,14 @@ int mi8_moe_binned_scatter_wgrad(const void* x, const void* grad, int dtype, int
                                  const int32_t* indices, const int32_t* bins, int32_t experts, int64_t capacity,
                                  int32_t top_k, void* out, void* stream);
 
+/* ---------------------------------------------------------------------------------------------
+ * Diagnostics (no counterpart in the reference): `workgroups` x 4 waves issue back-to-back fp8 MFMAs on resident
+ * registers, 2 * 128^3 flop per wave and iteration, shape 0 = 32x32x64, 1 = 16x16x128, on all-zero or on random
+ * operand bytes.  Timed by the caller; on random operands this is the matrix throughput the chip sustains under
+ * its power limit.  sink: float32 [workgroups * 256], overwritten.
+ * ------------------------------------------------------------------------------------------- */
+int mi8_probe_mfma_loop(int mfma_shape, int random_operands, int iterations, int workgroups, float* sink, void* stream);
+
 #ifdef __cplusplus
 }
 #endif
