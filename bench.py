@@ -398,33 +398,51 @@ def profile_summary(path):
 
 
 def traffic_probe():
-    """Workload for the rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs: a plain 256 MiB device copy (the
-    calibration: 268435456 bytes read and written), then the three GEMM shapes of the benchmark step and the
-    amax + cast of the 16384 x 4096 activation, a few launches each, nothing timed."""
-    from olmo_core_amd.float8 import ops
-
+    """Workload for the rocprofv3 --pmc runs (FETCH_SIZE, WRITE_SIZE, matrix-pipe counters): a plain 256 MiB device
+    copy (the calibration: 268435456 bytes read and written per launch), then three steps of the benchmark's
+    feed-forward block, nothing timed."""
     dev = torch.device("cuda:0")
-    e4m3, e5m2 = torch.float8_e4m3fn, torch.float8_e5m2
     src = torch.randint(0, 255, (1 << 28,), dtype=torch.uint8, device=dev)
     dst = torch.empty_like(src)
     for _ in range(3):
         dst.copy_(src)
     torch.cuda.synchronize()
-    one = torch.ones(1, device=dev)
-    shapes = [(TOKENS, HIDDEN, D_MODEL, e4m3), (TOKENS, D_MODEL, HIDDEN, e5m2), (HIDDEN, D_MODEL, TOKENS, e5m2)]
-    for M, N, K, da in shapes:
-        a = torch.randn(M, K, device=dev).to(da)
-        b = torch.randn(N, K, device=dev).to(e4m3)
-        for _ in range(3):
-            ops.gemm_fp8(a, one, b, one)
-        torch.cuda.synchronize()
-        del a, b
-    x = torch.randn(TOKENS, D_MODEL, device=dev, dtype=torch.bfloat16)
+    del src, dst
+    mlp, x, go = build_mlp(dev)
     for _ in range(3):
-        slots = ops.amax_partials(x)
-        ops.cast_tensorwise(x, e4m3, want_transposed=True, slots=slots)
+        step(mlp, x, go)
     torch.cuda.synchronize()
     print("traffic probe done", flush=True)
+
+
+def counter_summary(path):
+    """Per kernel and counter: dispatches, mean counter value and mean duration of a `rocprofv3 --pmc ... --kernel-trace
+    --output-format csv` run (its *_counter_collection.csv)."""
+    import csv
+    import glob
+    from collections import defaultdict
+
+    files = [path] if os.path.isfile(path) else sorted(glob.glob(os.path.join(path, "**", "*counter_collection.csv"), recursive=True))
+    if not files:
+        print(f"no *counter_collection.csv under {path}", file=sys.stderr)
+        sys.exit(2)
+    acc = defaultdict(lambda: [0, 0.0, 0.0])
+    for r in csv.DictReader(open(files[0])):
+        name = " ".join(r["Kernel_Name"].split())
+        name = name.replace("(anonymous namespace)::", "").replace("mi8::gemm::", "").replace("mi8::", "")
+        if len(name) > 90:
+            name = name[:87] + "..."
+        key = (name, int(r["Grid_Size"]), r["Counter_Name"])
+        a = acc[key]
+        a[0] += 1
+        a[1] += float(r["Counter_Value"])
+        a[2] += (int(r["End_Timestamp"]) - int(r["Start_Timestamp"])) / 1e3
+    print(f"{'kernel':90s} {'grid':>9s} {'counter':28s} {'n':>4s} {'mean value':>16s} {'mean us':>9s}")
+    for (name, grid, counter), (n, v, us) in sorted(acc.items(), key=lambda kv: -kv[1][2]):
+        if us / n < 5.0:
+            continue
+        print(f"{name:90s} {grid:9d} {counter:28s} {n:4d} {v / n:16.1f} {us / n:9.1f}")
+    print("(kernels shorter than 5 us are left out)")
 
 
 def step(mlp, x, go):
@@ -488,12 +506,17 @@ def main():
     ap.add_argument("--power-probe", action="store_true", help="bare MFMA loops and the GEMM on zero / random operands")
     ap.add_argument("--profile-summary", type=str, default=None, metavar="DIR_OR_CSV",
                     help="print the per-kernel table of a rocprofv3 --stats --output-format csv run (no GPU needed)")
-    ap.add_argument("--traffic-probe", action="store_true", help="workload for the FETCH_SIZE/WRITE_SIZE counter runs")
+    ap.add_argument("--counter-summary", type=str, default=None, metavar="DIR_OR_CSV",
+                    help="print per-kernel means of a rocprofv3 --pmc --output-format csv run (no GPU needed)")
+    ap.add_argument("--traffic-probe", action="store_true", help="workload for the rocprofv3 --pmc counter runs (a calibration copy, then three benchmark steps)")
     ap.add_argument("--gemm", type=str, default=None, metavar="M,N,K[;M,N,K...]",
                     help="time single scaled GEMMs of these shapes (library's choice of kernel) instead of a step")
     ns = ap.parse_args()
     if ns.profile_summary:
         profile_summary(ns.profile_summary)
+        return
+    if ns.counter_summary:
+        counter_summary(ns.counter_summary)
         return
     if ns.gpus != 1:
         print("bench.py: this build measures the float8 linear path on ONE GPU; --gpus must be 1", file=sys.stderr)
