@@ -306,16 +306,19 @@ int mi8_swiglu_bwd_cast(const void* x1, const void* x3, const void* gh, int64_t 
 int mi8_moe_gather(const void* x, int dtype, int64_t tokens, int64_t hidden, const int32_t* indices,
                    const void* weights, int w_dtype, int32_t top_k, void* out, void* stream);
 
-/* mi8_moe_gather (unweighted) followed by mi8_grouped_cast_rows_and_colwise_t, without the gathered high-precision
+/* mi8_moe_gather (weights NULL: unweighted) followed by mi8_grouped_cast_rows_and_colwise_t, without the gathered high-precision
  * tensor in between: the token rows are read through `indices` in both passes (x stays cache resident: every token
  * row is read top_k times), and only the float8 products are written - the per-row cast [tokens * top_k, ld_rows]
  * with its scales and the per-(group, column) transposed cast with its scales, i.e. the operands of the expert
  * GEMMs of a dropless mixture-of-experts layer (the copy kernel of src/olmo_core/kernels/moe.py:42-139 fused with the
- * quantisation that follows it in a float8 expert layer; its backward stays mi8_moe_scatter).  A slot index outside
+ * quantisation that follows it in a float8 expert layer; its backward stays mi8_moe_scatter).  With weights (the
+ * backward of the weighted scatter: grad_output rows times the router weight of the slot) every product is rounded to
+ * the element type before it is quantised, as mi8_moe_gather writes it.  A slot index outside
  * [0, tokens * top_k) reads as a row of zeros.  Workspaces, outputs and group semantics as
  * mi8_grouped_cast_rows_and_colwise_t with T = tokens * top_k; bytes and scales equal the two-call route. */
 int mi8_moe_gather_cast_rows_and_colwise_t(const void* x, int hp_dtype, int64_t tokens, int64_t cols,
-                                           const int32_t* indices, int32_t top_k, const int64_t* group_sizes,
+                                           const int32_t* indices, int32_t top_k, const void* weights, int w_dtype,
+                                           const int64_t* group_sizes,
                                            int32_t num_groups, int fp8_dtype, uint32_t flags, uint32_t* amax_ws,
                                            void* out_t, int64_t ld_t, float* scale_out, uint32_t* row_amax_ws,
                                            void* out_rows, int64_t ld_rows, float* row_scale_out, void* stream);

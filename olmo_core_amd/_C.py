@@ -139,8 +139,8 @@ _SIGNATURES = {
     ),
     "mi8_moe_gather_cast_rows_and_colwise_t": (
         c_int,
-        [c_void_p, c_int, c_int64, c_int64, c_void_p, c_int32, c_void_p, c_int32, c_int, c_uint32, c_void_p, c_void_p,
-         c_int64, c_void_p, c_void_p, c_void_p, c_int64, c_void_p, c_void_p],
+        [c_void_p, c_int, c_int64, c_int64, c_void_p, c_int32, c_void_p, c_int, c_void_p, c_int32, c_int, c_uint32, c_void_p,
+         c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_int64, c_void_p, c_void_p],
     ),
     "mi8_grouped_gemm_fp8": (
         c_int,

@@ -141,6 +141,24 @@ __device__ __forceinline__ int64_t gathered_row(const int32_t* gather, int top_k
     return (slot < 0 || slot >= src_rows * top_k) ? -1 : slot / top_k;
 }
 
+// Weight of the slot that logical row r holds (weighted gather: the row is the token's row times this weight, the
+// product rounded to the element type as the gather kernel does); 1 without weights.
+__device__ __forceinline__ float gathered_weight(const int32_t* gather, const void* w, int w_dtype, int64_t r, bool ok)
+{
+    if (!w || !ok) return 1.0f;
+    const int64_t slot = gather[r];
+    if (w_dtype == MI8_F32) return reinterpret_cast<const float*>(w)[slot];
+    const uint16_t v = reinterpret_cast<const uint16_t*>(w)[slot];
+    return w_dtype == MI8_BF16 ? bits_to_f32((uint32_t)v << 16) : (float)__builtin_bit_cast(_Float16, v);
+}
+
+template <int HP>
+__device__ __forceinline__ float round_to_hp(float f)
+{
+    if constexpr (HP == MI8_BF16) return (float)(__bf16)f;
+    return f;
+}
+
 // LDS holds the transposed tile as 128 columns x 128 row-bytes.  Two columns share a 256-byte line; the
 // 16-byte chunk index inside the line is XORed with a function of the column's group of eight so that
 // both the dword writes (lanes spread over 16 column groups x 4 row groups) and the 16-byte reads
@@ -162,7 +180,7 @@ __device__ __forceinline__ void tile_cast_body(const void* x, int64_t row_end, i
                                                int64_t dst0, int64_t dst_end, uint32_t* lds_t,
                                                uint8_t* out_r = nullptr, int64_t ld_r = 0, const float* row_scale = nullptr,
                                                int64_t row_scale_row0 = 0, const int32_t* gather = nullptr, int top_k = 1,
-                                               int64_t src_rows = 0)
+                                               int64_t src_rows = 0, const void* gather_w = nullptr, int gather_w_dtype = 0)
 {
     const int tid = threadIdx.x;
     const int wave = tid >> 6, lane = tid & 63;
@@ -184,6 +202,11 @@ __device__ __forceinline__ void tile_cast_body(const void* x, int64_t row_end, i
                 ok = ok && src >= 0;
             }
             HpVec<HP>::load8(xb + (src * cols + c8) * HpVec<HP>::kBytes, ok, f[it][j]);
+            if (gather_w) {  // (uniform) weighted gather: the product, rounded to the element type
+                const float w = gathered_weight(gather, gather_w, gather_w_dtype, r, ok);
+#pragma unroll
+                for (int k = 0; k < 8; ++k) f[it][j][k] = round_to_hp<HP>(f[it][j][k] * w);
+            }
         }
 
     // the rows' own scales, read ahead of the stores below (a read placed between them would wait for them)
@@ -434,6 +457,8 @@ struct GroupedCastArgs {
     const int32_t* gather;
     int top_k;
     int64_t src_rows;
+    const void* gather_w;  // optional weight per slot (weighted gather), of element type gather_w_dtype
+    int gather_w_dtype;
 };
 
 // Tile p of the padded row space (128 rows each; group e owns ceil(m_e / 128) consecutive tiles) -> its group,
@@ -471,6 +496,23 @@ __device__ __forceinline__ bool locate_padded_tile(const int64_t* sizes, int E, 
     return true;
 }
 
+// the 16 bytes of a row times the row's gather weight, each product rounded to the element type
+template <int HP>
+__device__ __forceinline__ uint4 scale_vec(uint4 v, float w)
+{
+    uint32_t d[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        if constexpr (HP == MI8_BF16) {
+            const __bf16 lo = (__bf16)(bits_to_f32(d[i] << 16) * w), hi = (__bf16)(bits_to_f32(d[i] & 0xFFFF0000u) * w);
+            d[i] = (uint32_t)__builtin_bit_cast(uint16_t, lo) | ((uint32_t)__builtin_bit_cast(uint16_t, hi) << 16);
+        } else {
+            d[i] = f32_to_bits(bits_to_f32(d[i]) * w);
+        }
+    }
+    return make_uint4(d[0], d[1], d[2], d[3]);
+}
+
 template <int HP>
 __global__ __launch_bounds__(kThreads) void grouped_colamax_kernel(GroupedCastArgs a)
 {
@@ -495,9 +537,11 @@ __global__ __launch_bounds__(kThreads) void grouped_colamax_kernel(GroupedCastAr
         uint32_t rowacc[4] = {0, 0, 0, 0};
         const int64_t src = a.gather ? gathered_row(a.gather, a.top_k, a.src_rows, r, r < row_end) : r;
         if (c8 < a.cols && r < row_end && src >= 0) {
+            const float w = gathered_weight(a.gather, a.gather_w, a.gather_w_dtype, r, true);
 #pragma unroll
             for (int k = 0; k < NV; ++k) {
-                const uint4 v = reinterpret_cast<const uint4*>(xb + (src * a.cols + c8) * HpVec<HP>::kBytes)[k];
+                uint4 v = reinterpret_cast<const uint4*>(xb + (src * a.cols + c8) * HpVec<HP>::kBytes)[k];
+                if (a.gather_w) v = scale_vec<HP>(v, w);
                 absmax_accumulate<HP>(v, acc[k]);
                 if (a.row_amax) absmax_accumulate<HP>(v, rowacc);
             }
@@ -773,7 +817,7 @@ __global__ __launch_bounds__(kThreads) void grouped_tile_cast_kernel(GroupedCast
     for (int i = 0; i < 8; ++i) sc[i] = s_scale[8 * cl + i];
     const int64_t dst0 = (int64_t)kTile * blockIdx.y;
     tile_cast_body<HP, FP8, SW>(a.x, row_end, a.cols, row0, col0, sc, nullptr, 0, a.out_t, a.ld_t, dst0, a.ld_t, lds_t,
-                                a.out_r, a.ld_r, s_row_scale, row0, a.gather, a.top_k, a.src_rows);
+                                a.out_r, a.ld_r, s_row_scale, row0, a.gather, a.top_k, a.src_rows, a.gather_w, a.gather_w_dtype);
 }
 
 // ---- dispatch helpers ------------------------------------------------------------------------------
@@ -1251,7 +1295,8 @@ namespace {
 int grouped_cast_launch(const char* what, const void* x, int hp_dtype, int64_t T, int64_t cols, const int64_t* group_sizes,
                         int32_t num_groups, int fp8_dtype, uint32_t flags, uint32_t* amax_ws, void* out_t, int64_t ld_t,
                         float* scale_out, uint32_t* row_amax_ws, void* out_rows, int64_t ld_rows, float* row_scale_out,
-                        void* stream, const int32_t* gather = nullptr, int32_t top_k = 1, int64_t src_rows = 0)
+                        void* stream, const int32_t* gather = nullptr, int32_t top_k = 1, int64_t src_rows = 0,
+                        const void* gather_w = nullptr, int gather_w_dtype = 0)
 {
     MI8_REQUIRE(x && group_sizes && amax_ws && out_t && scale_out, MI8_ERR_ARG, "%s: null pointer", what);
     MI8_REQUIRE(!gather || (top_k > 0 && src_rows > 0 && src_rows * top_k < ((int64_t)1 << 31)), MI8_ERR_ARG,
@@ -1271,7 +1316,8 @@ int grouped_cast_launch(const char* what, const void* x, int hp_dtype, int64_t T
     MI8_REQUIRE(ptiles <= 65535, MI8_ERR_UNSUPPORTED, "%s: too many row tiles (%lld)", what, (long long)ptiles);
     const bool pow2 = (flags & MI8_FLAG_POW2_SCALE) != 0;
     GroupedCastArgs a{x, T, cols, group_sizes, num_groups, pow2, amax_ws, (uint8_t*)out_t, ld_t, scale_out,
-                      out_rows ? row_amax_ws : nullptr, (uint8_t*)out_rows, ld_rows, row_scale_out, gather, top_k, src_rows};
+                      out_rows ? row_amax_ws : nullptr, (uint8_t*)out_rows, ld_rows, row_scale_out, gather, top_k, src_rows, gather_w,
+                      gather_w_dtype};
     hipStream_t st = (hipStream_t)stream;
     dim3 grid((unsigned)ceil_div(cols, kTile), (unsigned)ptiles);
     int rc = MI8_OK;
@@ -1365,7 +1411,8 @@ extern "C" int mi8_grouped_swiglu_bwd(const void* x1, const void* x2, const void
 }
 
 extern "C" int mi8_moe_gather_cast_rows_and_colwise_t(const void* x, int hp_dtype, int64_t tokens, int64_t cols,
-                                                      const int32_t* indices, int32_t top_k, const int64_t* group_sizes,
+                                                      const int32_t* indices, int32_t top_k, const void* weights,
+                                                      int w_dtype, const int64_t* group_sizes,
                                                       int32_t num_groups, int fp8_dtype, uint32_t flags,
                                                       uint32_t* amax_ws, void* out_t, int64_t ld_t, float* scale_out,
                                                       uint32_t* row_amax_ws, void* out_rows, int64_t ld_rows,
@@ -1375,7 +1422,9 @@ extern "C" int mi8_moe_gather_cast_rows_and_colwise_t(const void* x, int hp_dtyp
     MI8_REQUIRE(tokens > 0 && top_k > 0, MI8_ERR_ARG, "mi8_moe_gather_cast_rows_and_colwise_t: empty input");
     MI8_REQUIRE(!(flags & MI8_FLAG_AMAX_READY), MI8_ERR_ARG,
                 "mi8_moe_gather_cast_rows_and_colwise_t: the amax pass is part of this call");
+    MI8_REQUIRE(!weights || w_dtype == MI8_BF16 || w_dtype == MI8_F16 || w_dtype == MI8_F32, MI8_ERR_ARG,
+                "mi8_moe_gather_cast_rows_and_colwise_t: unknown weight dtype %d", w_dtype);
     return grouped_cast_launch("mi8_moe_gather_cast_rows_and_colwise_t", x, hp_dtype, tokens * top_k, cols, group_sizes,
                                num_groups, fp8_dtype, flags, amax_ws, out_t, ld_t, scale_out, row_amax_ws, out_rows,
-                               ld_rows, row_scale_out, stream, indices, top_k, tokens);
+                               ld_rows, row_scale_out, stream, indices, top_k, tokens, weights, w_dtype);
 }

@@ -567,10 +567,11 @@ def grouped_cast_rows_and_colwise_t(
 
 def gather_cast_rows_and_colwise_t(
     x: torch.Tensor, indices: torch.Tensor, top_k: int, group_sizes: torch.Tensor, fp8_dtype: torch.dtype, *,
-    pow2: bool = False,
+    pow2: bool = False, weights: Optional[torch.Tensor] = None,
 ) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]:
     """
-    The unweighted token gather of a dropless-MoE layer (row ``i`` of the expert-sorted side is token
+    The token gather of a dropless-MoE layer (``weights``, one per slot: every gathered row times its slot's weight,
+    rounded to the element type - the backward of the weighted scatter) (row ``i`` of the expert-sorted side is token
     ``indices[i] // top_k`` of ``x [tokens, cols]``) fused with :func:`grouped_cast_rows_and_colwise_t`: the gathered
     bf16 tensor is never written.  Returns ``(q [tokens * top_k, cols], row_scale, q_t [cols, ld_t], col_scale [E, cols])``
     with the bytes and scales of the two-step route.
@@ -590,9 +591,16 @@ def gather_cast_rows_and_colwise_t(
     q = torch.empty((T, cols), dtype=fp8_dtype, device=x.device)
     row_scale = torch.empty(T, dtype=torch.float32, device=x.device)
     ws = _grouped_amax_workspace(T, cols, E, x.device)
+    wp, wd = None, 0
+    if weights is not None:
+        if weights.dim() != 1 or weights.shape[0] != T or weights.device != x.device:
+            raise ValueError(f"gather_cast_rows_and_colwise_t: expected {T} weights on {x.device}")
+        weights = weights.contiguous()
+        wd = {torch.bfloat16: _C.MI8_BF16, torch.float32: _C.MI8_F32, torch.float16: _C.MI8_F16}[weights.dtype]
+        wp = weights.data_ptr()
     _C.check(
         _C.lib().mi8_moe_gather_cast_rows_and_colwise_t(
-            x.data_ptr(), _HP_CODE[x.dtype], tokens, cols, indices.data_ptr(), top_k, sizes.data_ptr(), E,
+            x.data_ptr(), _HP_CODE[x.dtype], tokens, cols, indices.data_ptr(), top_k, wp, wd, sizes.data_ptr(), E,
             _FP8_CODE[fp8_dtype], _flags(pow2), ws.data_ptr(), q_t.data_ptr(), ld_t, scale.data_ptr(),
             ws.data_ptr() + 4 * E * cols, q.data_ptr(), cols, row_scale.data_ptr(), _stream(x),
         ),

@@ -31,9 +31,11 @@ STAGE_SINK = None
 
 class _Float8DroplessMLP(torch.autograd.Function):
     @staticmethod
-    def forward(ctx, x, w1, w2, w3, sizes, num_experts, pow2, indices=None, top_k=1, kept=None):
+    def forward(ctx, x, w1, w2, w3, sizes, num_experts, pow2, indices=None, top_k=1, kept=None, scatter_weights=None):
         # indices: None - the rows of x are already sorted by expert; else x is [tokens, D] in token order and row i
-        # of the expert-sorted side is token indices[i] // top_k: the gather is fused into the casts of x
+        # of the expert-sorted side is token indices[i] // top_k: the gather is fused into the casts of x.
+        # scatter_weights (with indices): the expert outputs are scattered back to token order, weighted per slot,
+        # inside this function, so that the backward can quantise the weighted gather of grad_output directly
         E = num_experts
         D = x.shape[1]
         T = x.shape[0] if indices is None else x.shape[0] * top_k
@@ -88,23 +90,48 @@ class _Float8DroplessMLP(torch.autograd.Function):
         y = ops.grouped_gemm_fp8(hq, sh, w2t, s2, sizes, n=D, k=H, b_group_stride=Hp, sb_group_stride=D)
         none = x.new_empty(0)
         opt = lambda t: none if t is None else t  # noqa: E731
+        y_sorted = None
+        ctx.scattered = scatter_weights is not None
+        if ctx.scattered:
+            from ..ops import moe as moe_ops
+
+            if indices is None:
+                raise ValueError("scatter_weights needs the permutation (indices)")
+            if len(need) > 10 and need[10]:
+                y_sorted = y  # the router-weight gradient is a dot product with the unweighted expert output
+            y = moe_ops._scatter(y, indices, scatter_weights, top_k)
         ctx.save_for_backward(opt(xt), opt(sxc), x1, x2, opt(ht), opt(shc), opt(w1t), opt(s1c), opt(w3t), opt(s3c),
-                              opt(w2q), opt(s2r), sizes, opt(indices))
+                              opt(w2q), opt(s2r), sizes, opt(indices), opt(scatter_weights), opt(y_sorted))
         ctx.top_k = top_k if indices is not None else 0
         ctx.meta = (E, T, D, H, Hp, pow2, (x.dtype, w1.dtype, w2.dtype, w3.dtype))
         return y
 
     @staticmethod
     def backward(ctx, gy):
-        xt, sxc, x1, x2, ht, shc, w1t, s1c, w3t, s3c, w2q, s2r, sizes, indices = ctx.saved_tensors
+        (xt, sxc, x1, x2, ht, shc, w1t, s1c, w3t, s3c, w2q, s2r, sizes, indices, scatter_weights,
+         y_sorted) = ctx.saved_tensors
         E, T, D, H, Hp, pow2, (x_dt, w1_dt, w2_dt, w3_dt) = ctx.meta
-        gy = gy.reshape(T, D).contiguous()
+        gy = gy.reshape(-1, D).contiguous()
         if gy.dtype != x_dt:
             gy = gy.to(x_dt)
         need_x, need_w1, need_w2, need_w3 = ctx.needs_input_grad[:4]
 
-        gw2 = None
-        if need_w2:
+        gw2 = g_router = None
+        if ctx.scattered:
+            # gy is in token order: the gradient of the expert outputs is its weighted gather, which goes straight to
+            # float8 (both layouts) without being written in bf16
+            from ..ops import moe as moe_ops
+
+            if y_sorted.numel():
+                g_router = moe_ops._scatter_wgrad(y_sorted, gy, indices, ctx.top_k)
+                if g_router.dtype != scatter_weights.dtype:
+                    g_router = g_router.to(scatter_weights.dtype)
+            gyq, sgy, gyt, sgyc = ops.gather_cast_rows_and_colwise_t(gy, indices, ctx.top_k, sizes, _E4M3, pow2=pow2,
+                                                                     weights=scatter_weights)
+            if need_w2:
+                gw2 = ops.grouped_wgrad_fp8(ht, shc, gyt, sgyc, sizes, tokens=T, out_dtype=x_dt).reshape(E * H, D)
+            del gyt
+        elif need_w2:
             gyq, sgy, gyt, sgyc = ops.grouped_cast_rows_and_colwise_t(gy, sizes, _E4M3, pow2=pow2)
             # gw2[e] [H, D] = h_e^T @ gy_e : contraction over the group's tokens
             gw2 = ops.grouped_wgrad_fp8(ht, shc, gyt, sgyc, sizes, tokens=T, out_dtype=x_dt).reshape(E * H, D)
@@ -156,17 +183,21 @@ class _Float8DroplessMLP(torch.autograd.Function):
             from ..ops import moe as moe_ops
 
             gx = moe_ops._scatter(gx, indices, None, ctx.top_k)
-        return gx, as_param(gw1, w1_dt), as_param(gw2, w2_dt), as_param(gw3, w3_dt), None, None, None, None, None, None
+        return (gx, as_param(gw1, w1_dt), as_param(gw2, w2_dt), as_param(gw3, w3_dt), None, None, None, None, None, None,
+                g_router)
 
 
 @torch.compiler.disable
 def float8_dropless_mlp(x, w1, w2, w3, batch_size_per_expert, num_experts: int, pow2: bool = True, indices=None,
-                        top_k: int = 1, kept=None):
+                        top_k: int = 1, kept=None, scatter_weights=None):
     """``gmm(silu(gmm(x, w1^T)) * gmm(x, w3^T), w2)`` with float8 grouped GEMMs; ``x`` is ``[T, d_model]`` bf16 with
     rows sorted by expert, or, with ``indices`` (int32 ``[tokens * top_k]``, the slot held by each sorted row),
     ``[tokens, d_model]`` in token order: the result is then the expert output of the gathered rows,
-    ``[tokens * top_k, d_model]``, and the gather never writes its bf16 result."""
-    return _Float8DroplessMLP.apply(x, w1, w2, w3, batch_size_per_expert, num_experts, pow2, indices, top_k, kept)
+    ``[tokens * top_k, d_model]``, and the gather never writes its bf16 result.  With ``scatter_weights`` (one router
+    weight per slot) the weighted scatter back to token order happens here as well (result ``[tokens, d_model]``), and
+    the backward quantises the weighted gather of the incoming gradient without writing it in bf16 either."""
+    return _Float8DroplessMLP.apply(x, w1, w2, w3, batch_size_per_expert, num_experts, pow2, indices, top_k, kept,
+                                    scatter_weights)
 
 
 class DroplessMoEMLP(nn.Module):
@@ -247,6 +278,19 @@ class DroplessMoEMLP(nn.Module):
                                 indices=indices, top_k=top_k, kept=self.weight_operands())
         return y.to(x.dtype)
 
+    def forward_routed(self, x: torch.Tensor, indices: torch.Tensor, expert_weights: torch.Tensor, top_k: int,
+                       batch_size_per_expert: torch.Tensor) -> torch.Tensor:
+        """``scatter(forward(gather(x, ...)), ..., expert_weights, ...)`` (``olmo_core_amd.ops.moe``) as one autograd
+        function: ``x`` ``(tokens, d_model)`` and the result are in token order; neither the gathered inputs nor, in
+        backward, the weighted gather of the incoming gradient is written in bf16."""
+        x2 = x.reshape(-1, self.d_model)
+        if x2.dtype != torch.bfloat16:
+            x2 = x2.to(torch.bfloat16)
+        y = float8_dropless_mlp(x2, self.w1, self.w2, self.w3, batch_size_per_expert, self.num_experts,
+                                indices=indices, top_k=top_k, kept=self.weight_operands(),
+                                scatter_weights=expert_weights)
+        return y.to(x.dtype)
+
 
 class ParallelDroplessMLP(nn.Module):
     """
@@ -308,6 +352,8 @@ class ParallelDroplessMLP(nn.Module):
         from ..ops import moe as moe_ops
 
         x = x.view(-1, x.shape[-1])
+        if self.fuse_gather and x.is_cuda and expert_weights is not None:
+            return self.mlp.forward_routed(x, indices, expert_weights, top_k, batch_size_per_expert)
         if self.fuse_gather and x.is_cuda:
             x = self.mlp.forward_gathered(x, indices, top_k, batch_size_per_expert)
         else:

@@ -168,6 +168,21 @@ def test_gather_fused_with_the_grouped_cast(dev, sl, hs, ne, top_k, pow2):
             seg += pad
         start += n
 
+    # weighted: the rows of the weighted gather, quantised
+    w = torch.rand((sl * top_k,), generator=torch.Generator().manual_seed(5)).to(torch.bfloat16)
+    qw, srw, qtw, scw = f8.gather_cast_rows_and_colwise_t(d(x), d(indices), top_k, d(sizes), E4M3, pow2=pow2, weights=d(w))
+    xw_dev = ops._gather(d(x), d(indices), d(w), top_k)
+    assert torch.equal(xw_dev.cpu(), M.gather(x, indices, w, top_k))
+    q2w, sr2w, qt2w, sc2w = f8.grouped_cast_rows_and_colwise_t(xw_dev, d(sizes), E4M3, pow2=pow2)
+    assert torch.equal(u8(qw), u8(q2w)) and torch.equal(srw.cpu(), sr2w.cpu())
+    seg = 0
+    for e, n in enumerate(sizes.tolist()):
+        if n:
+            pad = (n + 127) // 128 * 128
+            assert torch.equal(u8(qtw[:, seg:seg + pad]), u8(qt2w[:, seg:seg + pad])), f"expert {e}: weighted, transposed copy"
+            assert_scale_equal(scw[e], sc2w[e], f"expert {e}: weighted, column scales")
+            seg += pad
+
     # a slot index that points nowhere reads as a row of zeros (zero bytes; scale of an all-zero row)
     bad = indices.clone()
     bad[0] = sl * top_k + 5
