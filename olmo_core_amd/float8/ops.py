@@ -3,8 +3,10 @@ Torch-level wrappers over the C ABI: quantised operands and the scaled GEMM.
 
 torch is used here for device memory and streams only: every wrapper allocates its outputs with
 ``torch.empty`` on the input's device, passes raw pointers plus the current HIP stream to
-``libmi8.so``, and returns tensors.  Nothing here computes on the host and nothing falls back to
-PyTorch arithmetic.
+``libmi8.so``, and returns tensors.  Nothing in this file computes on the host or falls back to PyTorch
+arithmetic.  (What the callers in ``linear.py`` leave to torch is what the reference leaves in high precision
+too: a GEMM whose two cast configs are DISABLED - ``rowwise_with_gw_hp``'s grad_weight - is a bf16 ``torch.mm``,
+and the bias is added by ``+``.)
 """
 
 from __future__ import annotations
