@@ -171,12 +171,16 @@ int mi8_gemm_fp8_accumulate(const void* a, int a_dtype, int64_t lda, const void*
  * Every workgroup computes matching 128-column tiles of x1 and x3 and forms h in its epilogue, so x1 and x3 are written
  * once and never read back.  A fp8 [M, lda]; B1, B3 fp8 [H, ldb] of one type; single scales (float32 [1] each);
  * x1, x3, h bf16 [M, ldc]; slots_h must hold MI8_AMAX_SLOTS uint32.  Needs M >= 256, H >= 128, H % 8 == 0,
- * K % 128 == 0 (MI8_ERR_UNSUPPORTED otherwise: run the three calls it stands for). */
+ * K % 128 == 0 (MI8_ERR_UNSUPPORTED otherwise: run the three calls it stands for).
+ * x_codes: NULL, or uint16[mi8_rowseg_code_count(M, H)] that receives the row-segment codes of the element-wise
+ * larger of x1 and x3 (what mi8_rowseg_max_codes(x1, x3) computes; needs H % 64 == 0), for the backward pass's
+ * mi8_swiglu_bwd_amax_from_codes. */
 int mi8_gemm_fp8_swiglu_matches_separate(int64_t M, int64_t H, int64_t K); /* host only: 1 if the fused launch takes
     the shape and mi8_gemm_fp8 would run both projections on the same tile kernel, so that the bits agree as well */
 int mi8_gemm_fp8_swiglu(const void* a, int a_dtype, int64_t lda, const void* b1, const void* b3, int b_dtype, int64_t ldb,
                         int64_t M, int64_t H, int64_t K, const float* sa, const float* sb1, const float* sb3, void* x1,
-                        void* x3, void* h, int64_t ldc, uint32_t* slots_h, int32_t* n_slots_used, void* stream);
+                        void* x3, void* h, int64_t ldc, uint32_t* slots_h, int32_t* n_slots_used, uint16_t* x_codes,
+                        void* stream);
 
 /* The same product with K cut into `splits` slices, for problems whose few output tiles would leave most of the
  * GPU idle (a few hundred rows of A against a weight matrix): every slice is summed by its own workgroups into
@@ -285,6 +289,32 @@ int mi8_swiglu_bwd_cast(const void* x1, const void* x3, const void* gh, int64_t 
                         const uint32_t* slots_g1, const uint32_t* slots_g3, int32_t n_slots, int fp8_dtype, uint32_t flags,
                         void* out1, void* out3, int64_t ld_out, void* out1_t, void* out3_t, int64_t ld_t,
                         float* scale_out1, float* scale_out3, void* stream);
+
+/* The amax of g1 and g3 without computing every element (the tensorwise scale of the gradient operands,
+ * torchao tensor_to_amax over what src/olmo_core/nn/feed_forward.py:171 back-propagates).
+ *
+ * A row segment is 64 consecutive columns of a row (the last one of a row may be shorter).  Its code is the largest
+ * magnitude in it as a 16-bit integer: the exponent and mantissa bits of the bf16 value, which grow with the
+ * magnitude and add like logarithms.  codes = uint16[mi8_rowseg_code_count(rows, cols)], segment (r, c / 64) at
+ * index (c / 64) * rows + r.  mi8_rowseg_max_codes computes them for one tensor, or for the element-wise larger of
+ * two (b may be NULL); mi8_gemm_fp8_codes and mi8_gemm_fp8_swiglu write them for the tensors they produce.
+ *
+ * The sum of a segment's codes in gh and in (x1, x3) bounds log2 of both gradients on all its elements.
+ * mi8_swiglu_bwd_amax_from_codes computes exactly only the segments whose bound could still raise the maxima (all
+ * segments that may hold a non-finite input among them) and leaves state[0] = amax bits of g1, state[1] = of g3
+ * (float32 bit patterns, the values mi8_swiglu_bwd's partials reduce to; pass them to mi8_swiglu_bwd_cast with
+ * n_slots = 1); state is uint32[4], overwritten.  Tensors are bf16 [rows, cols] contiguous, cols % 8 == 0. */
+int64_t mi8_rowseg_code_count(int64_t rows, int64_t cols);
+int mi8_rowseg_max_codes(const void* a, const void* b, int64_t rows, int64_t cols, uint16_t* codes, void* stream);
+int mi8_swiglu_bwd_amax_from_codes(const void* x1, const void* x3, const void* gh, int64_t rows, int64_t cols,
+                                   const uint16_t* gh_codes, const uint16_t* x_codes, uint32_t* state, void* stream);
+/* out = mi8_gemm_fp8(a, b) for single scales and a bf16 output, with the row-segment codes of out written by the
+ * epilogue (the gradient reaching h = silu(x1) * x3, grad_h = grad_y W2 of src/olmo_core/nn/feed_forward.py:171, is
+ * produced this way).  mi8_gemm_fp8_codes_supported: shapes it takes (those mi8_gemm_fp8 runs on the same kernel, so
+ * out has the same bits; N % 64 == 0). */
+int mi8_gemm_fp8_codes_supported(int64_t M, int64_t N, int64_t K);
+int mi8_gemm_fp8_codes(const void* a, int a_dtype, int64_t lda, const void* b, int b_dtype, int64_t ldb, int64_t M, int64_t N,
+                       int64_t K, const float* sa, const float* sb, void* out, int64_t ldc, uint16_t* codes, void* stream);
 
 /* ---------------------------------------------------------------------------------------------
  * Token permutation around the expert GEMMs of a mixture-of-experts layer.  These replace the copy kernels of

@@ -69,7 +69,7 @@ _SIGNATURES = {
     "mi8_gemm_fp8_swiglu": (
         c_int,
         [c_void_p, c_int, c_int64, c_void_p, c_void_p, c_int, c_int64, c_int64, c_int64, c_int64, c_void_p, c_void_p,
-         c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_void_p, POINTER(c_int32), c_void_p],
+         c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_void_p, POINTER(c_int32), c_void_p, c_void_p],
     ),
     "mi8_gemm_fp8_splitk": (
         c_int,
@@ -89,6 +89,18 @@ _SIGNATURES = {
         c_int,
         [c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_void_p, c_void_p, c_int32, c_int, c_uint32, c_void_p, c_void_p,
          c_int64, c_void_p, c_void_p, c_int64, c_void_p, c_void_p, c_void_p],
+    ),
+    "mi8_rowseg_code_count": (c_int64, [c_int64, c_int64]),
+    "mi8_rowseg_max_codes": (c_int, [c_void_p, c_void_p, c_int64, c_int64, c_void_p, c_void_p]),
+    "mi8_swiglu_bwd_amax_from_codes": (
+        c_int,
+        [c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_void_p, c_void_p, c_void_p, c_void_p],
+    ),
+    "mi8_gemm_fp8_codes_supported": (c_int, [c_int64, c_int64, c_int64]),
+    "mi8_gemm_fp8_codes": (
+        c_int,
+        [c_void_p, c_int, c_int64, c_void_p, c_int, c_int64, c_int64, c_int64, c_int64, c_void_p, c_void_p, c_void_p,
+         c_int64, c_void_p, c_void_p],
     ),
     "mi8_moe_gather": (
         c_int,

@@ -20,7 +20,7 @@ CSRC = PKG_DIR / "csrc"
 LIB_PATH = PKG_DIR / "lib" / "libmi8.so"
 OBJ_DIR = PKG_DIR / "lib" / "obj"
 
-SOURCES = ["mi8_api.hip", "mi8_cast.hip", "mi8_gemm.hip", "mi8_gemm_m16.hip", "mi8_gemm_skinny.hip", "mi8_pointwise.hip", "mi8_grouped.hip", "mi8_permute.hip", "mi8_probe.hip"]
+SOURCES = ["mi8_api.hip", "mi8_cast.hip", "mi8_gemm.hip", "mi8_gemm_m16.hip", "mi8_gemm_skinny.hip", "mi8_pointwise.hip", "mi8_swiglu_amax.hip", "mi8_grouped.hip", "mi8_permute.hip", "mi8_probe.hip"]
 
 HIPCC_FLAGS = [
     "--offload-arch=gfx950",

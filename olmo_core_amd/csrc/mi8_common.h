@@ -64,6 +64,23 @@ __device__ __forceinline__ uint32_t wave_umax(uint32_t v)
     return v;
 }
 
+// The contiguous range [lo, hi) of n items that workgroup blockIdx.x of a 256-thread, one-dimensional-in-x grid
+// streams: ranges are multiples of 256 items (4 KB of 16-byte vectors), the last ones may be short or empty.
+// A workgroup that walks its own contiguous range keeps DRAM pages open; the same loads issued grid-stride
+// (every workgroup touching 4 KB every gridDim.x * 4 KB) reach 10-15 % less of the HBM bandwidth.
+struct BlockRange {
+    int64_t lo, hi;
+};
+__device__ __forceinline__ BlockRange block_range(int64_t n)
+{
+    const int64_t per = (((n + gridDim.x - 1) / gridDim.x) + 255) & ~(int64_t)255;
+    int64_t lo = (int64_t)blockIdx.x * per;
+    lo = lo < n ? lo : n;
+    int64_t hi = lo + per;
+    hi = hi < n ? hi : n;
+    return BlockRange{lo, hi};
+}
+
 // scale = float32(FP8_MAX * (1 / max(float64(amax), 1e-12))); NaN amax gives a NaN scale, +inf gives 0.
 // Optional round-down to a power of two clears the mantissa (scale is always a normal float or 0 here).
 template <int FP8>

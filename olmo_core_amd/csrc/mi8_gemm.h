@@ -92,10 +92,13 @@ __device__ __forceinline__ bool tile_of_block(const GemmArgs& g, int& tm, int& t
 // persistent direct-to-LDS kernel, four waves of 128 x 128 on 16x16x128 MFMAs (mi8_gemm_m16.hip); requires
 // M, N >= 256, K % 128 == 0, N % 8 == 0, ldc % 8 == 0, a 16-byte aligned bf16 output
 int launch_m16(GemmArgs& g, int a_dtype, int b_dtype, hipStream_t st);  // (honours g.accumulate)
+// the same with single scales, also recording the row-segment codes of C (uint16 [N / 64][M], N % 64 == 0)
+int launch_m16_codes(GemmArgs& g, uint16_t* codes, int a_dtype, int b_dtype, hipStream_t st);
 // the two input projections of a SwiGLU block and h = silu(x1) * x3 in one launch (g: A, B = B1, C = x1, N = H,
 // single scales sa, sb = scale of B1); writes 4 * workgroups partial maxima of |h| and their count
+// (x_codes: null, or uint16 [H / 64][M] row-segment codes of the larger of x1 and x3, H % 64 == 0)
 int launch_m16_swiglu(GemmArgs& g, const uint8_t* b3, const float* sb3, uint16_t* x3, uint16_t* h, uint32_t* h_slots,
-                      int* n_slots, int a_dtype, int b_dtype, hipStream_t st);
+                      int* n_slots, uint16_t* x_codes, int a_dtype, int b_dtype, hipStream_t st);
 // a few rows of A (M <= kSkinnyMaxM) against all of B, bound by reading B once (mi8_gemm_skinny.hip): any N,
 // K % 16 == 0, any mix of single scales and scale vectors, bf16 or fp32 output
 constexpr int kSkinnyMaxM = 64;

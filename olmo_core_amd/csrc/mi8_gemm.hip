@@ -279,7 +279,7 @@ extern "C" int mi8_gemm_fp8_swiglu_matches_separate(int64_t M, int64_t H, int64_
 extern "C" int mi8_gemm_fp8_swiglu(const void* a, int a_dtype, int64_t lda, const void* b1, const void* b3, int b_dtype,
                                    int64_t ldb, int64_t M, int64_t H, int64_t K, const float* sa, const float* sb1,
                                    const float* sb3, void* x1, void* x3, void* h, int64_t ldc, uint32_t* slots_h,
-                                   int32_t* n_slots_used, void* stream)
+                                   int32_t* n_slots_used, uint16_t* x_codes, void* stream)
 {
     MI8_REQUIRE(a && b1 && b3 && sa && sb1 && sb3 && x1 && x3 && h && slots_h && n_slots_used, MI8_ERR_ARG,
                 "mi8_gemm_fp8_swiglu: null pointer");
@@ -296,12 +296,44 @@ extern "C" int mi8_gemm_fp8_swiglu(const void* a, int a_dtype, int64_t lda, cons
     MI8_REQUIRE(M * lda < (int64_t)1 << 32 && H * ldb < (int64_t)1 << 32 && M < (1 << 30) && H < (1 << 30) &&
                     K < (1 << 30),
                 MI8_ERR_UNSUPPORTED, "mi8_gemm_fp8_swiglu: operand larger than 4 GiB");
+    MI8_REQUIRE(!x_codes || H % 64 == 0, MI8_ERR_UNSUPPORTED,
+                "mi8_gemm_fp8_swiglu: row-segment codes need H (%lld) to be a multiple of 64", (long long)H);
     GemmArgs g{(const uint8_t*)a, (const uint8_t*)b1, x1, 0, lda, ldb, ldc, (int)M, (int)H, (int)K, sa, sb1, 0, 0, 0, 0, 0};
     int used = 0;
-    const int rc = launch_m16_swiglu(g, (const uint8_t*)b3, sb3, (uint16_t*)x3, (uint16_t*)h, slots_h, &used, a_dtype,
-                                     b_dtype, (hipStream_t)stream);
+    const int rc = launch_m16_swiglu(g, (const uint8_t*)b3, sb3, (uint16_t*)x3, (uint16_t*)h, slots_h, &used, x_codes,
+                                     a_dtype, b_dtype, (hipStream_t)stream);
     *n_slots_used = used;
     return rc;
+}
+
+// 1 if mi8_gemm_fp8_codes takes the shape: the shapes mi8_gemm_fp8 runs on the persistent tile kernel (so that the
+// output has the bits of the plain call) whose row segments line up with the output tiles
+extern "C" int mi8_gemm_fp8_codes_supported(int64_t M, int64_t N, int64_t K)
+{
+    if (M < 256 || N < 256 || K <= 0 || K % 128 || N % 64) return 0;
+    const int64_t tiles256 = ((M + 255) / 256) * ((N + 255) / 256);
+    return tiles256 > 96 ? 1 : 0;
+}
+
+extern "C" int mi8_gemm_fp8_codes(const void* a, int a_dtype, int64_t lda, const void* b, int b_dtype, int64_t ldb, int64_t M,
+                                  int64_t N, int64_t K, const float* sa, const float* sb, void* out, int64_t ldc,
+                                  uint16_t* codes, void* stream)
+{
+    MI8_REQUIRE(a && b && sa && sb && out && codes, MI8_ERR_ARG, "mi8_gemm_fp8_codes: null pointer");
+    MI8_REQUIRE((a_dtype == MI8_E4M3 || a_dtype == MI8_E5M2) && (b_dtype == MI8_E4M3 || b_dtype == MI8_E5M2),
+                MI8_ERR_ARG, "mi8_gemm_fp8_codes: unknown fp8 dtype");
+    MI8_REQUIRE(mi8_gemm_fp8_codes_supported(M, N, K), MI8_ERR_UNSUPPORTED,
+                "mi8_gemm_fp8_codes: needs N %% 64 == 0, K %% 128 == 0 and more than 96 tiles of 256 x 256 (got %lld x %lld x "
+                "%lld); use mi8_gemm_fp8 and mi8_rowseg_max_codes",
+                (long long)M, (long long)N, (long long)K);
+    MI8_REQUIRE(lda % 16 == 0 && ldb % 16 == 0 && lda >= K && ldb >= K && ldc >= N && ldc % 8 == 0, MI8_ERR_UNSUPPORTED,
+                "mi8_gemm_fp8_codes: lda, ldb must be multiples of 16 and >= K, ldc a multiple of 8 and >= N");
+    MI8_REQUIRE(aligned16(a) && aligned16(b) && aligned16(out), MI8_ERR_UNSUPPORTED,
+                "mi8_gemm_fp8_codes: operands and output must be 16-byte aligned");
+    MI8_REQUIRE(M * lda < (int64_t)1 << 32 && N * ldb < (int64_t)1 << 32 && M < (1 << 30) && N < (1 << 30) && K < (1 << 30),
+                MI8_ERR_UNSUPPORTED, "mi8_gemm_fp8_codes: operand larger than 4 GiB");
+    GemmArgs g{(const uint8_t*)a, (const uint8_t*)b, out, 0, lda, ldb, ldc, (int)M, (int)N, (int)K, sa, sb, 0, 0, 0, 0, 0};
+    return launch_m16_codes(g, codes, a_dtype, b_dtype, (hipStream_t)stream);
 }
 
 extern "C" int mi8_gemm_splitk_suggest(int64_t M, int64_t N, int64_t K)

@@ -52,6 +52,17 @@ constexpr int kLoads = 8;                    // direct loads per operand, step a
 // (SQ_LDS_BANK_CONFLICT: half of the LDS cycles of the GEMM).
 __device__ __forceinline__ int swz16(int r) { return ((r >> 2) & 1) | (((r >> 1) & 1) << 2); }
 
+// Maximum over every aligned group of eight lanes, of two independent 16-bit halves per register, by DPP moves (no
+// LDS traffic: an LDS instruction the compiler knows of would make it wait for the direct-to-LDS loads in flight);
+// all eight lanes end up with the result.
+__device__ __forceinline__ uint32_t dpp_pk_umax16_over8(uint32_t v)
+{
+    v = pk_umax16(v, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0xB1, 0xF, 0xF, true));   // quad_perm [1,0,3,2]
+    v = pk_umax16(v, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x4E, 0xF, 0xF, true));   // quad_perm [2,3,0,1]
+    v = pk_umax16(v, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x141, 0xF, 0xF, true));  // row_half_mirror
+    return v;
+}
+
 template <typename Problem, int CBSZ_A, int BLGP_B>
 __global__ __launch_bounds__(kThreads, 1) void gemm_fp8_m16_kernel(Problem pb)
 {
@@ -272,11 +283,19 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_fp8_m16_kernel(Problem pb)
             }
             // All but this phase's eight loads have landed: the other stage (step + 1) is complete.  (The
             // compiler does not track direct-to-LDS loads across a barrier.)
-            // A tile's first step follows the previous tile's epilogue, whose 32 stores are younger than the loads
-            // waited for here (one in-order counter): they may stay outstanding as well.
-            if (fresh)
-                __builtin_amdgcn_s_waitcnt(Problem::kSwiglu ? 0xCF78 : 0x8F78);  // vmcnt(56) / vmcnt(40)
-            else
+            // A tile's first step follows the previous tile's epilogue, whose 32 stores (40 with row-segment codes, 48
+            // or 52 of the fused SwiGLU problem) are younger than the loads waited for here (one in-order counter):
+            // they may stay outstanding as well.
+            if (fresh) {
+                if constexpr (Problem::kSwiglu) {
+                    if (pb.x_codes)  // (uniform)
+                        __builtin_amdgcn_s_waitcnt(0xCF7C);  // vmcnt(60): 8 loads, 48 + 4 stores
+                    else
+                        __builtin_amdgcn_s_waitcnt(0xCF78);  // vmcnt(56)
+                } else {
+                    __builtin_amdgcn_s_waitcnt(Problem::kOutCodes ? 0xCF70 : 0x8F78);  // vmcnt(48) / vmcnt(40)
+                }
+            } else
                 __builtin_amdgcn_s_waitcnt(0x0F78);  // vmcnt(8)
             asm volatile("s_barrier" ::: "memory");
             flip_read_stage(cur ^ 1);
@@ -354,6 +373,33 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_fp8_m16_kernel(Problem pb)
         auto add_held = [&]() __attribute__((always_inline)) {
 #pragma unroll
             for (int it = 0; it < 4; ++it) staged[it] = add_bf16x8(staged[it], held[it]);
+        };
+        // Row-segment codes (kOutCodes, and the x codes of the fused SwiGLU problem): a pass holds 32 row segments of
+        // 64 columns, eight lanes each (staged[it]: row 8 it + lane / 8).  A lane's eight values give one code per
+        // row; a DPP butterfly over the eight lanes leaves the segment's code in all of them; lane j < 4 of every
+        // group of eight then stores the code of row 8 j + lane / 8, so the pass writes its 32 codes (64 contiguous
+        // bytes) with one store instruction.
+        const int code_lane = (lane & 7) * 8 + (lane >> 3);
+        auto lane_codes = [&](uint32_t& c01, uint32_t& c23) __attribute__((always_inline)) {
+            c01 = (max_code8((uint32_t)staged[0][0], (uint32_t)staged[0][1], (uint32_t)staged[0][2], (uint32_t)staged[0][3]) & 0xFFFFu) |
+                  (max_code8((uint32_t)staged[1][0], (uint32_t)staged[1][1], (uint32_t)staged[1][2], (uint32_t)staged[1][3]) & 0xFFFF0000u);
+            c23 = (max_code8((uint32_t)staged[2][0], (uint32_t)staged[2][1], (uint32_t)staged[2][2], (uint32_t)staged[2][3]) & 0xFFFFu) |
+                  (max_code8((uint32_t)staged[3][0], (uint32_t)staged[3][1], (uint32_t)staged[3][2], (uint32_t)staged[3][3]) & 0xFFFF0000u);
+        };
+        auto store_codes = [&](uint16_t* codes, int64_t rows_total, int col_block, int ih, uint32_t c01, uint32_t c23)
+                               __attribute__((always_inline)) {
+            c01 = dpp_pk_umax16_over8(c01);
+            c23 = dpp_pk_umax16_over8(c23);
+            const uint32_t w = (lane & 2) ? c23 : c01;
+            const uint16_t code = (uint16_t)((lane & 1) ? (w >> 16) : (w & 0xFFFFu));
+            if ((lane & 7) < 4) codes[(int64_t)col_block * rows_total + td.m0 + wm * WT + ih * 32 + code_lane] = code;
+        };
+        auto record_codes = [&](int p) __attribute__((always_inline)) {  // p = 4 * jq + ih: the pass whose rows are staged
+            if constexpr (Problem::kOutCodes) {
+                uint32_t c01, c23;
+                lane_codes(c01, c23);
+                store_codes(pb.codes, pb.g.M, td.n0 / 64 + wn * 2 + (p >> 2), p & 3, c01, c23);
+            }
         };
         auto store_staged = [&](int jq, int ih) __attribute__((always_inline)) {
             const int rt = wm * WT + ih * 32;  // first tile row of the pass
@@ -445,6 +491,8 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_fp8_m16_kernel(Problem pb)
                 uint2 o1[2][4], o3[2][4], oh[2][4];
                 scaled(o1, ih, 0, aux[0]);
                 stage(o1, ih == 0 ? -1 : 2, ih - 1);
+                uint32_t cx01 = 0, cx23 = 0;  // codes of the x1 rows now staged
+                if (pb.x_codes) lane_codes(cx01, cx23);
                 scaled(o3, ih, 4, aux[1]);
 #pragma unroll
                 for (int t = 0; t < 2; ++t)
@@ -457,6 +505,11 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_fp8_m16_kernel(Problem pb)
                         hmax = umax32(hmax, oh[t][jj].y & 0x7FFF0000u);
                     }
                 stage(o3, 0, ih);
+                if (pb.x_codes) {  // (uniform) the x3 rows are staged: the larger of the two codes per row segment
+                    uint32_t c01, c23;
+                    lane_codes(c01, c23);
+                    store_codes(pb.x_codes, pb.g.M, td.n0 / 64 + wn, ih, pk_umax16(c01, cx01), pk_umax16(c23, cx23));
+                }
                 stage(oh, 1, ih);
             }
             __builtin_amdgcn_s_waitcnt(0xc07f);
@@ -517,6 +570,7 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_fp8_m16_kernel(Problem pb)
                     // the previous pass's rows have arrived in registers (so its staging area is free again)
                     __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0)
                     if constexpr (Problem::kAccumulate) add_held();
+                    record_codes(4 * jq + ih - 1);
                 }
                 // (this pass's old C values are requested before the previous pass's stores are issued: the wait for
                 // them, one pass later, then leaves those stores outstanding)
@@ -547,6 +601,7 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_fp8_m16_kernel(Problem pb)
         }
         __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0)
         if constexpr (Problem::kAccumulate) add_held();
+        record_codes(7);
         store_staged(1, 3);
         }
         // The last step's phase B has read the next tile's first fragments like any other step; reading them
@@ -609,13 +664,22 @@ int launch_m16(GemmArgs& g, int a_dtype, int b_dtype, hipStream_t st)
     return launch_typed(DenseProblem<false>{g, g.lda, g.ldb, g.ldc}, tiles, true, a_dtype, b_dtype, st);
 }
 
+int launch_m16_codes(GemmArgs& g, uint16_t* codes, int a_dtype, int b_dtype, hipStream_t st)
+{
+    g.tiles_m = (g.M + BM - 1) / BM;
+    g.tiles_n = (g.N + BN - 1) / BN;
+    DenseProblem<false, false, true> pb{g, g.lda, g.ldb, g.ldc};
+    pb.codes = codes;
+    return launch_typed(pb, g.tiles_m * g.tiles_n, true, a_dtype, b_dtype, st);
+}
+
 int launch_m16_swiglu(GemmArgs& g, const uint8_t* b3, const float* sb3, uint16_t* x3, uint16_t* h, uint32_t* h_slots,
-                      int* n_slots, int a_dtype, int b_dtype, hipStream_t st)
+                      int* n_slots, uint16_t* x_codes, int a_dtype, int b_dtype, hipStream_t st)
 {
     g.tiles_m = (g.M + BM - 1) / BM;
     g.tiles_n = (g.N + 127) / 128;
     SwigluProblem pb{g, g.lda, g.ldb, g.ldc, (int64_t)(b3 - g.B), (int64_t)(x3 - reinterpret_cast<uint16_t*>(g.C)),
-                     (int64_t)(h - reinterpret_cast<uint16_t*>(g.C)), sb3, h_slots};
+                     (int64_t)(h - reinterpret_cast<uint16_t*>(g.C)), sb3, h_slots, x_codes};
     const int tiles = g.tiles_m * g.tiles_n;
     int blocks = num_compute_units();
     const int wanted = (tiles + 7) / 8 * 8;

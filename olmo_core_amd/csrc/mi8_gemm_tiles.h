@@ -20,18 +20,24 @@ struct TileDesc {
     const float* sb;   // scale of the tile's first column (or the single scale)
     uint16_t* c;       // C element (first row, first column) of the tile; null: the slot holds no tile
     int row_lo, row_hi;  // rows [row_lo, row_hi) of the 256 are stored
+    int m0, n0;          // (problems that record row-segment codes) first row and column of the tile
 };
 
 struct NoCache {};
 
 // Dense problem: C[M, N] = A[M, K] . B[N, K]^T.  The last tile row / column is shifted back so that every tile
 // is full (M, N >= 256): the overlap is recomputed with the same K order and rewritten with identical values.
-template <bool VEC, bool ACC = false>
+// CODES: the epilogue also records, per row segment (64 consecutive columns of a row) of C, the largest magnitude it
+// wrote as a 16-bit code (mi8_swiglu.h; codes[(column / 64) * M + row], N % 64 == 0: shifted tiles then start on
+// segment boundaries).
+template <bool VEC, bool ACC = false, bool CODES = false>
 struct DenseProblem {
     GemmArgs g;
     int64_t lda, ldb, ldc;
+    uint16_t* codes = nullptr;  // (CODES)
     static constexpr bool kVecScales = VEC;  // both scales are vectors (per row / per column) or both single
     static constexpr bool kAccumulate = ACC;  // C += the rounded product
+    static constexpr bool kOutCodes = CODES;
     static constexpr bool kSwiglu = false;
     static constexpr bool kMaskRows = false, kXcdRanges = true, kPeelFirstStep = true;
     using Cache = NoCache;
@@ -55,6 +61,8 @@ struct DenseProblem {
         d.c = reinterpret_cast<uint16_t*>(g.C) + (int64_t)m0 * g.ldc + n0;
         d.row_lo = 0;
         d.row_hi = BM;
+        d.m0 = m0;
+        d.n0 = n0;
         return d;
     }
 };
@@ -72,7 +80,8 @@ struct SwigluProblem {
     int64_t h_offset;
     const float* sb3;       // scale of B3
     uint32_t* h_slots;      // [4 * workgroups] partial maxima of |h| (float32 bit patterns)
-    static constexpr bool kVecScales = false, kAccumulate = false, kSwiglu = true;
+    uint16_t* x_codes;      // null, or [H / 64][M] codes of the larger of x1 and x3 per row segment (H % 64 == 0)
+    static constexpr bool kVecScales = false, kAccumulate = false, kSwiglu = true, kOutCodes = false;
     static constexpr bool kMaskRows = false, kXcdRanges = true, kPeelFirstStep = true;
     using Cache = NoCache;
     __device__ __forceinline__ Cache prepare() const { return Cache{}; }
@@ -94,6 +103,8 @@ struct SwigluProblem {
         d.c = reinterpret_cast<uint16_t*>(g.C) + (int64_t)m0 * g.ldc + n0;
         d.row_lo = 0;
         d.row_hi = BM;
+        d.m0 = m0;
+        d.n0 = n0;
         return d;
     }
 };
@@ -154,7 +165,7 @@ __device__ __forceinline__ GroupSpan locate_group_cached(const GroupCache& c, co
 template <bool ACC = false>
 struct GroupedProblem {
     static constexpr bool kAccumulate = ACC;
-    static constexpr bool kSwiglu = false;
+    static constexpr bool kSwiglu = false, kOutCodes = false;
     const uint8_t* A;
     const uint8_t* B;
     uint16_t* C;
@@ -225,7 +236,7 @@ struct GroupedWgradProblem {
     const float* sa;  // [E, N]
     const float* sb;  // [E, Kl]
     static constexpr bool kVecScales = true, kMaskRows = false, kXcdRanges = false, kPeelFirstStep = true;
-    static constexpr bool kAccumulate = false, kSwiglu = false;
+    static constexpr bool kAccumulate = false, kSwiglu = false, kOutCodes = false;
     using Cache = WgradCache;
     __device__ __forceinline__ Cache prepare() const
     {

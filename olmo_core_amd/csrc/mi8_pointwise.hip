@@ -36,8 +36,17 @@ __global__ __launch_bounds__(kThreads) void swiglu_fwd_kernel(const uint4* __res
                                                               int64_t nvec, uint32_t* __restrict__ slots)
 {
     uint32_t m = 0;
-    const int64_t stride = (int64_t)gridDim.x * kThreads;
-    for (int64_t i = (int64_t)blockIdx.x * kThreads + threadIdx.x; i < nvec; i += stride) {
+    // every workgroup streams its own contiguous range, two vectors per lane in flight
+    const BlockRange r = block_range(nvec);
+    int64_t i = r.lo + threadIdx.x;
+    for (; i + kThreads < r.hi; i += 2 * kThreads) {
+        const uint4 a0 = x1[i], b0 = x3[i], a1 = x1[i + kThreads], b1 = x3[i + kThreads];
+        const uint4 o0 = swiglu_fwd8(a0, b0), o1 = swiglu_fwd8(a1, b1);
+        h[i] = o0;
+        h[i + kThreads] = o1;
+        m = umax32(m, umax32(absmax_packed(o0), absmax_packed(o1)));
+    }
+    for (; i < r.hi; i += kThreads) {
         const uint4 out = swiglu_fwd8(x1[i], x3[i]);
         h[i] = out;
         m = umax32(m, absmax_packed(out));
@@ -53,11 +62,28 @@ __global__ __launch_bounds__(kThreads) void swiglu_bwd_kernel(const uint4* __res
                                                               uint32_t* __restrict__ slots3)
 {
     uint32_t m1 = 0, m3 = 0;
-    const int64_t stride = (int64_t)gridDim.x * kThreads;
-    for (int64_t i = (int64_t)blockIdx.x * kThreads + threadIdx.x; i < nvec; i += stride) {
+    // every workgroup streams its own contiguous range, two vectors of each input per lane in flight
+    const BlockRange r = block_range(nvec);
+    int64_t i = r.lo + threadIdx.x;
+    for (; i + kThreads < r.hi; i += 2 * kThreads) {
+        const uint4 a0 = x1[i], b0 = x3[i], c0 = gh[i];
+        const uint4 a1 = x1[i + kThreads], b1 = x3[i + kThreads], c1 = gh[i + kThreads];
+        uint4 p1, p3, q1, q3;
+        swiglu_bwd8(a0, b0, c0, p1, p3);
+        swiglu_bwd8(a1, b1, c1, q1, q3);
+        if (g1) {  // (without outputs: only the amax of what would be written)
+            g1[i] = p1;
+            g3[i] = p3;
+            g1[i + kThreads] = q1;
+            g3[i + kThreads] = q3;
+        }
+        m1 = umax32(m1, umax32(absmax_packed(p1), absmax_packed(q1)));
+        m3 = umax32(m3, umax32(absmax_packed(p3), absmax_packed(q3)));
+    }
+    for (; i < r.hi; i += kThreads) {
         uint4 p1, p3;
         swiglu_bwd8(x1[i], x3[i], gh[i], p1, p3);
-        if (g1) {  // (without outputs: only the amax of what would be written)
+        if (g1) {
             g1[i] = p1;
             g3[i] = p3;
         }

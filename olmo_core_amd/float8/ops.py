@@ -319,11 +319,13 @@ def swiglu_gemm_matches_separate(M: int, H: int, K: int) -> bool:
 
 
 def gemm_fp8_swiglu(a: torch.Tensor, sa: torch.Tensor, b1: torch.Tensor, sb1: torch.Tensor, b3: torch.Tensor,
-                    sb3: torch.Tensor, *, k: Optional[int] = None):
+                    sb3: torch.Tensor, *, k: Optional[int] = None, want_codes: bool = False):
     """
     ``x1 = a @ b1.T``, ``x3 = a @ b3.T`` (scaled, bf16) and ``h = silu(x1) * x3`` from one launch, with the amax
     partials of ``h``: ``(x1, x3, h, (slots, n_slots))``, each bit-identical to :func:`gemm_fp8` / :func:`swiglu_fwd`.
-    Single scales only (the tensorwise recipe).
+    Single scales only (the tensorwise recipe).  ``want_codes`` (H % 64 == 0): a fifth result, the row-segment codes
+    of the larger of ``x1`` and ``x3`` (:func:`rowseg_max_codes`), which the backward pass's
+    :func:`swiglu_bwd_cast` takes.
     """
     _require_gpu(a, "gemm_fp8_swiglu")
     if a.dim() != 2 or b1.dim() != 2 or b1.shape != b3.shape or b1.dtype != b3.dtype or b1.stride(0) != b3.stride(0):
@@ -339,6 +341,7 @@ def gemm_fp8_swiglu(a: torch.Tensor, sa: torch.Tensor, b1: torch.Tensor, sb1: to
     x1, x3, h = (torch.empty((M, H), dtype=torch.bfloat16, device=a.device) for _ in range(3))
     slots = torch.empty(_C.AMAX_SLOTS, dtype=torch.int32, device=a.device)
     used = _C.c_int32(0)
+    codes = torch.empty(_C.lib().mi8_rowseg_code_count(M, H), dtype=torch.int16, device=a.device) if want_codes else None
     sink = GEMM_EVENT_SINK
     if sink is not None:
         ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
@@ -347,14 +350,54 @@ def gemm_fp8_swiglu(a: torch.Tensor, sa: torch.Tensor, b1: torch.Tensor, sb1: to
         _C.lib().mi8_gemm_fp8_swiglu(
             a.data_ptr(), _FP8_CODE[a.dtype], a.stride(0), b1.data_ptr(), b3.data_ptr(), _FP8_CODE[b1.dtype],
             b1.stride(0), M, H, K, sa.data_ptr(), sb1.data_ptr(), sb3.data_ptr(), x1.data_ptr(), x3.data_ptr(),
-            h.data_ptr(), H, slots.data_ptr(), used, _stream(a),
+            h.data_ptr(), H, slots.data_ptr(), used, codes.data_ptr() if want_codes else None, _stream(a),
         ),
         "mi8_gemm_fp8_swiglu",
     )
     if sink is not None:
         ev1.record()
         sink.append((ev0, ev1, (M, 2 * H, K)))
+    if want_codes:
+        return x1, x3, h, (slots, used.value), codes
     return x1, x3, h, (slots, used.value)
+
+
+def gemm_codes_supported(M: int, N: int, K: int) -> bool:
+    """Shapes :func:`gemm_fp8_codes` takes (the result then has the bits of :func:`gemm_fp8`)."""
+    return bool(_C.lib().mi8_gemm_fp8_codes_supported(M, N, K))
+
+
+def gemm_fp8_codes(a: torch.Tensor, sa: torch.Tensor, b: torch.Tensor, sb: torch.Tensor, *, k: Optional[int] = None):
+    """
+    ``out = gemm_fp8(a, sa, b, sb)`` (single scales, bf16) together with the row-segment codes of ``out``
+    (:func:`rowseg_max_codes`), written by the GEMM's epilogue.  Returns ``(out, codes)``.
+    """
+    _require_gpu(a, "gemm_fp8_codes")
+    if a.dim() != 2 or b.dim() != 2 or a.stride(1) != 1 or b.stride(1) != 1:
+        raise ValueError("gemm_fp8_codes: operands must be 2-D with contiguous rows")
+    if a.dtype not in _FP8_CODE or b.dtype not in _FP8_CODE:
+        raise TypeError("gemm_fp8_codes: operands must be float8")
+    if sa.numel() != 1 or sb.numel() != 1:
+        raise ValueError("gemm_fp8_codes: single scales only")
+    M, N = a.shape[0], b.shape[0]
+    K = min(a.shape[1], b.shape[1]) if k is None else k
+    out = torch.empty((M, N), dtype=torch.bfloat16, device=a.device)
+    codes = torch.empty(_C.lib().mi8_rowseg_code_count(M, N), dtype=torch.int16, device=a.device)
+    sink = GEMM_EVENT_SINK
+    if sink is not None:
+        ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        ev0.record()
+    _C.check(
+        _C.lib().mi8_gemm_fp8_codes(
+            a.data_ptr(), _FP8_CODE[a.dtype], a.stride(0), b.data_ptr(), _FP8_CODE[b.dtype], b.stride(0), M, N, K,
+            sa.data_ptr(), sb.data_ptr(), out.data_ptr(), N, codes.data_ptr(), _stream(a),
+        ),
+        "mi8_gemm_fp8_codes",
+    )
+    if sink is not None:
+        ev1.record()
+        sink.append((ev0, ev1, (M, N, K)))
+    return out, codes
 
 
 def gemm_variants() -> list:
@@ -399,14 +442,55 @@ def swiglu_bwd(x1: torch.Tensor, x3: torch.Tensor, gh: torch.Tensor, want_amax: 
     return g1, g3, ((s1, used) if want_amax else None), ((s3, used) if want_amax else None)
 
 
+def rowseg_max_codes(a: torch.Tensor, b: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """One 16-bit code per row segment (64 consecutive columns of a row) of a bf16 matrix: the largest magnitude in
+    it (of ``a``, or of ``a`` and ``b``), as the integer formed by the exponent and mantissa bits; int16
+    ``[ceil(cols / 64) * rows]``, the codes of one column block contiguous over the rows."""
+    _require_gpu(a, "rowseg_max_codes")
+    if a.dtype != torch.bfloat16 or a.dim() != 2 or (b is not None and (b.dtype != a.dtype or b.shape != a.shape)):
+        raise ValueError("rowseg_max_codes expects one or two bfloat16 matrices of one shape")
+    a = a.contiguous()
+    b = b.contiguous() if b is not None else None
+    rows, cols = a.shape
+    codes = torch.empty(_C.lib().mi8_rowseg_code_count(rows, cols), dtype=torch.int16, device=a.device)
+    _C.check(
+        _C.lib().mi8_rowseg_max_codes(a.data_ptr(), b.data_ptr() if b is not None else None, rows, cols, codes.data_ptr(),
+                                      _stream(a)),
+        "mi8_rowseg_max_codes",
+    )
+    return codes
+
+
+def swiglu_bwd_amax_from_codes(x1: torch.Tensor, x3: torch.Tensor, gh: torch.Tensor, gh_codes: torch.Tensor,
+                               x_codes: torch.Tensor) -> torch.Tensor:
+    """The amax of g1 and g3 (float32 bit patterns in words 0 and 1 of the returned int32[4]), computing only the
+    row segments whose codes say they could raise it; equal to the maxima of :func:`swiglu_bwd`'s partials."""
+    _require_gpu(x1, "swiglu_bwd_amax_from_codes")
+    rows, cols = x1.shape
+    n = _C.lib().mi8_rowseg_code_count(rows, cols)
+    for c in (gh_codes, x_codes):
+        if c.dtype != torch.int16 or c.numel() != n or not c.is_contiguous() or c.device != x1.device:
+            raise ValueError("swiglu_bwd_amax_from_codes: codes must be the int16 arrays of rowseg_max_codes for this shape")
+    state = torch.empty(4, dtype=torch.int32, device=x1.device)
+    _C.check(
+        _C.lib().mi8_swiglu_bwd_amax_from_codes(x1.data_ptr(), x3.data_ptr(), gh.data_ptr(), rows, cols, gh_codes.data_ptr(),
+                                                x_codes.data_ptr(), state.data_ptr(), _stream(x1)),
+        "mi8_swiglu_bwd_amax_from_codes",
+    )
+    return state
+
+
 def swiglu_bwd_cast(
     x1: torch.Tensor, x3: torch.Tensor, gh: torch.Tensor, fp8_dtype: torch.dtype, *, pow2: bool = False,
-    want_rowmajor: bool = True, want_transposed: bool = False,
+    want_rowmajor: bool = True, want_transposed: bool = False, codes: Optional[tuple] = None,
 ):
     """
     ``swiglu_bwd`` followed by ``cast_tensorwise`` of both gradients, without ever writing them in bf16: a first
     pass takes only their amax, a second recomputes them tile by tile and writes the fp8 copies.  Returns
     ``(g1q, g1q_t, scale1, g3q, g3q_t, scale3)`` with the bytes and scales of the two-step route.
+    ``codes`` = ``(gh_codes, x_codes)`` (from :func:`gemm_fp8_codes` / :func:`gemm_fp8_swiglu`, or
+    :func:`rowseg_max_codes`): the amax is then found by computing only the row segments that can hold it, instead
+    of by the pass over all three tensors.
     """
     _require_gpu(x1, "swiglu_bwd_cast")
     if not (x1.dtype == x3.dtype == gh.dtype == torch.bfloat16) or not (x1.shape == x3.shape == gh.shape) or x1.dim() != 2:
@@ -417,14 +501,18 @@ def swiglu_bwd_cast(
     rows, cols = x1.shape
     dev = x1.device
     n = x1.numel()
-    s1 = torch.empty(_C.AMAX_SLOTS, dtype=torch.int32, device=dev)
-    s3 = torch.empty(_C.AMAX_SLOTS, dtype=torch.int32, device=dev)
-    _C.check(
-        _C.lib().mi8_swiglu_bwd(x1.data_ptr(), x3.data_ptr(), gh.data_ptr(), None, None, n, s1.data_ptr(), s3.data_ptr(),
-                                _stream(x1)),
-        "mi8_swiglu_bwd",
-    )
-    used = _C.lib().mi8_amax_slots_for(n)
+    if codes is not None:
+        state = swiglu_bwd_amax_from_codes(x1, x3, gh, codes[0], codes[1])
+        s1, s3, used = state[0:1], state[1:2], 1
+    else:
+        s1 = torch.empty(_C.AMAX_SLOTS, dtype=torch.int32, device=dev)
+        s3 = torch.empty(_C.AMAX_SLOTS, dtype=torch.int32, device=dev)
+        _C.check(
+            _C.lib().mi8_swiglu_bwd(x1.data_ptr(), x3.data_ptr(), gh.data_ptr(), None, None, n, s1.data_ptr(), s3.data_ptr(),
+                                    _stream(x1)),
+            "mi8_swiglu_bwd",
+        )
+        used = _C.lib().mi8_amax_slots_for(n)
     q = [_operand((rows, cols), fp8_dtype, dev) if want_rowmajor else None for _ in range(2)]
     q_t = [_operand((cols, pad16(rows)), fp8_dtype, dev) if want_transposed else None for _ in range(2)]
     scales = [torch.empty(1, dtype=torch.float32, device=dev) for _ in range(2)]

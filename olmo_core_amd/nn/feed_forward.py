@@ -29,6 +29,11 @@ STAGE_SINK = None
 # three separate launches); a switch so that the two routes can be compared.
 FUSE_SWIGLU_EPILOGUE = True
 
+# Take the amax of the two gate gradients from the row-segment codes that the fused forward launch and the GEMM that
+# produces grad_h record (same bits as the pass over gh, x1 and x3 it replaces); a switch so that the two routes can be
+# compared.
+SWIGLU_AMAX_FROM_CODES = True
+
 
 class _SwiGLU(torch.autograd.Function):
     @staticmethod
@@ -64,6 +69,7 @@ class _Float8SwiGLUMLP(torch.autograd.Function):
         )
         need = ctx.needs_input_grad
         any_grad = any(need[:4])
+        x_codes = None
         xq, xq_t, sx = ops.cast_tensorwise(x, in_dt, pow2=pow2, want_transposed=need[1] or need[3])
         # ws*: weight scales precomputed after the optimizer step (None: reduce the amax here);
         # wo*: float8 copies the modules keep between calls (None: quantise the weight here)
@@ -72,7 +78,10 @@ class _Float8SwiGLUMLP(torch.autograd.Function):
         w2q, w2q_t, s2 = wo2 or ops.cast_tensorwise(w2, w_dt, pow2=pow2, want_transposed=any_grad, scale=ws2)
         if FUSE_SWIGLU_EPILOGUE and x.dtype == torch.bfloat16 and ops.swiglu_gemm_matches_separate(x.shape[0], w1.shape[0], x.shape[1]):
             # both input projections and the activation in one launch: x1 and x3 are never read back
-            x1, x3, h, h_slots = ops.gemm_fp8_swiglu(xq, sx, w1q, s1, w3q, s3)
+            if any_grad and SWIGLU_AMAX_FROM_CODES and w1.shape[0] % 64 == 0:
+                x1, x3, h, h_slots, x_codes = ops.gemm_fp8_swiglu(xq, sx, w1q, s1, w3q, s3, want_codes=True)
+            else:
+                x1, x3, h, h_slots = ops.gemm_fp8_swiglu(xq, sx, w1q, s1, w3q, s3)
         else:
             x1 = ops.gemm_fp8(xq, sx, w1q, s1, out_dtype=x.dtype)
             x3 = ops.gemm_fp8(xq, sx, w3q, s3, out_dtype=x.dtype)
@@ -88,13 +97,13 @@ class _Float8SwiGLUMLP(torch.autograd.Function):
         ctx.save_for_backward(
             xq_t if xq_t is not None else none, sx, x1, x3, hq_t if hq_t is not None else none, sh,
             w1q_t if w1q_t is not None else none, s1, w2q_t if w2q_t is not None else none, s2,
-            w3q_t if w3q_t is not None else none, s3,
+            w3q_t if w3q_t is not None else none, s3, x_codes if x_codes is not None else none,
         )
         return y
 
     @staticmethod
     def backward(ctx, gy):
-        xq_t, sx, x1, x3, hq_t, sh, w1q_t, s1, w2q_t, s2, w3q_t, s3 = ctx.saved_tensors
+        xq_t, sx, x1, x3, hq_t, sh, w1q_t, s1, w2q_t, s2, w3q_t, s3, x_codes = ctx.saved_tensors
         c = ctx.config
         pow2 = c.round_scales_to_power_of_2
         x_dt, w1_dt, w2_dt, w3_dt, go_dt = ctx.dtypes
@@ -108,13 +117,21 @@ class _Float8SwiGLUMLP(torch.autograd.Function):
         gw2 = ops.gemm_fp8(gyq_t, sgy, hq_t, sh, out_dtype=x_dt) if need_w2 else None
         gx = gw1 = gw3 = None
         if need_gh:
-            gh = ops.gemm_fp8(gyq, sgy, w2q_t, s2, k=D, out_dtype=x_dt)
+            # g1 and g3 are needed in fp8 only, and their tensorwise scales need the amax of both first.  Where the
+            # forward recorded the row-segment codes of x1 and x3, the GEMM that produces gh records those of gh, and the
+            # amax follows by computing a small share of the segments; otherwise a pass over the three tensors takes it.
+            codes = None
+            if x_codes.numel() and x_dt == torch.bfloat16 and ops.gemm_codes_supported(M, H, D):
+                gh, gh_codes = ops.gemm_fp8_codes(gyq, sgy, w2q_t, s2, k=D)
+                codes = (gh_codes, x_codes)
+            else:
+                gh = ops.gemm_fp8(gyq, sgy, w2q_t, s2, k=D, out_dtype=x_dt)
             if STAGE_SINK is not None:
                 STAGE_SINK.update(gh=gh.clone())
             need_t = need_w1 or need_w3
-            # g1 and g3 are needed in fp8 only: amax pass, then recompute-and-cast pass (no bf16 round trip)
+            # then the recompute-and-cast pass (no bf16 round trip of g1, g3)
             g1q, g1q_t, sg1, g3q, g3q_t, sg3 = ops.swiglu_bwd_cast(
-                x1, x3, gh, go_dt, pow2=pow2, want_rowmajor=need_x, want_transposed=need_t)
+                x1, x3, gh, go_dt, pow2=pow2, want_rowmajor=need_x, want_transposed=need_t, codes=codes)
             del gh
             if need_x:
                 # the sum of the two halves as autograd forms it (two bf16 tensors added), by the second GEMM's epilogue
