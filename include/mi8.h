@@ -303,8 +303,10 @@ int mi8_swiglu_bwd_cast(const void* x1, const void* x3, const void* gh, int64_t 
  * mi8_swiglu_bwd_amax_from_codes computes exactly only the segments whose bound could still raise the maxima (all
  * segments that may hold a non-finite input among them) and leaves state[0] = amax bits of g1, state[1] = of g3
  * (float32 bit patterns, the values mi8_swiglu_bwd's partials reduce to; pass them to mi8_swiglu_bwd_cast with
- * n_slots = 1); state is uint32[4], overwritten.  Tensors are bf16 [rows, cols] contiguous, cols % 8 == 0. */
+ * n_slots = 1); state is uint32[mi8_swiglu_amax_state_words(rows, cols)], overwritten (nothing to clear beforehand).
+ * Tensors are bf16 [rows, cols] contiguous, cols % 8 == 0; the code arrays 16-byte aligned. */
 int64_t mi8_rowseg_code_count(int64_t rows, int64_t cols);
+int64_t mi8_swiglu_amax_state_words(int64_t rows, int64_t cols);
 int mi8_rowseg_max_codes(const void* a, const void* b, int64_t rows, int64_t cols, uint16_t* codes, void* stream);
 int mi8_swiglu_bwd_amax_from_codes(const void* x1, const void* x3, const void* gh, int64_t rows, int64_t cols,
                                    const uint16_t* gh_codes, const uint16_t* x_codes, uint32_t* state, void* stream);

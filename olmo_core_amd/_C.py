@@ -91,6 +91,7 @@ _SIGNATURES = {
          c_int64, c_void_p, c_void_p, c_int64, c_void_p, c_void_p, c_void_p],
     ),
     "mi8_rowseg_code_count": (c_int64, [c_int64, c_int64]),
+    "mi8_swiglu_amax_state_words": (c_int64, [c_int64, c_int64]),
     "mi8_rowseg_max_codes": (c_int, [c_void_p, c_void_p, c_int64, c_int64, c_void_p, c_void_p]),
     "mi8_swiglu_bwd_amax_from_codes": (
         c_int,

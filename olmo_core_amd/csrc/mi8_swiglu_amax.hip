@@ -56,34 +56,60 @@ __global__ __launch_bounds__(kThreads) void rowseg_codes_kernel(const uint16_t* 
 }
 
 // ---- the largest sum ------------------------------------------------------------------------------------------------
-// state: [0] amax bits of g1, [1] of g3, [2] largest sum of codes, [3] unused
-__global__ void swiglu_amax_init_kernel(uint32_t* state)
+// Every lane of the scans below takes eight consecutive segments (one 16-byte load per code array), every wave 512.
+// state: [0] amax bits of g1, [1] of g3, [2] n = workgroups per launch, [4 .. 4 + n) one partial maximum of the sums per
+// workgroup of the first scan, then n partial maxima of g1 and n of g3 from the seeds (no atomics there, nothing to
+// clear beforehand: the first scan's first workgroup zeroes [0] and [1]).
+constexpr int kSegsPerLane = 8, kSegsPerWave = 64 * kSegsPerLane, kSegsPerBlock = (kThreads / 64) * kSegsPerWave;
+constexpr int kStateHeader = 4;
+
+// the eight sums of a lane (zero beyond the end of the arrays)
+__device__ __forceinline__ void load_sums(const uint16_t* __restrict__ gc, const uint16_t* __restrict__ xc, int64_t first,
+                                          int64_t nseg, uint32_t (&s)[kSegsPerLane])
 {
-    if (threadIdx.x < 4) state[threadIdx.x] = 0;
+    if (first + kSegsPerLane <= nseg) {
+        const uint4 g = *reinterpret_cast<const uint4*>(gc + first), x = *reinterpret_cast<const uint4*>(xc + first);
+        const uint32_t gw[4] = {g.x, g.y, g.z, g.w}, xw[4] = {x.x, x.y, x.z, x.w};
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            s[2 * k] = (gw[k] & 0xFFFFu) + (xw[k] & 0xFFFFu);
+            s[2 * k + 1] = (gw[k] >> 16) + (xw[k] >> 16);
+        }
+    } else {
+#pragma unroll
+        for (int k = 0; k < kSegsPerLane; ++k) s[k] = first + k < nseg ? (uint32_t)gc[first + k] + (uint32_t)xc[first + k] : 0u;
+    }
 }
 
 __global__ __launch_bounds__(kThreads) void swiglu_max_sum_kernel(const uint16_t* __restrict__ gc, const uint16_t* __restrict__ xc,
                                                                   int64_t nseg, uint32_t* __restrict__ state)
 {
-    uint32_t m = 0;
-    for (int64_t i = (int64_t)blockIdx.x * kThreads + threadIdx.x; i < nseg; i += (int64_t)gridDim.x * kThreads)
-        m = umax32(m, (uint32_t)gc[i] + (uint32_t)xc[i]);
     __shared__ uint32_t smem[kThreads / 64];
+    uint32_t s[kSegsPerLane];
+    load_sums(gc, xc, ((int64_t)blockIdx.x * kThreads + threadIdx.x) * kSegsPerLane, nseg, s);
+    uint32_t m = 0;
+#pragma unroll
+    for (int k = 0; k < kSegsPerLane; ++k) m = umax32(m, s[k]);
     m = wave_umax(m);
     if ((threadIdx.x & 63) == 0) smem[threadIdx.x >> 6] = m;
     __syncthreads();
     if (threadIdx.x == 0) {
-        m = umax32(umax32(smem[0], smem[1]), umax32(smem[2], smem[3]));
-        // (thousands of atomics on one word take as long as the scan: only a workgroup that can raise the value asks)
-        if (m > __hip_atomic_load(&state[2], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) atomicMax(&state[2], m);
+        state[kStateHeader + blockIdx.x] = umax32(umax32(smem[0], smem[1]), umax32(smem[2], smem[3]));
+        if (blockIdx.x == 0) {
+            state[0] = 0;
+            state[1] = 0;
+            state[2] = gridDim.x;
+        }
     }
 }
 
 // ---- exact maxima of the segments that need them ----------------------------------------------------------------
-// SEED: segments whose sums are within kSeedSlack of the largest (or may hold a non-finite input); otherwise: the
-// remaining segments whose sums exceed what has been found (the thresholds are read once per 64 segments; a stale
-// threshold only costs work).  A wave looks at 64 segments at a time, one per lane, and its eight groups of eight
-// lanes then compute the flagged ones, eight at a time.
+// SEED: segments whose sums are within kSeedSlack of the largest (or may hold a non-finite input); every workgroup
+// leaves its two maxima as partials (a thousand atomics on one word would take longer than the scan).  Otherwise:
+// the thresholds are the maxima of those partials, and the remaining segments whose sums exceed them are computed;
+// what they find is merged with the thresholds by atomics (few: only a wave that can raise a value asks).
+// A wave lists the flagged ones among its 512 segments in LDS, and its eight groups of eight lanes compute them,
+// eight segments at a time.
 template <bool SEED>
 __global__ __launch_bounds__(kThreads) void swiglu_sparse_amax_kernel(const uint16_t* __restrict__ x1,
                                                                       const uint16_t* __restrict__ x3,
@@ -93,56 +119,85 @@ __global__ __launch_bounds__(kThreads) void swiglu_sparse_amax_kernel(const uint
                                                                       const uint16_t* __restrict__ xc,
                                                                       uint32_t* __restrict__ state)
 {
-    __shared__ int32_t picked[kThreads / 64][64];
+    __shared__ uint16_t picked[kThreads / 64][kSegsPerWave];
+    __shared__ int32_t n_picked[kThreads / 64];
+    __shared__ uint32_t smem[3][kThreads / 64];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int sub = lane & 7, grp = lane >> 3;
-    const int64_t wave_id = (int64_t)blockIdx.x * (kThreads / 64) + wave;
-    const int64_t nwaves = (int64_t)gridDim.x * (kThreads / 64);
-    const uint32_t top = state[2];
+    const int n = (int)state[2];  // = gridDim.x of all three launches
+    uint32_t* const seed1 = state + kStateHeader + n;
+    uint32_t* const seed3 = seed1 + n;
+    // the largest sum (and, after the seeds, the thresholds): maxima over the previous launch's partials
+    uint32_t top = 0, t1 = 0, t3 = 0;
+    for (int i = threadIdx.x; i < n; i += kThreads) {
+        top = umax32(top, state[kStateHeader + i]);
+        if (!SEED) {
+            t1 = umax32(t1, seed1[i]);
+            t3 = umax32(t3, seed3[i]);
+        }
+    }
+    top = wave_umax(top);
+    t1 = wave_umax(t1);
+    t3 = wave_umax(t3);
+    if (lane == 0) {
+        smem[0][wave] = top;
+        smem[1][wave] = t1;
+        smem[2][wave] = t3;
+        n_picked[wave] = 0;
+    }
+    __syncthreads();
+    top = umax32(umax32(smem[0][0], smem[0][1]), umax32(smem[0][2], smem[0][3]));
+    t1 = umax32(umax32(smem[1][0], smem[1][1]), umax32(smem[1][2], smem[1][3]));
+    t3 = umax32(umax32(smem[2][0], smem[2][1]), umax32(smem[2][2], smem[2][3]));
+    __syncthreads();
+    if (!SEED && blockIdx.x == 0 && threadIdx.x == 0) {  // the result starts from the seeds' maxima
+        atomicMax(&state[0], t1);
+        atomicMax(&state[1], t3);
+    }
+
+    const int64_t wave_first = ((int64_t)blockIdx.x * (kThreads / 64) + wave) * kSegsPerWave;
+    uint32_t s[kSegsPerLane];
+    load_sums(gc, xc, wave_first + lane * kSegsPerLane, nseg, s);
+#pragma unroll
+    for (int k = 0; k < kSegsPerLane; ++k) {
+        const bool in_range = wave_first + lane * kSegsPerLane + k < nseg;
+        const bool seed = s[k] >= 0x7F80u || s[k] + kSeedSlack >= top;
+        const bool need = in_range && (SEED ? seed : (!seed && swiglu_segment_needed(s[k], t1, t3)));
+        if (need) picked[wave][atomicAdd(&n_picked[wave], 1)] = (uint16_t)(lane * kSegsPerLane + k);
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    const int count = n_picked[wave];
     uint32_t m1 = 0, m3 = 0;
-    for (int64_t base = wave_id * 64; base < nseg; base += nwaves * 64) {
-        const int64_t mine = base + lane;
-        bool need = false;
-        if (mine < nseg) {
-            const uint32_t s = (uint32_t)gc[mine] + (uint32_t)xc[mine];
-            const bool seed = s >= 0x7F80u || s + kSeedSlack >= top;
-            if (SEED) {
-                need = seed;
-            } else {
-                const uint32_t t1 = __hip_atomic_load(&state[0], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                const uint32_t t3 = __hip_atomic_load(&state[1], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                need = !seed && swiglu_segment_needed(s, t1, t3);
-            }
+    for (int k = grp; k < count; k += 8) {
+        const int64_t seg = wave_first + picked[wave][k];
+        const int64_t cb = seg / rows, r = seg % rows;
+        const int64_t c = cb * kSegCols + sub * 8;
+        if (c < cols) {
+            const int64_t off = r * cols + c;
+            uint4 p1, p3;
+            swiglu_bwd8(*reinterpret_cast<const uint4*>(x1 + off), *reinterpret_cast<const uint4*>(x3 + off),
+                        *reinterpret_cast<const uint4*>(gh + off), p1, p3);
+            m1 = umax32(m1, absmax_packed8(p1));
+            m3 = umax32(m3, absmax_packed8(p3));
         }
-        const uint64_t mask = __ballot(need);
-        if (mask == 0) continue;  // (wave-uniform)
-        const int count = __popcll(mask);
-        if (need) picked[wave][__popcll(mask & (((uint64_t)1 << lane) - 1))] = lane;
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-        __builtin_amdgcn_wave_barrier();
-        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-        for (int k = grp; k < count; k += 8) {
-            const int64_t seg = base + picked[wave][k];
-            const int64_t cb = seg / rows, r = seg % rows;
-            const int64_t c = cb * kSegCols + sub * 8;
-            if (c < cols) {
-                const int64_t off = r * cols + c;
-                uint4 p1, p3;
-                swiglu_bwd8(*reinterpret_cast<const uint4*>(x1 + off), *reinterpret_cast<const uint4*>(x3 + off),
-                            *reinterpret_cast<const uint4*>(gh + off), p1, p3);
-                m1 = umax32(m1, absmax_packed8(p1));
-                m3 = umax32(m3, absmax_packed8(p3));
-            }
-        }
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-        __builtin_amdgcn_wave_barrier();
-        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
     }
     m1 = wave_umax(m1);
     m3 = wave_umax(m3);
-    if (lane == 0) {
-        if (m1 > __hip_atomic_load(&state[0], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) atomicMax(&state[0], m1);
-        if (m3 > __hip_atomic_load(&state[1], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) atomicMax(&state[1], m3);
+    if (SEED) {
+        if (lane == 0) {
+            smem[1][wave] = m1;
+            smem[2][wave] = m3;
+        }
+        __syncthreads();
+        if (threadIdx.x == 0) {
+            seed1[blockIdx.x] = umax32(umax32(smem[1][0], smem[1][1]), umax32(smem[1][2], smem[1][3]));
+            seed3[blockIdx.x] = umax32(umax32(smem[2][0], smem[2][1]), umax32(smem[2][2], smem[2][3]));
+        }
+    } else if (lane == 0) {
+        if (m1 > t1 && m1 > __hip_atomic_load(&state[0], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) atomicMax(&state[0], m1);
+        if (m3 > t3 && m3 > __hip_atomic_load(&state[1], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) atomicMax(&state[1], m3);
     }
 }
 
@@ -155,6 +210,12 @@ extern "C" int64_t mi8_rowseg_code_count(int64_t rows, int64_t cols)
 {
     if (rows <= 0 || cols <= 0) return 0;
     return rows * ceil_div(cols, kSegCols);
+}
+
+extern "C" int64_t mi8_swiglu_amax_state_words(int64_t rows, int64_t cols)
+{
+    if (rows <= 0 || cols <= 0) return 0;
+    return kStateHeader + 3 * ceil_div(rows * ceil_div(cols, kSegCols), kSegsPerBlock);
 }
 
 extern "C" int mi8_rowseg_max_codes(const void* a, const void* b, int64_t rows, int64_t cols, uint16_t* codes, void* stream)
@@ -180,14 +241,14 @@ extern "C" int mi8_swiglu_bwd_amax_from_codes(const void* x1, const void* x3, co
                 "mi8_swiglu_bwd_amax_from_codes: tensors must be 16-byte aligned");
     const int64_t nseg = rows * ceil_div(cols, kSegCols);
     MI8_REQUIRE(nseg < ((int64_t)1 << 31), MI8_ERR_UNSUPPORTED, "mi8_swiglu_bwd_amax_from_codes: tensor too large");
+    MI8_REQUIRE(aligned16(gh_codes) && aligned16(x_codes), MI8_ERR_UNSUPPORTED,
+                "mi8_swiglu_bwd_amax_from_codes: code arrays must be 16-byte aligned");
     hipStream_t st = (hipStream_t)stream;
-    hipLaunchKernelGGL(swiglu_amax_init_kernel, dim3(1), dim3(64), 0, st, state);
-    int64_t grid = ceil_div(nseg, kThreads);
-    if (grid > 1024) grid = 1024;
-    hipLaunchKernelGGL(swiglu_max_sum_kernel, dim3((unsigned)grid), dim3(kThreads), 0, st, gh_codes, x_codes, nseg, state);
-    hipLaunchKernelGGL((swiglu_sparse_amax_kernel<true>), dim3((unsigned)grid), dim3(kThreads), 0, st, (const uint16_t*)x1,
+    const unsigned grid = (unsigned)ceil_div(nseg, kSegsPerBlock);
+    hipLaunchKernelGGL(swiglu_max_sum_kernel, dim3(grid), dim3(kThreads), 0, st, gh_codes, x_codes, nseg, state);
+    hipLaunchKernelGGL((swiglu_sparse_amax_kernel<true>), dim3(grid), dim3(kThreads), 0, st, (const uint16_t*)x1,
                        (const uint16_t*)x3, (const uint16_t*)gh, rows, cols, nseg, gh_codes, x_codes, state);
-    hipLaunchKernelGGL((swiglu_sparse_amax_kernel<false>), dim3((unsigned)grid), dim3(kThreads), 0, st, (const uint16_t*)x1,
+    hipLaunchKernelGGL((swiglu_sparse_amax_kernel<false>), dim3(grid), dim3(kThreads), 0, st, (const uint16_t*)x1,
                        (const uint16_t*)x3, (const uint16_t*)gh, rows, cols, nseg, gh_codes, x_codes, state);
     return launch_status("mi8_swiglu_bwd_amax_from_codes");
 }

@@ -463,7 +463,7 @@ def rowseg_max_codes(a: torch.Tensor, b: Optional[torch.Tensor] = None) -> torch
 
 def swiglu_bwd_amax_from_codes(x1: torch.Tensor, x3: torch.Tensor, gh: torch.Tensor, gh_codes: torch.Tensor,
                                x_codes: torch.Tensor) -> torch.Tensor:
-    """The amax of g1 and g3 (float32 bit patterns in words 0 and 1 of the returned int32[4]), computing only the
+    """The amax of g1 and g3 (float32 bit patterns in words 0 and 1 of the returned int32 array), computing only the
     row segments whose codes say they could raise it; equal to the maxima of :func:`swiglu_bwd`'s partials."""
     _require_gpu(x1, "swiglu_bwd_amax_from_codes")
     rows, cols = x1.shape
@@ -471,7 +471,7 @@ def swiglu_bwd_amax_from_codes(x1: torch.Tensor, x3: torch.Tensor, gh: torch.Ten
     for c in (gh_codes, x_codes):
         if c.dtype != torch.int16 or c.numel() != n or not c.is_contiguous() or c.device != x1.device:
             raise ValueError("swiglu_bwd_amax_from_codes: codes must be the int16 arrays of rowseg_max_codes for this shape")
-    state = torch.empty(4, dtype=torch.int32, device=x1.device)
+    state = torch.empty(_C.lib().mi8_swiglu_amax_state_words(rows, cols), dtype=torch.int32, device=x1.device)
     _C.check(
         _C.lib().mi8_swiglu_bwd_amax_from_codes(x1.data_ptr(), x3.data_ptr(), gh.data_ptr(), rows, cols, gh_codes.data_ptr(),
                                                 x_codes.data_ptr(), state.data_ptr(), _stream(x1)),
