@@ -339,6 +339,45 @@ def cast_table():
          2 * xt.numel() + 2 * n, 2 * xt.numel() + 2 * n)
 
 
+def feed_probe():
+    """What feeding operands costs a stream of MFMAs (mi8_probe_mfma_feed): shader cycles per 64-MFMA iteration, the
+    clock the chip held, and the rate, for the pieces of a GEMM K step one at a time and together."""
+    from olmo_core_amd import _C
+
+    dev = torch.device("cuda:0")
+    sink = torch.empty(256 * 256, dtype=torch.float32, device=dev)
+    window = torch.zeros((2 << 20) + (128 << 10), dtype=torch.uint8, device=dev)
+    clocks = torch.zeros(2, dtype=torch.int64, device=dev)
+    st = torch.cuda.current_stream().cuda_stream
+    iters = 20000
+    flop = 256 * 4 * iters * 2.0 * 128 ** 3
+    cases = (
+        (0, 0, 0, 0, "MFMAs only"),
+        (0, 0, 0, 2, "MFMAs, two barriers"),
+        (0, 0, 32, 0, "+ 32 LDS fragment reads (ds_read_b128)"),
+        (0, 8, 0, 0, "+ 8 direct-to-LDS loads (global_load_lds_dwordx4)"),
+        (0, 16, 0, 0, "+ 16 direct-to-LDS loads"),
+        (0, 16, 0, 2, "+ 16 direct-to-LDS loads, two barriers"),
+        (0, 16, 32, 0, "+ 16 direct-to-LDS loads + 32 LDS reads"),
+        (0, 16, 32, 1, "+ 16 direct-to-LDS loads + 32 LDS reads, one barrier"),
+        (0, 16, 32, 2, "+ 16 direct-to-LDS loads + 32 LDS reads, two barriers: the GEMM's K step"),
+        (1, 16, 0, 0, "+ 16 loads to registers (global_load_dwordx4)"),
+        (2, 16, 0, 0, "+ 16 LDS stores of resident registers (ds_write_b128)"),
+        (3, 16, 0, 0, "+ 16 loads to registers and 16 LDS stores, interleaved"),
+        (3, 16, 32, 2, "+ 16 loads to registers, 16 LDS stores, 32 LDS reads, two barriers"),
+    )
+    for rnd in (0, 1):
+        for kind, loads, reads, barriers, name in cases:
+            def run():
+                _C.check(_C.lib().mi8_probe_mfma_feed(kind, loads, reads, barriers, rnd, iters, window.data_ptr(), sink.data_ptr(),
+                                                      clocks.data_ptr(), st))
+            us = _time_us(run, iters=2, warmup=1)
+            cyc, ticks = (int(v) for v in clocks.tolist())
+            print(json.dumps({"probe": "64 MFMAs 16x16x128 per wave and iteration " + name, "operands": "random bytes" if rnd else "zeros",
+                              "cycles_per_iteration": round(cyc / iters, 1), "clock_MHz": round(cyc / (ticks / 100.0), 0),
+                              "TFLOP/s": round(flop / us / 1e6, 1)}), flush=True)
+
+
 def power_probe():
     """What the power limit leaves of the matrix peak: back-to-back MFMAs with nothing else running, and the
     benchmark's longest-K GEMM, each on all-zero and on random operands (under `rocprofv3 --pmc GRBM_GUI_ACTIVE` the
@@ -504,6 +543,7 @@ def main():
                     help="config 5: time the whole routed layer (fused gather, experts, weighted scatter)")
     ap.add_argument("--cast-table", action="store_true", help="time every HBM-bound kernel of the path at the benchmark's shapes")
     ap.add_argument("--power-probe", action="store_true", help="bare MFMA loops and the GEMM on zero / random operands")
+    ap.add_argument("--feed-probe", action="store_true", help="an MFMA stream with the loads and LDS reads of a GEMM K step beside it")
     ap.add_argument("--profile-summary", type=str, default=None, metavar="DIR_OR_CSV",
                     help="print the per-kernel table of a rocprofv3 --stats --output-format csv run (no GPU needed)")
     ap.add_argument("--counter-summary", type=str, default=None, metavar="DIR_OR_CSV",
@@ -532,6 +572,9 @@ def main():
         return
     if ns.cast_table:
         cast_table()
+        return
+    if ns.feed_probe:
+        feed_probe()
         return
     if ns.power_probe:
         power_probe()

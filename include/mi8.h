@@ -390,6 +390,16 @@ int mi8_moe_binned_scatter_wgrad(const void* x, const void* grad, int dtype, int
  * its power limit.  sink: float32 [workgroups * 256], overwritten.
  * ------------------------------------------------------------------------------------------- */
 int mi8_probe_mfma_loop(int mfma_shape, int random_operands, int iterations, int workgroups, float* sink, void* stream);
+/* What the operand feed of a GEMM K step costs a stream of MFMAs (diagnostic, no counterpart in the reference):
+ * 256 workgroups of four waves run 64 16x16x128 MFMAs per iteration from resident registers and, beside them,
+ * `loads` (0, 8, 16) loads of 1 KB per wave - kind 0: direct to LDS, 1: to registers, 2: LDS stores of resident
+ * registers instead, 3: loads to registers and LDS stores interleaved - and `reads` (0, 32) 16-byte LDS fragment
+ * reads per wave, with `barriers` (0..2) workgroup barriers per iteration.  window: at least 2 MiB + 128 KiB of
+ * readable device memory; sink: 65536 floats;
+ * clocks[0] = shader-clock cycles of the loop on one workgroup, clocks[1] = the same span in ticks of the constant
+ * 100 MHz clock (host-visible or device memory). */
+int mi8_probe_mfma_feed(int kind, int loads, int reads, int barriers, int random_operands, int iterations, const void* window,
+                        float* sink, unsigned long long* clocks, void* stream);
 
 #ifdef __cplusplus
 }

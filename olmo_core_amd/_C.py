@@ -130,6 +130,7 @@ _SIGNATURES = {
         [c_void_p, c_void_p, c_int, c_int64, c_int64, c_void_p, c_void_p, c_int32, c_int64, c_int32, c_void_p, c_void_p],
     ),
     "mi8_probe_mfma_loop": (c_int, [c_int, c_int, c_int, c_int, c_void_p, c_void_p]),
+    "mi8_probe_mfma_feed": (c_int, [c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p]),
     "mi8_grouped_padded_rows": (c_int64, [c_int64, c_int32]),
     "mi8_grouped_cast_colwise_t": (
         c_int,

@@ -22,6 +22,8 @@
 // (bank-conflict free for the fragment reads, see swz16).  The swizzle of a fragment row does not depend on the
 // tile it belongs to, so two address registers per operand serve all eight tiles through the instruction's
 // offset field.
+#include <type_traits>
+
 #include "mi8_gemm_tiles.h"
 #include "mi8_swiglu.h"
 
@@ -242,7 +244,9 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_fp8_m16_kernel(Problem pb)
             advance_load_cursor();
         }
     }
-    v4i fa_lo[4][2], fa_hi[4][2], fb[NT][2];  // A tiles 0-3, A tiles 4-7, B tiles 0-7
+    // A tiles 0-3, A tiles 4-7, and two sets of B tiles 0-7: a step multiplies from one set while the next step's B
+    // fragments are read into the other
+    v4i fa_lo[4][2], fa_hi[4][2], fb[2][NT][2];
     // fragments a step's phase A starts from: A tiles 0-3 and all B tiles of the stage the read addresses point at
     auto read_step_head = [&]() __attribute__((always_inline)) {
 #pragma unroll
@@ -252,8 +256,8 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_fp8_m16_kernel(Problem pb)
         }
 #pragma unroll
         for (int t = 0; t < NT; ++t) {
-            read_b(fb[t], t, 0);
-            read_b(fb[t], t, 1);
+            read_b(fb[0][t], t, 0);
+            read_b(fb[0][t], t, 1);
         }
     };
     __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wave's direct loads have landed
@@ -267,7 +271,13 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_fp8_m16_kernel(Problem pb)
         // One 128-byte K step.  `fresh`: the tile's first step; phase A touches the accumulators of A tiles 0-3,
         // phase B those of A tiles 4-7, so both start from 0 then.  The first step is written out separately
         // from the loop, not as a branch inside it.
-        auto k_step = [&](bool fresh) __attribute__((always_inline)) {
+        // S (a compile-time 0 or 1): the set of B fragments this step multiplies from; the next step's go into the other
+        // one.  With a single set, a B tile's next copy could only be requested once its last MFMA of the step was
+        // issued, the last tile's at the very end of the step - and the first MFMA of the next step then waited out the
+        // LDS latency (the wait at a loop head covers every read in flight).  Now all reads of a step are issued in the
+        // first three quarters of phase B.
+        auto k_step = [&](bool fresh, auto set_tag) __attribute__((always_inline)) {
+            constexpr int S = decltype(set_tag)::value;
             const int cur = step & 1;
             // every wave has issued its reads of this stage's B rows and A tiles 0-3 (previous phase B)
             asm volatile("s_barrier" ::: "memory");
@@ -276,7 +286,7 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_fp8_m16_kernel(Problem pb)
 #pragma unroll
             for (int x = 0; x < 32; ++x) {
                 const int j = x >> 2, i = x & 3;
-                mma(fa_lo[i], fb[j], acc[i][j], fresh);
+                mma(fa_lo[i], fb[S][j], acc[i][j], fresh);
                 if (x < 8) read_a(fa_hi[x >> 1], 4 + (x >> 1), x & 1);
                 if (x >= 8 && x % 3 == 2) dma_one(ld_a, ld_b, cur, kLoads + (x - 8) / 3);
                 __builtin_amdgcn_sched_barrier(0);
@@ -299,17 +309,14 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_fp8_m16_kernel(Problem pb)
                 __builtin_amdgcn_s_waitcnt(0x0F78);  // vmcnt(8)
             asm volatile("s_barrier" ::: "memory");
             flip_read_stage(cur ^ 1);
-            // phase B, B tile by B tile: the next step's copy of a B tile is read once its four MFMAs are issued;
-            // the A half of step + 2 is fetched into the A rows of this stage
+            // phase B: the next step's fragments - all B tiles (into the other set), then A tiles 0-3 - are read
+            // behind the first 24 MFMAs; the A half of step + 2 is fetched into the A rows of this stage
 #pragma unroll
             for (int x = 0; x < 32; ++x) {
                 const int j = x >> 2, i = x & 3;
-                mma(fa_hi[i], fb[j], acc[4 + i][j], fresh);
-                if (x < 8) read_a(fa_lo[x >> 1], x >> 1, x & 1);
-                if (i == 3) {
-                    read_b(fb[j], j, 0);
-                    read_b(fb[j], j, 1);
-                }
+                mma(fa_hi[i], fb[S][j], acc[4 + i][j], fresh);
+                if (x < 16) read_b(fb[S ^ 1][x >> 1], x >> 1, x & 1);
+                if (x >= 16 && x < 24) read_a(fa_lo[(x - 16) >> 1], (x - 16) >> 1, x & 1);
                 if (i == 1) dma_one(ld_a, ld_b, cur, x >> 2);
                 __builtin_amdgcn_sched_barrier(0);
             }
@@ -317,8 +324,17 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_fp8_m16_kernel(Problem pb)
             ++step;
         };
         if (td.nk > 0) {
-            k_step(true);
-            for (int kt = 1; kt < td.nk; ++kt) k_step(false);
+            // a tile starts from set 0 (read_step_head) and alternates; what the last step prefetched for the next
+            // tile is read again after the epilogue, into set 0
+            const std::integral_constant<int, 0> set0;
+            const std::integral_constant<int, 1> set1;
+            k_step(true, set0);
+            int kt = 1;
+            for (; kt + 1 < td.nk; kt += 2) {
+                k_step(false, set1);
+                k_step(false, set0);
+            }
+            if (kt < td.nk) k_step(false, set1);
         } else {  // nothing is accumulated (empty group): the tile is all zeros
 #pragma unroll
             for (int i = 0; i < NT; ++i)
