@@ -242,7 +242,23 @@ def cast_rates(iters: int = 10):
     end.record()
     torch.cuda.synchronize()
     us = start.elapsed_time(end) / iters * 1e3
+    # as the step runs them: the producers leave the amax (of h) or the codes it follows from (of g1, g3), so each
+    # tensor is read once
+    slots = ops.amax_partials(h)
+    us_h = _time_us(lambda: ops.cast_tensorwise(h, torch.float8_e4m3fn, want_rowmajor=True, want_transposed=True, slots=slots), iters)
+    x1 = torch.randn(TOKENS, HIDDEN, device=dev, dtype=torch.bfloat16)
+    gh = (torch.randn(TOKENS, HIDDEN, device=dev) * 1e-3).to(torch.bfloat16)
+    gc, xc = ops.rowseg_max_codes(gh), ops.rowseg_max_codes(x1, h)
+    us_g = _time_us(lambda: ops.swiglu_bwd_cast(x1, h, gh, torch.float8_e5m2, want_transposed=True, codes=(gc, xc)), iters)
+    in_step = {
+        "h (amax from the producing GEMM): tile_cast_kernel, 4 B/elem": {
+            "us": round(us_h, 1), "GB/s_algorithmic": round(4.0 * n / us_h / 1e3, 1), "frac_hbm_peak_algorithmic": round(4.0 * n / us_h / 1e3 / HBM_PEAK_GBS, 4)},
+        "g1, g3 (amax from row-segment codes): sparse amax + swiglu_bwd_cast_kernel, 10 B/elem": {
+            "us": round(us_g, 1), "GB/s_algorithmic": round(10.0 * n / us_g / 1e3, 1), "frac_hbm_peak_algorithmic": round(10.0 * n / us_g / 1e3 / HBM_PEAK_GBS, 4)},
+    }
+    del x1, gh, gc, xc
     return {
+        "as_run_in_the_step": in_step,
         "tensor": f"{TOKENS}x{HIDDEN} bf16 -> e4m3 row-major + transposed, tensorwise (amax pass + cast pass)",
         "us": round(us, 1),
         "GB/s_algorithmic_4B_per_elem": round(4.0 * n / us / 1e3, 1),
@@ -316,7 +332,18 @@ def cast_table():
                                                   s3.data_ptr(), st)), 6 * n, 6 * n)
     line("swiglu backward to float8 (amax pass + swiglu_bwd_cast_kernel): g1, g3 row-major + transposed", shape,
          _time_us(lambda: ops.swiglu_bwd_cast(x1, x3, gh, e5m2, want_transposed=True)), 10 * n, 16 * n)
-    del x1, x3, gh
+    # the route the feed-forward block takes: the producers of x1, x3 and gh leave row-segment codes, and the amax comes
+    # from the few segments that can hold it
+    gc, xc = ops.rowseg_max_codes(gh), ops.rowseg_max_codes(x1, x3)
+    line("amax of g1, g3 from row-segment codes (three sparse launches)", shape,
+         _time_us(lambda: ops.swiglu_bwd_amax_from_codes(x1, x3, gh, gc, xc)), 6 * n, 4 * (n // 64))
+    line("swiglu backward to float8 (amax from codes + swiglu_bwd_cast_kernel): g1, g3 row-major + transposed", shape,
+         _time_us(lambda: ops.swiglu_bwd_cast(x1, x3, gh, e5m2, want_transposed=True, codes=(gc, xc))), 10 * n, 10 * n)
+    h = torch.randn(*shape, device=dev).to(torch.bfloat16)
+    hs = ops.amax_partials(h)
+    line("tensorwise cast of h with the amax from the GEMM that wrote it: row-major + transposed (= tile_cast_kernel)", shape,
+         _time_us(lambda: ops.cast_tensorwise(h, e4m3, want_rowmajor=True, want_transposed=True, slots=hs)), 4 * n, 4 * n)
+    del x1, x3, gh, h
     # grouped (configuration 5): 131072 routed rows of 2048, the benchmark's group sizes
     _, _, _, _, desc = build_config(5, dev)
     g = torch.Generator().manual_seed(1005)
@@ -534,7 +561,7 @@ def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--config", type=int, default=2, help="benchmark configuration 1..5 (2 is the headline line)")
     ap.add_argument("--keep-float8-weights", action="store_true",
