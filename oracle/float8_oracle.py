@@ -354,6 +354,36 @@ def swiglu_backward(x1, x3, gh):
     return x1.grad, x3.grad
 
 
+# ---- magnitude codes: the bound behind the sparse amax of the SwiGLU gradients --------------------------------
+# (no counterpart in the reference, which takes the amax with a pass over the gradients, torchao tensor_to_amax;
+# the product finds the same amax from these codes and is tested against this restatement and against that pass)
+
+SWIGLU_MARGIN_G3, SWIGLU_MARGIN_G1, BF16_CODE_BIAS = 24, 44, 127 * 128
+
+
+def bf16_magnitude_code(x: torch.Tensor) -> torch.Tensor:
+    """L(x): the 15 exponent-and-mantissa bits of a bf16 value as an integer.  L / 128 - 127 <= log2 |x| <=
+    L / 128 - 127 + 0.0861 for normal values (a piecewise-linear logarithm)."""
+    assert x.dtype == torch.bfloat16
+    return x.contiguous().view(torch.int16).to(torch.int32) & 0x7FFF
+
+
+def rowseg_max_codes(a: torch.Tensor, b: Optional[torch.Tensor] = None, seg: int = 64) -> torch.Tensor:
+    """One code per `seg` consecutive columns of a row: the largest L in the segment (of a, or of a and b), laid out
+    [ceil(cols / seg)][rows] like the product's arrays."""
+    rows, cols = a.shape
+    nseg = -(-cols // seg)
+    la = bf16_magnitude_code(a) if b is None else torch.maximum(bf16_magnitude_code(a), bf16_magnitude_code(b))
+    padded = torch.zeros((rows, nseg * seg), dtype=torch.int32)
+    padded[:, :cols] = la
+    return padded.view(rows, nseg, seg).amax(dim=2).t().contiguous().reshape(-1)
+
+
+def swiglu_gradient_code_bounds(code_sum: torch.Tensor):
+    """Largest L a gradient can have where the codes of gh and of (x1, x3) sum to `code_sum`: (for g1, for g3)."""
+    return code_sum + SWIGLU_MARGIN_G1 - BF16_CODE_BIAS, code_sum + SWIGLU_MARGIN_G3 - BF16_CODE_BIAS
+
+
 def mlp_fwd_bwd(x, w1, w2, w3, grad_out, spec: LinearSpec) -> MLPTrace:
     """y = w2(silu(w1 x) * w3 x); all three projections float8; backward through all of them."""
     t1 = linear_forward(x, w1, None, spec)

@@ -6,7 +6,7 @@ consumes it writes the same bytes and scales."""
 import pytest
 import torch
 
-from helpers import E5M2, seeded
+from helpers import E5M2, O, seeded
 
 pytestmark = pytest.mark.gpu
 
@@ -81,6 +81,7 @@ def test_codes_kernel_equals_host_restatement(dev, shape):
     x1, x3, gh = _inputs(dev, *shape, "outliers")
     assert torch.equal(ops.rowseg_max_codes(gh), _host_codes(gh))
     assert torch.equal(ops.rowseg_max_codes(x1, x3), _host_codes(x1, x3))
+    assert torch.equal(ops.rowseg_max_codes(x1, x3).cpu().to(torch.int32), O.rowseg_max_codes(x1.cpu(), x3.cpu()))
 
 
 def test_bound_holds_for_every_x1_pattern(dev):

@@ -463,3 +463,42 @@ def test_dropless_mlp_exact_on_representable_inputs():
     want = torch.cat(outs)
     assert float(want.abs().max()) <= 2.0**15
     assert torch.equal(res["y"].float(), want.bfloat16().float())
+
+
+def test_magnitude_codes_bound_the_swiglu_gradients():
+    """The property the sparse amax of the gate gradients rests on, against torch's own bf16 autograd: for every bf16
+    pattern of x1 and a spread of gh and x3 values, the code of each gradient is at most the sum of the inputs' codes
+    plus its margin (checked where inputs and gradient are finite and the gradient is not in the denormal range);
+    and the codes are a lower bound on log2 |x| within 0.0861."""
+    import numpy as np
+
+    pats = torch.from_numpy(np.arange(65536, dtype=np.uint16).view(np.int16).copy()).view(torch.bfloat16)
+    lx = O.bf16_magnitude_code(pats)
+    finite = (lx < 0x7F80) & (lx >= 0x0080)
+    log2 = torch.log2(pats.double().abs()[finite])
+    est = lx[finite].double() / 128 - 127
+    assert (est <= log2 + 1e-12).all() and (log2 <= est + 0.0861).all()
+    others = torch.tensor([1.0, -3.0, 0.37, 1e-3, 255.0, 1.99, 1e-30, 3e20, -7.5e-4, 0.0078125], dtype=torch.bfloat16)
+    for gv in others:
+        for bv in others[:6]:
+            x1 = pats.clone()
+            x3 = torch.full_like(x1, bv.item())
+            gh = torch.full_like(x1, gv.item())
+            g1, g3 = O.swiglu_backward(x1, x3, gh)
+            lg, la, lb = O.bf16_magnitude_code(gh), O.bf16_magnitude_code(x1), O.bf16_magnitude_code(x3)
+            ok_in = (la < 0x7F80) & (lb < 0x7F80) & (lg < 0x7F80)
+            for grad, s, which in ((g1, lg + torch.maximum(la, lb), 0), (g3, lg + torch.maximum(la, lb), 1), (g1, lg + lb, 0), (g3, lg + la, 1)):
+                lgr = O.bf16_magnitude_code(grad)
+                bound = O.swiglu_gradient_code_bounds(s)[which]
+                ok = ok_in & (lgr < 0x7F80) & (lgr >= 0x0400)
+                assert not (ok & (lgr > bound)).any(), (gv.item(), bv.item(), which)
+
+
+def test_rowseg_codes_layout():
+    x = torch.zeros((3, 130), dtype=torch.bfloat16)
+    x[0, 5], x[1, 64], x[2, 129], x[2, 0] = -2.0, 0.5, 3.0, float("inf")
+    codes = O.rowseg_max_codes(x).view(3, 3)  # [segment][row]
+    two, half, three = 0x4000, 0x3F00, 0x4040
+    assert codes.tolist() == [[two, 0, 0x7F80], [0, half, 0], [0, 0, three]]
+    both = O.rowseg_max_codes(x, torch.full_like(x, 1.0)).view(3, 3)
+    assert both.tolist() == [[two, 0x3F80, 0x7F80], [0x3F80, 0x3F80, 0x3F80], [0x3F80, 0x3F80, three]]
