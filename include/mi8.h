@@ -71,6 +71,15 @@ const char* mi8_last_error(void);
  * The number of slots used depends only on n. */
 int mi8_amax_partials(const void* x, int hp_dtype, int64_t n, uint32_t* slots, int32_t* n_slots_used, void* stream);
 
+/* mi8_amax_partials for up to MI8_AMAX_BATCH tensors of one dtype in ONE launch (the input and the three weights of a
+ * feed-forward block, whose tensorwise scales the reference reduces one after the other: torchao tensor_to_scale per
+ * Float8Linear, reference src/olmo_core/float8/ao.py:76-86).  xs, ns, n_slots_used are HOST arrays of `count` entries;
+ * tensor t's partials go to slots[t * MI8_AMAX_SLOTS ...], n_slots_used[t] (may be NULL) = mi8_amax_slots_for(ns[t]);
+ * the values equal those of `count` separate mi8_amax_partials calls.  slots must hold count * MI8_AMAX_SLOTS uint32. */
+#define MI8_AMAX_BATCH 8
+int mi8_amax_partials_batch(const void* const* xs, const int64_t* ns, int32_t count, int hp_dtype, uint32_t* slots,
+                            int32_t* n_slots_used, void* stream);
+
 /* Number of slots mi8_amax_partials uses for n elements (host-side, no GPU work). */
 int32_t mi8_amax_slots_for(int64_t n);
 

@@ -31,6 +31,7 @@ _SIGNATURES = {
     "mi8_version": (c_int, []),
     "mi8_last_error": (c_char_p, []),
     "mi8_amax_partials": (c_int, [c_void_p, c_int, c_int64, c_void_p, POINTER(c_int32), c_void_p]),
+    "mi8_amax_partials_batch": (c_int, [POINTER(c_void_p), POINTER(c_int64), c_int32, c_int, c_void_p, POINTER(c_int32), c_void_p]),
     "mi8_amax_slots_for": (c_int32, [c_int64]),
     "mi8_scale_from_partials": (c_int, [c_void_p, c_int32, c_int, c_uint32, c_void_p, c_void_p]),
     "mi8_multi_tensor_scales": (

@@ -71,15 +71,16 @@ __device__ __forceinline__ uint32_t wave_umax(uint32_t v)
 struct BlockRange {
     int64_t lo, hi;
 };
-__device__ __forceinline__ BlockRange block_range(int64_t n)
+__device__ __forceinline__ BlockRange block_range(int64_t n, int64_t block, int64_t blocks)
 {
-    const int64_t per = (((n + gridDim.x - 1) / gridDim.x) + 255) & ~(int64_t)255;
-    int64_t lo = (int64_t)blockIdx.x * per;
+    const int64_t per = (((n + blocks - 1) / blocks) + 255) & ~(int64_t)255;
+    int64_t lo = block * per;
     lo = lo < n ? lo : n;
     int64_t hi = lo + per;
     hi = hi < n ? hi : n;
     return BlockRange{lo, hi};
 }
+__device__ __forceinline__ BlockRange block_range(int64_t n) { return block_range(n, blockIdx.x, gridDim.x); }
 
 // scale = float32(FP8_MAX * (1 / max(float64(amax), 1e-12))); NaN amax gives a NaN scale, +inf gives 0.
 // Optional round-down to a power of two clears the mantissa (scale is always a normal float or 0 here).

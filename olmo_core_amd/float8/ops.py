@@ -81,6 +81,31 @@ def amax_partials(x: torch.Tensor) -> Tuple[torch.Tensor, int]:
     return slots, used.value
 
 
+AMAX_BATCH = 8
+
+
+def amax_partials_batch(tensors) -> list:
+    """:func:`amax_partials` of up to ``AMAX_BATCH`` contiguous GPU tensors of one dtype in one launch: a list of
+    ``(slots, n_used)`` in the order given (same values as separate calls)."""
+    n = len(tensors)
+    if not 0 < n <= AMAX_BATCH:
+        raise ValueError(f"amax_partials_batch: {n} tensors (1..{AMAX_BATCH})")
+    t0 = tensors[0]
+    _require_gpu(t0, "amax_partials_batch")
+    for t in tensors:
+        if t.dtype != t0.dtype or t.device != t0.device or not t.is_contiguous():
+            raise ValueError("amax_partials_batch: tensors must be contiguous, on one GPU and of one dtype")
+    slots = torch.empty((n, _C.AMAX_SLOTS), dtype=torch.int32, device=t0.device)
+    ptrs = (_C.c_void_p * n)(*[t.data_ptr() for t in tensors])
+    numels = (_C.c_int64 * n)(*[t.numel() for t in tensors])
+    used = (_C.c_int32 * n)()
+    _C.check(
+        _C.lib().mi8_amax_partials_batch(ptrs, numels, n, _HP_CODE[t0.dtype], slots.data_ptr(), used, _stream(t0)),
+        "mi8_amax_partials_batch",
+    )
+    return [(slots[i], int(used[i])) for i in range(n)]
+
+
 def scale_from_partials(slots: torch.Tensor, n_slots: int, fp8_dtype: torch.dtype, pow2: bool = False) -> torch.Tensor:
     """Returns a float32 tensor [2] = (scale, amax)."""
     out = torch.empty(2, dtype=torch.float32, device=slots.device)

@@ -70,12 +70,20 @@ class _Float8SwiGLUMLP(torch.autograd.Function):
         need = ctx.needs_input_grad
         any_grad = any(need[:4])
         x_codes = None
-        xq, xq_t, sx = ops.cast_tensorwise(x, in_dt, pow2=pow2, want_transposed=need[1] or need[3])
         # ws*: weight scales precomputed after the optimizer step (None: reduce the amax here);
         # wo*: float8 copies the modules keep between calls (None: quantise the weight here)
-        w1q, w1q_t, s1 = wo1 or ops.cast_tensorwise(w1, w_dt, pow2=pow2, want_transposed=need[0], scale=ws1)
-        w3q, w3q_t, s3 = wo3 or ops.cast_tensorwise(w3, w_dt, pow2=pow2, want_transposed=need[0], scale=ws3)
-        w2q, w2q_t, s2 = wo2 or ops.cast_tensorwise(w2, w_dt, pow2=pow2, want_transposed=any_grad, scale=ws2)
+        # The amax of x and of every weight that still needs one is taken in a single launch.
+        todo = [x] + [w for w, ws, wo in ((w1, ws1, wo1), (w3, ws3, wo3), (w2, ws2, wo2)) if ws is None and wo is None]
+        part = {}
+        if len(todo) > 1 and all(t.dtype == x.dtype and t.is_contiguous() for t in todo):
+            part = {id(t): p for t, p in zip(todo, ops.amax_partials_batch(todo))}
+        xq, xq_t, sx = ops.cast_tensorwise(x, in_dt, pow2=pow2, want_transposed=need[1] or need[3], slots=part.get(id(x)))
+        w1q, w1q_t, s1 = wo1 or ops.cast_tensorwise(w1, w_dt, pow2=pow2, want_transposed=need[0], scale=ws1,
+                                                    slots=part.get(id(w1)))
+        w3q, w3q_t, s3 = wo3 or ops.cast_tensorwise(w3, w_dt, pow2=pow2, want_transposed=need[0], scale=ws3,
+                                                    slots=part.get(id(w3)))
+        w2q, w2q_t, s2 = wo2 or ops.cast_tensorwise(w2, w_dt, pow2=pow2, want_transposed=any_grad, scale=ws2,
+                                                    slots=part.get(id(w2)))
         if FUSE_SWIGLU_EPILOGUE and x.dtype == torch.bfloat16 and ops.swiglu_gemm_matches_separate(x.shape[0], w1.shape[0], x.shape[1]):
             # both input projections and the activation in one launch: x1 and x3 are never read back
             if any_grad and SWIGLU_AMAX_FROM_CODES and w1.shape[0] % 64 == 0:

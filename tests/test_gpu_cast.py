@@ -169,6 +169,29 @@ def test_amax_partials_and_scale(dev):
                 assert float(out[1]) == float(x.abs().max().float())
 
 
+def test_amax_partials_batch_equals_separate_calls(dev):
+    """One launch over several tensors leaves, per tensor, exactly the partials of its own launch (ragged sizes,
+    a tail shorter than a vector, float32 as well as bf16, the maximum in the last element)."""
+    sizes = (5, 8, 8191, 1 << 20, (1 << 22) + 3, 4096 * 11008, 1000, 64)
+    for dt in (torch.bfloat16, torch.float32):
+        xs = [seeded((n,), seed=100 + n % 97, std=1.0 + i).to(dt) for i, n in enumerate(sizes)]
+        xs[4][-1] = 1e4
+        xs[0][4] = -77.0
+        xd = [x.to(dev) for x in xs]
+        for count in (1, 3, len(xd)):
+            got = ops.amax_partials_batch(xd[:count])
+            assert len(got) == count
+            for x, xdev, (slots, used) in zip(xs, xd, got):
+                ref_slots, ref_used = ops.amax_partials(xdev)
+                assert used == ref_used
+                assert torch.equal(slots[:used], ref_slots[:used])
+                assert float(slots[:used].view(torch.float32).max().cpu()) == float(x.abs().max().float())
+    with pytest.raises(ValueError):
+        ops.amax_partials_batch([xd[0]] * 9)
+    with pytest.raises(ValueError):
+        ops.amax_partials_batch([xd[0].float(), xd[1].bfloat16()])
+
+
 def test_scale_every_bf16_amax(dev):
     """Scale for every positive finite bf16 amax value (one row each) - the f64 route on the GPU."""
     vals = all_bf16_patterns()
