@@ -114,17 +114,23 @@ def build_config(n, dev, keep_float8_weights=False, routed=False):
                 p.copy_(rand(p.shape, g, 0.02))
         mods = mods.to(dev)
         Float8Config(ao_recipe=AOFloat8LinearRecipe.rowwise).apply_float8_linear(mods)
+        # q, k and v are applied to one tensor, as in the attention block (they share its float8 copy); the output
+        # projection has an input of its own
         x = rand((m, d), g).to(dev).requires_grad_(True)
+        x_o = rand((m, d), g).to(dev).requires_grad_(True)
         go = rand((m, d), g, 1e-3).to(dev)
 
         def fn():
-            x.grad = None
+            x.grad = x_o.grad = None
             for lin in mods:
                 lin.weight.grad = None
-                lin(x).backward(go)
+            ys = [lin(x) for lin in mods[:3]] + [mods[3](x_o)]
+            for y in ys:
+                y.backward(go)
 
         f = 2.0 * m * d * d
-        return fn, 12 * f, 12, f, "config 3: OLMo-3-7B q/k/v/o projections fwd+bwd, tokens 16384, rowwise recipe"
+        return fn, 12 * f, 12, f, ("config 3: OLMo-3-7B q/k/v/o projections fwd+bwd, tokens 16384, rowwise recipe "
+                                   "(q, k, v on one input, o on another)")
     if n == 5:
         g = torch.Generator().manual_seed(1005)
         E, d, h, T, top_k = 64, 2048, 1024, 16384, 8

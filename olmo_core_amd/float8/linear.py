@@ -21,6 +21,7 @@ transposed copy for operands reduced along their columns.
 
 from __future__ import annotations
 
+import weakref
 from typing import Callable, Optional, Tuple
 
 import torch
@@ -83,27 +84,59 @@ def _saves_quantised(c: Float8LinearConfig, need_gx: bool, need_gw: bool) -> Tup
     return x_is_q, w_is_q
 
 
-def _forward_impl(x2, weight, c: Float8LinearConfig, weight_scale, need_gx: bool, need_gw: bool, weight_ops=None):
-    """y = x2 @ weight^T in float8.  Returns ``(y, x_saved, w_saved)``: the tensors the backward needs for x and
-    for the weight, each either ``(q_t, scale)`` (see :func:`_saves_quantised`) or ``None`` (keep the input).
-    ``weight_ops``: ``(q, q_t, scale)`` of the weight kept by the module (:meth:`Float8Linear.weight_operands`);
-    the weight is then not quantised here."""
-    pow2 = c.round_scales_to_power_of_2
-    share_x, share_w = _saves_quantised(c, need_gx, need_gw)
-    x_saved = w_saved = None
-    if _is_disabled(c.cast_config_input):
-        return torch.mm(x2, weight.t().to(x2.dtype)), None, None
-    if _is_tensorwise(c.cast_config_input):
-        xq, xq_t, sx = ops.cast_tensorwise(
-            x2, c.cast_config_input.target_dtype, pow2=pow2, want_rowmajor=True, want_transposed=share_x
-        )
+# Sibling projections applied to one tensor (q, k and v of an attention block) would each quantise it again, to the
+# same bytes and scales (the reference does: every Float8Linear casts its own input).  The operands of the last input
+# are remembered - keyed by the identity of the tensor the module was called with, its address and version counter,
+# and the cast - and dropped when that tensor dies or another input arrives.  Eager mode only.
+SHARE_INPUT_CASTS = True
+_INPUT_MEMO = None  # (weakref to the input, version, address, key, operands)
+
+
+def _drop_input_memo(_ref=None) -> None:
+    global _INPUT_MEMO
+    if _ref is None or (_INPUT_MEMO is not None and _INPUT_MEMO[0] is _ref):
+        _INPUT_MEMO = None
+
+
+def _input_operands(x2, c: Float8LinearConfig, pow2: bool, share_x: bool, origin):
+    """``(xq, sx, x_saved)`` for the forward GEMM: the by-rows operand, its scale, and what the backward keeps."""
+    global _INPUT_MEMO
+    ci = c.cast_config_input
+    key = (ci.scaling_type, ci.scaling_granularity, ci.target_dtype, pow2, share_x, tuple(x2.shape), x2.dtype)
+    src = origin[0] if origin is not None and SHARE_INPUT_CASTS else None
+    memo = _INPUT_MEMO
+    if (src is not None and memo is not None and memo[0]() is src and memo[1] == src._version
+            and memo[2] == x2.data_ptr() and memo[3] == key):
+        return memo[4]
+    x_saved = None
+    if _is_tensorwise(ci):
+        xq, xq_t, sx = ops.cast_tensorwise(x2, ci.target_dtype, pow2=pow2, want_rowmajor=True, want_transposed=share_x)
         if share_x:
             x_saved = (xq_t, sx)
     elif share_x:  # per-row copy for this GEMM, per-column transposed copy for grad_weight, one cast
-        xq, sx, xq_t, sxc = ops.cast_rows_and_colwise_t(x2, c.cast_config_input.target_dtype, pow2=pow2)
+        xq, sx, xq_t, sxc = ops.cast_rows_and_colwise_t(x2, ci.target_dtype, pow2=pow2)
         x_saved = (xq_t, sxc)
     else:
-        xq, sx = ops.cast_rowwise(x2, c.cast_config_input.target_dtype, pow2=pow2)
+        xq, sx = ops.cast_rowwise(x2, ci.target_dtype, pow2=pow2)
+    res = (xq, sx, x_saved)
+    if src is not None:
+        _INPUT_MEMO = (weakref.ref(src, _drop_input_memo), src._version, x2.data_ptr(), key, res)
+    return res
+
+
+def _forward_impl(x2, weight, c: Float8LinearConfig, weight_scale, need_gx: bool, need_gw: bool, weight_ops=None,
+                  origin=None):
+    """y = x2 @ weight^T in float8.  Returns ``(y, x_saved, w_saved)``: the tensors the backward needs for x and
+    for the weight, each either ``(q_t, scale)`` (see :func:`_saves_quantised`) or ``None`` (keep the input).
+    ``weight_ops``: ``(q, q_t, scale)`` of the weight kept by the module (:meth:`Float8Linear.weight_operands`);
+    the weight is then not quantised here.  ``origin``: ``(tensor,)``, the tensor the module was called with (x2 is
+    a view of it), for :func:`_input_operands`."""
+    pow2 = c.round_scales_to_power_of_2
+    share_x, share_w = _saves_quantised(c, need_gx, need_gw)
+    w_saved = None
+    if _is_disabled(c.cast_config_input):
+        return torch.mm(x2, weight.t().to(x2.dtype)), None, None
+    xq, sx, x_saved = _input_operands(x2, c, pow2, share_x, origin)
     if weight_ops is not None:
         wq, wq_t, sw = weight_ops
         if share_w:
@@ -167,9 +200,9 @@ class _Float8Matmul(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, x2: torch.Tensor, weight: torch.Tensor, config: Float8LinearConfig, weight_scale=None,
-                weight_ops=None):
+                weight_ops=None, origin=None):
         need_gx, need_gw = ctx.needs_input_grad[0], ctx.needs_input_grad[1]
-        y, x_saved, w_saved = _forward_impl(x2, weight, config, weight_scale, need_gx, need_gw, weight_ops)
+        y, x_saved, w_saved = _forward_impl(x2, weight, config, weight_scale, need_gx, need_gw, weight_ops, origin)
         ctx.config = config
         ctx.x_dtype, ctx.w_dtype = x2.dtype, weight.dtype
         ctx.shapes = (x2.shape[0], x2.shape[1], weight.shape[0])
@@ -191,7 +224,7 @@ class _Float8Matmul(torch.autograd.Function):
             go.reshape(M, N), ctx.config, N, ctx.x_dtype, ctx.w_dtype, saved[: ctx.n_x], saved[ctx.n_x :],
             ctx.x_is_q, ctx.w_is_q, ctx.needs_input_grad[0], ctx.needs_input_grad[1],
         )
-        return gx, gw, None, None, None
+        return gx, gw, None, None, None, None
 
 
 # Operator arguments must be plain values: under torch.compile a config travels as its index in this list.  Configs
@@ -209,8 +242,8 @@ def _register_config(c: Float8LinearConfig) -> int:
 
 
 @torch.compiler.disable
-def _eager_matmul(x2, weight, config, weight_scale, weight_ops=None):
-    return _Float8Matmul.apply(x2, weight, config, weight_scale, weight_ops)
+def _eager_matmul(x2, weight, config, weight_scale, weight_ops=None, origin=None):
+    return _Float8Matmul.apply(x2, weight, config, weight_scale, weight_ops, origin)
 
 
 def float8_linear_function(
@@ -239,9 +272,9 @@ def float8_linear_function(
         y = compiled.linear(x2, weight, cfg_id, weight_scale)
     elif not compiling and not (torch.is_grad_enabled() and (x2.requires_grad or weight.requires_grad)):
         # nothing to differentiate (evaluation, generation): no autograd node, nothing kept for a backward
-        y = _forward_impl(x2, weight, config, weight_scale, False, False, weight_ops)[0]
+        y = _forward_impl(x2, weight, config, weight_scale, False, False, weight_ops, (x,))[0]
     else:  # eager, or a config no module registered: a graph break
-        y = _eager_matmul(x2, weight, config, weight_scale, weight_ops)
+        y = _eager_matmul(x2, weight, config, weight_scale, weight_ops, None if compiling else (x,))
     return y.reshape(*x.shape[:-1], weight.shape[0])
 
 

@@ -355,6 +355,78 @@ def test_kept_weight_operands(dev, monkeypatch):
     assert len(casts) == 8
 
 
+
+@pytest.mark.parametrize("recipe", RECIPES)
+def test_sibling_projections_share_the_input_cast(dev, recipe, monkeypatch):
+    """q/k/v-style modules applied to one tensor quantise it once; outputs and gradients are the bits of modules that
+    each quantise it themselves; writing to the tensor in place, or another tensor at the same address, is seen."""
+    from olmo_core_amd.float8 import linear as L
+
+    M, K, N = 384, 256, 320
+    mods = []
+    for i in range(3):
+        lin = nn.Linear(K, N, bias=False, dtype=torch.bfloat16)
+        with torch.no_grad():
+            lin.weight.copy_(seeded((N, K), 40 + i, std=0.02))
+        mods.append(Float8Linear.from_float(lin.to(dev), Float8LinearConfig.from_recipe_name(recipe)))
+    gos = [seeded((M, N), 50 + i, std=1e-3).to(dev) for i in range(3)]
+
+    calls = {"n": 0}
+    for name in ("cast_tensorwise", "cast_rows_and_colwise_t", "cast_rowwise"):
+        orig = getattr(ops, name)
+
+        def counted(t, *a, _orig=orig, **k):
+            if t.shape == (M, K):
+                calls["n"] += 1
+            return _orig(t, *a, **k)
+
+        monkeypatch.setattr(ops, name, counted)
+
+    def run(share):
+        monkeypatch.setattr(L, "SHARE_INPUT_CASTS", share)
+        L._drop_input_memo()
+        calls["n"] = 0
+        x = seeded((M, K), 7).to(dev).requires_grad_(True)
+        for m in mods:
+            m.weight.grad = None
+        ys = [m(x) for m in mods]
+        n_fwd = calls["n"]
+        for y, go in zip(ys, gos):
+            y.backward(go)
+        return n_fwd, ys, x.grad, [m.weight.grad.clone() for m in mods]
+
+    n1, ys1, gx1, gw1 = run(True)
+    n0, ys0, gx0, gw0 = run(False)
+    assert (n1, n0) == (1, 3)
+    assert torch.equal(gx1, gx0)
+    for a, b in zip(ys1 + gw1, ys0 + gw0):
+        assert torch.equal(a, b)
+
+    # an in-place write invalidates the remembered operands
+    monkeypatch.setattr(L, "SHARE_INPUT_CASTS", True)
+    L._drop_input_memo()
+    with torch.no_grad():
+        x = seeded((M, K), 8).to(dev)
+        y_a = mods[0](x)
+        x.mul_(2.0)
+        y_b = mods[0](x)
+        monkeypatch.setattr(L, "SHARE_INPUT_CASTS", False)
+        assert torch.equal(y_b, mods[0](x)) and not torch.equal(y_a, y_b)
+        monkeypatch.setattr(L, "SHARE_INPUT_CASTS", True)
+        # a different tensor object (here: at the same address, the first one having died) is never taken for the old one
+        L._drop_input_memo()
+        x1 = seeded((M, K), 9).to(dev)
+        y1 = mods[1](x1)
+        ptr = x1.data_ptr()
+        del x1
+        assert L._INPUT_MEMO is None  # dropped with the tensor
+        x2 = seeded((M, K), 10).to(dev)
+        y2 = mods[1](x2)
+        monkeypatch.setattr(L, "SHARE_INPUT_CASTS", False)
+        assert torch.equal(y2, mods[1](x2))
+        assert x2.data_ptr() != ptr or not torch.equal(y1, y2)
+
+
 @pytest.mark.parametrize("tokens", [16, 300], ids=["few_rows", "split_k"])
 def test_forward_replays_from_a_captured_graph(dev, tokens):
     """A generation loop captures one step in a HIP graph and replays it: every launch of the forward (casts,
