@@ -51,11 +51,35 @@ def test_host_only_entry_points():
     assert L.mi8_gemm_splitk_workspace_bytes(0, 30, 4) == 0
 
 
+def test_host_only_shape_helpers():
+    """Sizes and shape predicates the callers plan with (no GPU work)."""
+    L = _C.lib()
+    # one code per 64 columns of a row, ragged last segment included
+    assert L.mi8_rowseg_code_count(16384, 11008) == 16384 * 172
+    assert L.mi8_rowseg_code_count(3, 65) == 6 and L.mi8_rowseg_code_count(0, 64) == 0
+    assert L.mi8_swiglu_amax_state_words(16384, 11008) >= 4 and L.mi8_swiglu_amax_state_words(0, 0) == 0
+    # the GEMM that records codes is the persistent tile kernel: full tiles, K in 128-byte steps, whole segments
+    assert L.mi8_gemm_fp8_codes_supported(16384, 11008, 4096) == 1
+    for shape in ((128, 11008, 4096), (16384, 11008, 4000), (16384, 11000, 4096)):
+        assert L.mi8_gemm_fp8_codes_supported(*shape) == 0, shape
+    # the fused SwiGLU launch replaces the separate GEMMs only where both run on that kernel
+    assert L.mi8_gemm_fp8_swiglu_matches_separate(16384, 11008, 4096) == 1
+    assert L.mi8_gemm_fp8_swiglu_matches_separate(64, 11008, 4096) == 0
+    # the padded token axis of the grouped transposed copies: groups whose sizes sum to T fill at most
+    # ceil(T / 128) + groups - 1 tiles of 128 rows
+    assert L.mi8_grouped_padded_rows(131072, 64) == 131072 + 63 * 128
+    assert L.mi8_grouped_padded_rows(5, 2) == 2 * 128
+
+
 def test_argument_validation_happens_before_any_gpu_call():
     L = _C.lib()
     assert L.mi8_cast_rowwise(None, 0, 4, 16, 0, 0, None, 16, None, None) == -1
     assert "null" in _C.last_error()
     assert L.mi8_gemm_fp8(None, 0, 16, None, 0, 16, 1, 1, 16, None, 0, None, 0, None, 0, 16, -1, None) == -1
     assert L.mi8_gemm_fp8_splitk(None, 0, 16, None, 0, 16, 1, 1, 16, None, 0, None, 0, None, 0, 16, 2, None, 0, None) == -1
+    assert L.mi8_amax_partials_batch(None, None, 1, 0, None, None, None) == -1
+    ptrs, ns = (ctypes.c_void_p * 9)(), (ctypes.c_int64 * 9)()
+    assert L.mi8_amax_partials_batch(ptrs, ns, 9, 0, ctypes.c_void_p(16), None, None) == -1 and "9 tensors" in _C.last_error()
+    assert L.mi8_amax_partials_batch(ptrs, ns, 2, 0, ctypes.c_void_p(16), None, None) == -1 and "tensor 0 is null" in _C.last_error()
     with pytest.raises(Exception):
         _C.check(-2, "x")
