@@ -1,6 +1,6 @@
 // Problem policies of the persistent direct-to-LDS fp8 GEMM kernels: how a linear tile index maps to operand
 // panels, scales and output rows for the dense problem and for the ragged grouped problems (forward /
-// grad_input and grad_weight of a dropless-MoE expert layer).  Shared by the 32x32x64 and 16x16x128 kernels.
+// grad_input and grad_weight of a dropless-MoE expert layer).
 #pragma once
 #include "mi8_gemm.h"
 #include "mi8_groups.h"
@@ -39,7 +39,7 @@ struct DenseProblem {
     static constexpr bool kAccumulate = ACC;  // C += the rounded product
     static constexpr bool kOutCodes = CODES;
     static constexpr bool kSwiglu = false;
-    static constexpr bool kMaskRows = false, kXcdRanges = true, kPeelFirstStep = true;
+    static constexpr bool kMaskRows = false, kXcdRanges = true;
     using Cache = NoCache;
     __device__ __forceinline__ Cache prepare() const { return Cache{}; }
     __device__ __forceinline__ int total_tiles(const Cache&) const { return g.tiles_m * g.tiles_n; }
@@ -82,7 +82,7 @@ struct SwigluProblem {
     uint32_t* h_slots;      // [4 * workgroups] partial maxima of |h| (float32 bit patterns)
     uint16_t* x_codes;      // null, or [H / 64][M] codes of the larger of x1 and x3 per row segment (H % 64 == 0)
     static constexpr bool kVecScales = false, kAccumulate = false, kSwiglu = true, kOutCodes = false;
-    static constexpr bool kMaskRows = false, kXcdRanges = true, kPeelFirstStep = true;
+    static constexpr bool kMaskRows = false, kXcdRanges = true;
     using Cache = NoCache;
     __device__ __forceinline__ Cache prepare() const { return Cache{}; }
     __device__ __forceinline__ int total_tiles(const Cache&) const { return g.tiles_m * g.tiles_n; }
@@ -176,7 +176,7 @@ struct GroupedProblem {
     int N, K, tiles_n;
     const float* sa;
     const float* sb;
-    static constexpr bool kVecScales = true, kMaskRows = true, kXcdRanges = true, kPeelFirstStep = false;
+    static constexpr bool kVecScales = true, kMaskRows = true, kXcdRanges = true;
     using Cache = GroupCache;
     __device__ __forceinline__ Cache prepare() const { return build_group_cache<BM>(sizes, E, T); }
     __device__ __forceinline__ int total_tiles(const Cache& c) const
@@ -235,7 +235,7 @@ struct GroupedWgradProblem {
     int N, Kl, tiles_n, tiles_k;
     const float* sa;  // [E, N]
     const float* sb;  // [E, Kl]
-    static constexpr bool kVecScales = true, kMaskRows = false, kXcdRanges = false, kPeelFirstStep = true;
+    static constexpr bool kVecScales = true, kMaskRows = false, kXcdRanges = false;
     static constexpr bool kAccumulate = false, kSwiglu = false, kOutCodes = false;
     using Cache = WgradCache;
     __device__ __forceinline__ Cache prepare() const
