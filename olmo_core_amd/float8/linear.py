@@ -102,8 +102,14 @@ def _input_operands(x2, c: Float8LinearConfig, pow2: bool, share_x: bool, origin
     """``(xq, sx, x_saved)`` for the forward GEMM: the by-rows operand, its scale, and what the backward keeps."""
     global _INPUT_MEMO
     ci = c.cast_config_input
-    key = (ci.scaling_type, ci.scaling_granularity, ci.target_dtype, pow2, share_x, tuple(x2.shape), x2.dtype)
-    src = origin[0] if origin is not None and SHARE_INPUT_CASTS else None
+    src = origin[0] if origin is not None and SHARE_INPUT_CASTS and x2.is_cuda else None
+    if src is not None and torch.cuda.is_current_stream_capturing():
+        src = None  # what a graph capture allocates belongs to the graph's memory pool: nothing of it is remembered
+    key = None
+    if src is not None:
+        # (the stream is part of the key: operands made on one stream are not handed to work queued on another)
+        key = (ci.scaling_type, ci.scaling_granularity, ci.target_dtype, pow2, share_x, tuple(x2.shape), x2.dtype,
+               torch.cuda.current_stream(x2.device).cuda_stream)
     memo = _INPUT_MEMO
     if (src is not None and memo is not None and memo[0]() is src and memo[1] == src._version
             and memo[2] == x2.data_ptr() and memo[3] == key):
