@@ -279,3 +279,20 @@ def test_kept_weight_operands_need_the_switch_and_a_gpu_weight():
         Float8Config(ao=cfg).apply_float8_linear(model)
         assert isinstance(model[0], Float8Linear)
         assert model[0].weight_operands() is None
+
+
+def test_product_never_reaches_for_the_checker_or_working_files():
+    """The package (Python and HIP sources) imports, reads and names nothing under oracle/ or _work/: the oracle is
+    test infrastructure, working files are not part of the repository."""
+    import re
+    from pathlib import Path
+
+    pkg = Path(__file__).resolve().parent.parent / "olmo_core_amd"
+    offenders = []
+    for path in pkg.rglob("*"):
+        if path.suffix not in (".py", ".hip", ".h") or "__pycache__" in path.parts:
+            continue
+        text = path.read_text()
+        if re.search(r"\b(from|import)\s+oracle\b|oracle/|_work/|liboracle", text):
+            offenders.append(str(path.relative_to(pkg)))
+    assert offenders == []
