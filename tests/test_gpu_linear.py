@@ -402,8 +402,21 @@ def test_sibling_projections_share_the_input_cast(dev, recipe, monkeypatch):
     for a, b in zip(ys1 + gw1, ys0 + gw0):
         assert torch.equal(a, b)
 
-    # an in-place write invalidates the remembered operands
+    # operands made on one stream are not handed to work queued on another
     monkeypatch.setattr(L, "SHARE_INPUT_CASTS", True)
+    L._drop_input_memo()
+    with torch.no_grad():
+        xs = seeded((M, K), 11).to(dev)
+        calls["n"] = 0
+        y_main = mods[0](xs)
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            y_side = mods[0](xs)
+        torch.cuda.current_stream().wait_stream(side)
+        assert calls["n"] == 2 and torch.equal(y_main, y_side)
+
+    # an in-place write invalidates the remembered operands
     L._drop_input_memo()
     with torch.no_grad():
         x = seeded((M, K), 8).to(dev)
