@@ -22,7 +22,8 @@ from ..float8.linear import Float8Linear, _is_tensorwise, _shared_tensorwise
 __all__ = ["FeedForward", "swiglu"]
 
 # Test hook: when set to a dict, the fused function stores clones of its bf16 intermediates (x1, x3, h, gh) there,
-# so that a checker can feed each stage's actual input to a reference of that stage.
+# so that a checker can feed each stage's actual input to a reference of that stage, together with the float8
+# operands it made of h, g1 and g3 and their scales (sh, hq, sg1, g1q, sg3, g3q): what the GEMMs actually consumed.
 STAGE_SINK = None
 
 # Run the two input projections and the SwiGLU between them as one launch where the shape allows (same bits as the
@@ -97,6 +98,8 @@ class _Float8SwiGLUMLP(torch.autograd.Function):
         if STAGE_SINK is not None:
             STAGE_SINK.update(x1=x1.clone(), x3=x3.clone(), h=h.clone())
         hq, hq_t, sh = ops.cast_tensorwise(h, in_dt, pow2=pow2, want_transposed=need[2], slots=h_slots)
+        if STAGE_SINK is not None:
+            STAGE_SINK.update(sh=sh.clone(), hq=hq.clone())
         y = ops.gemm_fp8(hq, sh, w2q, s2, out_dtype=x.dtype)
         ctx.config = c
         ctx.dtypes = (x.dtype, w1.dtype, w2.dtype, w3.dtype, go_dt)
@@ -141,6 +144,9 @@ class _Float8SwiGLUMLP(torch.autograd.Function):
             g1q, g1q_t, sg1, g3q, g3q_t, sg3 = ops.swiglu_bwd_cast(
                 x1, x3, gh, go_dt, pow2=pow2, want_rowmajor=need_x, want_transposed=need_t, codes=codes)
             del gh
+            if STAGE_SINK is not None:
+                STAGE_SINK.update(sg1=sg1.clone(), sg3=sg3.clone(), amax_from_codes=codes is not None,
+                                  g1q=None if g1q is None else g1q.clone(), g3q=None if g3q is None else g3q.clone())
             if need_x:
                 # the sum of the two halves as autograd forms it (two bf16 tensors added), by the second GEMM's epilogue
                 gx = ops.gemm_fp8(g1q, sg1, w1q_t, s1, k=H, out_dtype=x_dt)

@@ -13,8 +13,18 @@ from helpers import (E4M3, E5M2, assert_bf16_pointwise_close, assert_bytes_equal
 from oracle import float8_oracle as O
 
 
-def check_mlp_stages(dev, ff, x, go, recipe="tensorwise"):
-    """ff: a converted olmo_core_amd.nn.FeedForward on `dev` (tensorwise recipe, fused); x, go: host bf16 tensors."""
+def _sample(n, count, first):
+    """`count` indices spread over range(n), starting at `first` (so that tile edges and interiors are both hit)."""
+    step = max(n // count, 1)
+    return torch.arange(first % step, n, step)[:count]
+
+
+def check_mlp_stages(dev, ff, x, go, recipe="tensorwise", sample=None):
+    """ff: a converted olmo_core_amd.nn.FeedForward on `dev` (tensorwise recipe, fused); x, go: host bf16 tensors.
+    sample: None - every GEMM stage is compared on the whole result; n - on n rows and n columns of the result (the
+    oracle's operands are still the casts of the whole tensors: a tensorwise scale depends on every element), which
+    keeps the host side at seconds for the benchmark's shapes.  Casts and pointwise stages are always compared on the
+    whole tensor."""
     from olmo_core_amd.float8 import ops
     from olmo_core_amd.nn import feed_forward as ff_mod
 
@@ -28,45 +38,80 @@ def check_mlp_stages(dev, ff, x, go, recipe="tensorwise"):
         y.backward(go.to(dev))
     finally:
         ff_mod.STAGE_SINK = None
-    assert set(sink) == {"x1", "x3", "h", "gh"}, "the fused function did not run"
+    assert {"x1", "x3", "h", "gh", "sh", "hq", "sg1", "sg3", "g1q", "g3q"} <= set(sink), "the fused function did not run"
     gx, gw1, gw2, gw3 = xd.grad, ff.w1.weight.grad, ff.w2.weight.grad, ff.w3.weight.grad
     x1, x3, h, gh = (sink[k].cpu() for k in ("x1", "x3", "h", "gh"))
 
+    # the oracle's float8 operands of the host tensors (x, the weights, grad_output)
+    xq, sx = O.cast(x, E4M3)
+    w1q, s1 = O.cast(w1, E4M3)
+    w3q, s3 = O.cast(w3, E4M3)
+    w2q, s2 = O.cast(w2, E4M3)
+    goq, sgo = O.cast(go, E5M2)
+
+    def mm(aq, sa, bq_t, sb, got, what):
+        """got [R, C] against (aq [R, K] / sa) @ (bq_t [K, C] / sb), whole or on sampled rows and columns."""
+        if sample is None:
+            assert_gemm_close(got, O.emulated_mm_f32(aq, sa, bq_t, sb), what)
+            return
+        rows = _sample(aq.shape[0], sample, 7)
+        cols = _sample(bq_t.shape[1], sample, 3)
+        assert_gemm_close(got[rows.to(got.device)], O.emulated_mm_f32(aq[rows], sa, bq_t, sb), what + " (rows)")
+        assert_gemm_close(got[:, cols.to(got.device)], O.emulated_mm_f32(aq, sa, bq_t[:, cols], sb), what + " (columns)")
+
     # stage 1: the two input projections from x
-    assert_gemm_close(x1, O.linear_forward(x, w1, None, spec).out, "x1 = x W1^T")
-    assert_gemm_close(x3, O.linear_forward(x, w3, None, spec).out, "x3 = x W3^T")
+    mm(xq, sx, w1q.t(), s1, sink["x1"], "x1 = x W1^T")
+    mm(xq, sx, w3q.t(), s3, sink["x3"], "x3 = x W3^T")
     # stage 2: h from the device's x1, x3
     assert_bf16_pointwise_close(h, O.swiglu(x1, x3), "h = silu(x1) * x3")
-    # stage 3: the cast of the device's h (bytes and scale bit-exact), then y and w2's backward from it
-    hq, hq_t, sh = ops.cast_tensorwise(sink["h"], E4M3, want_transposed=True)
+    # stage 3: the cast of the device's h - the scale and bytes the block itself used (its amax came out of the
+    # GEMM epilogue) and those of the stand-alone cast kernel - then y and w2's backward from it
     ref_hq, ref_sh = O.cast(h, E4M3)
+    assert_scale_equal(sink["sh"], ref_sh, "scale of h used by the block")
+    assert_bytes_equal(sink["hq"], ref_hq, what="q(h) used by the block")
+    hq, hq_t, sh = ops.cast_tensorwise(sink["h"], E4M3, want_transposed=True)
     assert_scale_equal(sh, ref_sh, "scale of h")
     assert_bytes_equal(hq, ref_hq, what="q(h)")
     assert_bytes_equal(hq_t[:, :M], ref_hq.t(), what="q(h)^T")
-    t2 = O.linear_fwd_bwd(h, w2, None, go, spec)
-    assert_gemm_close(y, t2.out, "y = h W2^T")
-    assert_gemm_close(gw2, t2.grad_weight, "grad_w2 = go^T h")
-    assert_gemm_close(gh, t2.grad_input, "grad_h = go W2")
+    del hq, hq_t
+    mm(ref_hq, ref_sh, w2q.t(), s2, y, "y = h W2^T")
+    mm(goq.t(), sgo, ref_hq, ref_sh, gw2, "grad_w2 = go^T h")
+    mm(goq, sgo, w2q, s2, sink["gh"], "grad_h = go W2")
     # stage 4: the gate gradients from the device's x1, x3, grad_h.  The fused block never writes them in bf16: the
     # two-step kernels (bit-identical to the fused route, test_swiglu_backward_cast_equals_two_steps) are compared
-    # with the host's autograd, and the fused cast's bytes with the oracle's cast of the device's g1, g3
+    # with the host's autograd, and the bytes and scales the block used (its amax came from the row-segment codes,
+    # where the shape allows) with the oracle's cast of the device's g1, g3
     g1, g3, _, _ = ops.swiglu_bwd(sink["x1"], sink["x3"], sink["gh"])
     r1, r3 = O.swiglu_backward(x1, x3, gh)
     assert_bf16_pointwise_close(g1, r1, "g1", max_frac=2e-2)
     assert_bf16_pointwise_close(g3, r3, "g3", max_frac=2e-2)
-    q1, q1t, s1, q3, q3t, s3 = ops.swiglu_bwd_cast(sink["x1"], sink["x3"], sink["gh"], E5M2, want_transposed=True)
+    del r1, r3
+    q1, q1t, sc1, q3, q3t, sc3 = ops.swiglu_bwd_cast(sink["x1"], sink["x3"], sink["gh"], E5M2, want_transposed=True)
     g1, g3 = g1.cpu(), g3.cpu()
-    for name, g, q, qt, s in (("g1", g1, q1, q1t, s1), ("g3", g3, q3, q3t, s3)):
+    ref = {}
+    for name, g, q, qt, s in (("g1", g1, q1, q1t, sc1), ("g3", g3, q3, q3t, sc3)):
         ref_q, ref_s = O.cast(g, E5M2)
+        ref[name] = (ref_q, ref_s)
+        assert_scale_equal(sink["s" + name], ref_s, f"scale of {name} used by the block (amax from codes: {sink['amax_from_codes']})")
+        assert_bytes_equal(sink[name + "q"], ref_q, what=f"q({name}) used by the block")
         assert_scale_equal(s, ref_s, f"scale of {name}")
         assert_bytes_equal(q, ref_q, what=f"q({name})")
         assert_bytes_equal(qt[:, :M], ref_q.t(), what=f"q({name})^T")
+    del q1, q1t, q3, q3t
     # stage 5: w1 / w3 backward from the device's g1, g3
-    b1 = O.linear_backward(x, w1, g1, spec)
-    b3 = O.linear_backward(x, w3, g3, spec)
-    assert_gemm_close(gw1, b1.grad_weight, "grad_w1 = g1^T x")
-    assert_gemm_close(gw3, b3.grad_weight, "grad_w3 = g3^T x")
-    assert_gemm_close(gx, b1.grad_input + b3.grad_input, "grad_x = g1 W1 + g3 W3")
+    (g1q, sg1), (g3q, sg3) = ref["g1"], ref["g3"]
+    mm(g1q.t(), sg1, xq, sx, gw1, "grad_w1 = g1^T x")
+    mm(g3q.t(), sg3, xq, sx, gw3, "grad_w3 = g3^T x")
+    if sample is None:
+        want = O.emulated_mm(g1q, sg1, w1q, s1) + O.emulated_mm(g3q, sg3, w3q, s3)
+        assert_gemm_close(gx, want, "grad_x = g1 W1 + g3 W3")
+    else:
+        rows, cols = _sample(M, sample, 7), _sample(x.shape[1], sample, 3)
+        want = O.emulated_mm(g1q[rows], sg1, w1q, s1) + O.emulated_mm(g3q[rows], sg3, w3q, s3)
+        assert_gemm_close(gx[rows.to(dev)], want, "grad_x = g1 W1 + g3 W3 (rows)")
+        want = O.emulated_mm(g1q, sg1, w1q[:, cols], s1) + O.emulated_mm(g3q, sg3, w3q[:, cols], s3)
+        assert_gemm_close(gx[:, cols.to(dev)], want, "grad_x = g1 W1 + g3 W3 (columns)")
+    return sink
 
 
 def check_dropless_stages(dev, mlp, x, go, sizes, experts):

@@ -1,7 +1,8 @@
-"""Parity at the stated shapes of the benchmark configurations 3, 4 and 5 (the 7B shapes of configuration 2 are in
-test_gpu_gemm.py): casts bit-exact on the whole tensor or on whole experts, GEMM outputs on samples of rows so that
-the host side stays at seconds.
+"""Parity at the stated shapes of the benchmark configurations 2, 3, 4 and 5 (single GEMMs of the 7B shapes of
+configuration 2 are in test_gpu_gemm.py): casts bit-exact on the whole tensor or on whole experts, GEMM outputs on
+samples of rows and columns so that the host side stays at seconds.
 
+  config 2: the fused 7B feed-forward block fwd+bwd at the shape bench.py times (16384 tokens, 4096 -> 11008 -> 4096)
   config 3: q/k/v/o projection 4096 -> 4096 at 16384 tokens, rowwise recipe (per-row, per-channel, power-of-two scales)
   config 4: 32B-shape MLP, d_model 5120, hidden 27648, 8192 tokens, tensorwise, 0.1 % of x scaled x100
   config 5: 64 experts, d_model 2048, hidden 1024, 131072 routed rows with Zipf-skewed group sizes (7 empty, one of 1 row)
@@ -19,6 +20,29 @@ from olmo_core_amd.float8 import AOFloat8LinearRecipe, Float8Config, ops  # noqa
 from olmo_core_amd.float8.linear import Float8Linear  # noqa: E402
 from olmo_core_amd.float8.native_config import Float8LinearConfig  # noqa: E402
 from olmo_core_amd.nn import DroplessMoEMLP, FeedForward  # noqa: E402
+
+
+# ---- config 2 ------------------------------------------------------------------------------------------------------
+
+
+def test_config2_fused_mlp_bench_shape(dev):
+    """The block bench.py times, at its shape and seed: the dual-B SwiGLU launch over 86 x 64 tiles, the code-recording
+    grad_h GEMM, the amax of g1, g3 from 2.8 M row segments and the accumulating grad_x GEMM, stage by stage; every
+    byte and the scale of q(h), q(g1), q(g3) as the block used them against the oracle's cast of the device's tensors."""
+    from stage_checks import check_mlp_stages
+
+    M, D, H = 16384, 4096, 11008
+    g = torch.Generator().manual_seed(1002)
+    ff = FeedForward(d_model=D, hidden_size=H, bias=False, dtype=torch.bfloat16)
+    with torch.no_grad():
+        for p in ff.parameters():
+            p.copy_((torch.randn(p.shape, generator=g) * 0.02).to(torch.bfloat16))
+    ff = ff.to(dev)
+    Float8Config(ao_recipe=AOFloat8LinearRecipe.tensorwise).apply_float8_linear(ff)
+    x = torch.randn(M, D, generator=g).to(torch.bfloat16)
+    go = (torch.randn(M, D, generator=g) * 1e-3).to(torch.bfloat16)
+    sink = check_mlp_stages(dev, ff, x, go, sample=12)
+    assert sink["amax_from_codes"], "the benchmark's shape takes the row-segment-code route"
 
 
 # ---- config 3 ------------------------------------------------------------------------------------------------------

@@ -89,11 +89,15 @@ def test_bound_holds_for_every_x1_pattern(dev):
     magnitude is below what the element's own bound allows (the property the skipping of blocks rests on)."""
     pats = torch.arange(65536, dtype=torch.int32).to(torch.int16).view(torch.bfloat16).to(dev)
     others = torch.tensor([1.0, -3.0, 0.37, 1e-3, 255.0, 1.99, 1e-30, 3e20, -7.5e-4, 0.0078125], dtype=torch.bfloat16, device=dev)
-    for gv in others:
-        for bv in others[:6]:
+    # mantissas where the sum of two codes under-estimates the product's logarithm the most (around sqrt(2) - 1) and
+    # where the product's mantissa wraps (around 2 - sqrt(2)), on several exponents, for gh and for x3
+    worst = torch.tensor([m * e for m in (1.4140625, 1.4765625, 1.171875, 1.5859375, 1.40625, 1.421875)
+                          for e in (1.0, -2.0 ** -10, 2.0 ** 7, 2.0 ** -20)], dtype=torch.bfloat16, device=dev)
+    for gv in torch.cat([others, worst]).tolist():
+        for bv in torch.cat([others[:6], worst[::4], worst[1::4]]).tolist():
             x1 = pats.view(256, 256).contiguous()
-            x3 = torch.full_like(x1, bv.item())
-            gh = torch.full_like(x1, gv.item())
+            x3 = torch.full_like(x1, bv)
+            gh = torch.full_like(x1, gv)
             g1, g3, _, _ = ops.swiglu_bwd(x1, x3, gh, want_amax=False)
             lg, la, lb = _L(gh), _L(x1), _L(x3)
             finite_in = (la < 0x7F80) & (lb < 0x7F80) & (lg < 0x7F80)
@@ -103,7 +107,7 @@ def test_bound_holds_for_every_x1_pattern(dev):
                 # log2 |grad| >= L(grad) / 128 - 127 must not exceed the bound (s + margin) / 128 - 254 (the sum of the
                 # elements' own codes: segment codes are maxima of these and only loosen the bound)
                 bad = ok & (lgr + BIAS > s + margin)
-                assert not bad.any(), f"{name}: bound violated for x1 pattern {int(pats.view(-1)[bad.view(-1)][0].view(torch.int16))}, gh {gv.item()}, x3 {bv.item()}"
+                assert not bad.any(), f"{name}: bound violated for x1 pattern {int(pats.view(-1)[bad.view(-1)][0].view(torch.int16))}, gh {gv}, x3 {bv}"
 
 
 @pytest.mark.parametrize("kind", KINDS)

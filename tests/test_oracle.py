@@ -479,8 +479,15 @@ def test_magnitude_codes_bound_the_swiglu_gradients():
     est = lx[finite].double() / 128 - 127
     assert (est <= log2 + 1e-12).all() and (log2 <= est + 0.0861).all()
     others = torch.tensor([1.0, -3.0, 0.37, 1e-3, 255.0, 1.99, 1e-30, 3e20, -7.5e-4, 0.0078125], dtype=torch.bfloat16)
-    for gv in others:
-        for bv in others[:6]:
+    # The code of a product exceeds the sum of the factors' codes the most when both mantissas sit near sqrt(2) - 1
+    # (a piecewise-linear logarithm under-estimates most in the middle of a binade: the gap is 21.96 of the margin's
+    # 24 units there); around 2 - sqrt(2) the mantissa of the product wraps.  Those mantissas, on several exponents,
+    # for gh and for x3 (x1 runs over every pattern anyway).
+    worst = torch.tensor([m * e for m in (1.4140625, 1.4765625, 1.171875, 1.5859375, 1.40625, 1.421875)
+                          for e in (1.0, -2.0 ** -10, 2.0 ** 7, 2.0 ** -20)], dtype=torch.bfloat16)
+    assert torch.equal(worst.float()[:4], torch.tensor([1.4140625, -1.4140625 * 2.0 ** -10, 1.4140625 * 128, 1.4140625 * 2.0 ** -20]))
+    for gv in torch.cat([others, worst]):
+        for bv in torch.cat([others[:6], worst[::4], worst[1::4]]):
             x1 = pats.clone()
             x3 = torch.full_like(x1, bv.item())
             gh = torch.full_like(x1, gv.item())
