@@ -60,13 +60,18 @@ def build_mlp(dev):
 # ---- the other benchmark configurations (parity-test shapes; measured with --config N) ----
 
 
-def build_config(n, dev, keep_float8_weights=False, routed=False):
+def build_config(n, dev, keep_float8_weights=False, routed=False, compile_model=False, recommended=False):
     """Returns (step_fn, flops_per_step, gemms_per_step, flops_per_gemm_launch or None, description).
+    Configurations 2 and 4 only: `compile_model` runs the block through torch.compile (the mode the reference's training
+    scripts run every block in); `recommended` converts with AOFloat8LinearConfig.recommended() (what those scripts
+    set: power-of-two scales, float8 weights kept between weight updates) instead of the plain tensorwise recipe, and
+    the timed steps are then micro-batches between two optimizer steps: no weight is quantised inside them.
     Configuration 5 only: `keep_float8_weights` keeps the experts' float8 weight copies from step to step (the
     steady state of gradient-accumulation micro-batches; by default every step quantises the weights again, as a
     step that follows an optimizer update must); `routed` times the whole routed layer (token gather fused into
     the quantisation, experts, weighted scatter back to token order) instead of the experts alone."""
     from olmo_core_amd.float8 import AOFloat8LinearRecipe, Float8Config
+    from olmo_core_amd.float8.linear import float8_projections
     from olmo_core_amd.nn import DroplessMoEMLP, FeedForward, ParallelDroplessMLP
 
     def rand(shape, g, std=1.0):
@@ -95,7 +100,14 @@ def build_config(n, dev, keep_float8_weights=False, routed=False):
             for p in mlp.parameters():
                 p.copy_(rand(p.shape, g, 0.02))
         mlp = mlp.to(dev)
-        Float8Config(ao_recipe=AOFloat8LinearRecipe.tensorwise).apply_float8_linear(mlp)
+        if recommended:
+            from olmo_core_amd.float8 import AOFloat8LinearConfig
+
+            Float8Config(ao=AOFloat8LinearConfig.recommended()).apply_float8_linear(mlp)
+        else:
+            Float8Config(ao_recipe=AOFloat8LinearRecipe.tensorwise).apply_float8_linear(mlp)
+        params = list(mlp.parameters())
+        run = torch.compile(mlp) if compile_model else mlp
         x = torch.randn(m, d, generator=g)
         if n == 4:  # 0.1 % of the entries x100
             pos = torch.randperm(m * d, generator=g)[: m * d // 1000]
@@ -104,7 +116,19 @@ def build_config(n, dev, keep_float8_weights=False, routed=False):
         go = rand((m, d), g, 1e-3).to(dev)
         f = 2.0 * m * d * h
         name = "OLMo-2-7B" if n == 2 else "OLMo-2-32B (0.1 % outliers x100)"
-        return (lambda: step(mlp, x, go)), 9 * f, 9, f, f"config {n}: {name} SwiGLU MLP fwd+bwd, tokens {m}, tensorwise"
+        desc = f"config {n}: {name} SwiGLU MLP fwd+bwd, tokens {m}, tensorwise"
+        if recommended:
+            desc += ", AOFloat8LinearConfig.recommended() (float8 weights kept between weight updates: micro-batch steady state)"
+        if compile_model:
+            desc += ", block under torch.compile"
+
+        def fn_mlp():
+            x.grad = None
+            for p in params:
+                p.grad = None
+            run(x).backward(go)
+
+        return fn_mlp, 9 * f, 9, f, desc
     if n == 3:
         g = torch.Generator().manual_seed(1003)
         m, d = 16384, 4096
@@ -114,8 +138,8 @@ def build_config(n, dev, keep_float8_weights=False, routed=False):
                 p.copy_(rand(p.shape, g, 0.02))
         mods = mods.to(dev)
         Float8Config(ao_recipe=AOFloat8LinearRecipe.rowwise).apply_float8_linear(mods)
-        # q, k and v are applied to one tensor, as in the attention block (they share its float8 copy); the output
-        # projection has an input of its own
+        # q, k and v are applied to one tensor, as in the attention block (float8_projections: one quantisation of
+        # x, grad_x summed by the GEMM epilogues); the output projection has an input of its own
         x = rand((m, d), g).to(dev).requires_grad_(True)
         x_o = rand((m, d), g).to(dev).requires_grad_(True)
         go = rand((m, d), g, 1e-3).to(dev)
@@ -124,9 +148,8 @@ def build_config(n, dev, keep_float8_weights=False, routed=False):
             x.grad = x_o.grad = None
             for lin in mods:
                 lin.weight.grad = None
-            ys = [lin(x) for lin in mods[:3]] + [mods[3](x_o)]
-            for y in ys:
-                y.backward(go)
+            ys = list(float8_projections(x, *mods[:3])) + [mods[3](x_o)]
+            torch.autograd.backward(ys, [go] * 4)
 
         f = 2.0 * m * d * d
         return fn, 12 * f, 12, f, ("config 3: OLMo-3-7B q/k/v/o projections fwd+bwd, tokens 16384, rowwise recipe "
@@ -180,9 +203,10 @@ def build_config(n, dev, keep_float8_weights=False, routed=False):
     raise ValueError(n)
 
 
-def run_other_config(n, steps, warmup, keep_float8_weights=False, routed=False):
+def measure_config(n, steps, warmup, **kw):
+    """One line for configuration n: `warmup` untimed steps, `steps` timed ones between two device synchronisations."""
     dev = torch.device("cuda:0")
-    fn, flops, _, _, desc = build_config(n, dev, keep_float8_weights, routed)
+    fn, flops, _, _, desc = build_config(n, dev, **kw)
     for _ in range(warmup):
         fn()
     torch.cuda.synchronize()
@@ -191,8 +215,30 @@ def run_other_config(n, steps, warmup, keep_float8_weights=False, routed=False):
         fn()
     torch.cuda.synchronize()
     ms = (time.perf_counter() - t0) / steps * 1e3
-    print(json.dumps({"config": desc, "ms_per_step": round(ms, 4), "TFLOP/s": round(flops / ms / 1e9, 1),
-                      "pct_fp8_mfma_peak": round(100 * flops / ms / 1e9 / FP8_MFMA_PEAK_TFLOPS, 2), "steps": steps}), flush=True)
+    del fn
+    torch.cuda.empty_cache()
+    return {"config": desc, "ms_per_step": round(ms, 4), "TFLOP/s": round(flops / ms / 1e9, 1),
+            "pct_fp8_mfma_peak": round(100 * flops / ms / 1e9 / FP8_MFMA_PEAK_TFLOPS, 2), "steps": steps}
+
+
+def run_other_config(n, steps, warmup, **kw):
+    print(json.dumps(measure_config(n, steps, warmup, **kw)), flush=True)
+
+
+def other_configs(steps=8, warmup=3):
+    """The other benchmark configurations and the headline block's other modes, one line each (a failure is reported
+    in its line and does not stop the rest)."""
+    cases = (
+        (1, {}), (3, {}), (4, {}), (5, {}), (5, {"keep_float8_weights": True}),
+        (2, {"compile_model": True}), (2, {"recommended": True}),
+    )
+    lines = []
+    for n, kw in cases:
+        try:
+            lines.append(measure_config(n, steps, warmup, **kw))
+        except Exception as e:  # noqa: BLE001
+            lines.append({"config": f"config {n} {kw}", "error": f"{type(e).__name__}: {e}"[:300]})
+    return lines
 
 
 def gemm_shapes(shapes, steps, warmup):
@@ -402,7 +448,7 @@ def feed_probe():
     for rnd in (0, 1):
         for kind, loads, reads, barriers, name in cases:
             def run():
-                _C.check(_C.lib().mi8_probe_mfma_feed(kind, loads, reads, barriers, rnd, iters, window.data_ptr(), sink.data_ptr(),
+                _C.check_diag(_C.diag().mi8_probe_mfma_feed(kind, loads, reads, barriers, rnd, iters, window.data_ptr(), sink.data_ptr(),
                                                       clocks.data_ptr(), st))
             us = _time_us(run, iters=2, warmup=1)
             cyc, ticks = (int(v) for v in clocks.tolist())
@@ -425,7 +471,7 @@ def power_probe():
     flop = 256 * 4 * iters * 2.0 * 128 ** 3
     for shape, name in ((1, "16x16x128"), (0, "32x32x64")):
         for rnd in (0, 1):
-            us = _time_us(lambda: _C.check(_C.lib().mi8_probe_mfma_loop(shape, rnd, iters, 256, sink.data_ptr(), st)), iters=3, warmup=1)
+            us = _time_us(lambda: _C.check_diag(_C.diag().mi8_probe_mfma_loop(shape, rnd, iters, 256, sink.data_ptr(), st)), iters=3, warmup=1)
             print(json.dumps({"probe": f"bare v_mfma_f32_{name}_f8f6f4 loop, 256 workgroups x 4 waves",
                               "operands": "random bytes" if rnd else "zeros", "ms": round(us / 1e3, 2),
                               "TFLOP/s": round(flop / us / 1e6, 1), "frac_of_5.0_PFLOP/s": round(flop / us / 1e6 / FP8_MFMA_PEAK_TFLOPS, 3)}), flush=True)
@@ -574,6 +620,10 @@ def main():
                     help="config 5: keep the experts' float8 weight copies across steps (micro-batch steady state)")
     ap.add_argument("--routed", action="store_true",
                     help="config 5: time the whole routed layer (fused gather, experts, weighted scatter)")
+    ap.add_argument("--compile", action="store_true", help="configs 2, 4: run the block through torch.compile")
+    ap.add_argument("--recommended", action="store_true",
+                    help="configs 2, 4: convert with AOFloat8LinearConfig.recommended() (float8 weights kept between updates)")
+    ap.add_argument("--no-other-configs", action="store_true", help="skip the other configurations after the headline")
     ap.add_argument("--cast-table", action="store_true", help="time every HBM-bound kernel of the path at the benchmark's shapes")
     ap.add_argument("--power-probe", action="store_true", help="bare MFMA loops and the GEMM on zero / random operands")
     ap.add_argument("--feed-probe", action="store_true", help="an MFMA stream with the loads and LDS reads of a GEMM K step beside it")
@@ -615,8 +665,9 @@ def main():
     if ns.gemm:
         gemm_shapes([tuple(int(v) for v in part.split(",")) for part in ns.gemm.split(";")], ns.steps, ns.warmup)
         return
-    if ns.config != 2:
-        run_other_config(ns.config, ns.steps, ns.warmup, ns.keep_float8_weights, ns.routed)
+    if ns.config != 2 or ns.compile or ns.recommended:
+        run_other_config(ns.config, ns.steps, ns.warmup, keep_float8_weights=ns.keep_float8_weights, routed=ns.routed,
+                         compile_model=ns.compile, recommended=ns.recommended)
         return
 
     dev = torch.device("cuda:0")
@@ -692,6 +743,22 @@ def main():
     }
     del mlp, x, go
     result["cast"] = cast_rates()
+    # everything of the step that is not a GEMM launch: casts, amax passes, the SwiGLU backward pass
+    n_x, n_w, n_h = TOKENS * D_MODEL, HIDDEN * D_MODEL, TOKENS * HIDDEN
+    algorithmic = 4 * (2 * n_x + 3 * n_w + n_h) + 10 * n_h  # x, grad_y, three weights, h: 2 B read + 2 copies; g1, g3: 6 read + 4 written
+    streamed = algorithmic + 2 * (2 * n_x + 3 * n_w)        # + the separate amax pass over x, grad_y and the weights
+    non_gemm_ms = ms_per_step - sum(gemm_ms) / sampled_steps
+    result["cast"]["step_totals"] = {
+        "what": "all non-GEMM work of one step (casts of x, grad_y, W1, W2, W3, h; SwiGLU backward to float8 of g1, g3; amax passes): step time minus the event-timed GEMM launches",
+        "ms": round(non_gemm_ms, 4),
+        "algorithmic_GB": round(algorithmic / 1e9, 3),
+        "streamed_GB": round(streamed / 1e9, 3),
+        "GB/s_algorithmic": round(algorithmic / non_gemm_ms / 1e6, 1),
+        "frac_hbm_peak_algorithmic": round(algorithmic / non_gemm_ms / 1e6 / HBM_PEAK_GBS, 4),
+        "frac_hbm_peak_streamed": round(streamed / non_gemm_ms / 1e6 / HBM_PEAK_GBS, 4),
+    }
+    if not ns.no_other_configs:
+        result["other_configs"] = other_configs()
     if not ns.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline()
     print(json.dumps(result), flush=True)

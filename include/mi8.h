@@ -9,7 +9,8 @@
  *     synchronises, never allocates or frees device memory, and keeps no state between calls that a caller could
  *     observe (the only memory of the library is per-device one-time set-up: a kernel's dynamic-LDS attribute and
  *     the compute-unit count, both latched with atomics, so first calls from several threads or on several
- *     devices are safe);
+ *     devices are safe).  The one exception is mi8_cast_tensorwise_static, which works in a scratch array the
+ *     library owns per GPU (see there);
  *   - requires every pointer to be 16-byte aligned device memory of at least the stated size.
  * All matrices are dense row-major with the row pitch given (or implied) in elements.
  *
@@ -121,7 +122,10 @@ int mi8_cast_tensorwise(const void* x, int hp_dtype, int64_t rows, int64_t cols,
  * caller-owned workspace.  No counterpart in the reference.  Same outputs, bytes and scale as the two-call
  * route.  Limits: rows, cols <= MI8_STATIC_CAST_MAX_DIM and rows * cols <= MI8_STATIC_CAST_MAX_ELEMS, larger
  * inputs are refused with MI8_ERR_UNSUPPORTED.  All calls on one GPU share that GPU's array: calls that may
- * overlap on one GPU (different streams, different threads) race; calls ordered on one stream do not. */
+ * overlap on one GPU (different streams, different threads, replays of two captured graphs side by side) race and
+ * nothing in the library guards against it; calls ordered on one stream do not.  The first call on a device looks
+ * up the array's address (hipGetSymbolAddress, a host-side query that is no stream operation): make one call per
+ * device outside of any stream capture before capturing calls into a graph. */
 #define MI8_STATIC_CAST_MAX_DIM ((int64_t)1 << 22)
 #define MI8_STATIC_CAST_MAX_ELEMS ((int64_t)1 << 32)
 int mi8_cast_tensorwise_static(const void* x, int hp_dtype, int64_t rows, int64_t cols, int fp8_dtype, uint32_t flags,
@@ -391,24 +395,6 @@ int mi8_moe_scatter_wgrad(const void* x, const void* grad, int dtype, int64_t to
 int mi8_moe_binned_scatter_wgrad(const void* x, const void* grad, int dtype, int64_t tokens, int64_t hidden,
                                  const int32_t* indices, const int32_t* bins, int32_t experts, int64_t capacity,
                                  int32_t top_k, void* out, void* stream);
-
-/* ---------------------------------------------------------------------------------------------
- * Diagnostics (no counterpart in the reference): `workgroups` x 4 waves issue back-to-back fp8 MFMAs on resident
- * registers, 2 * 128^3 flop per wave and iteration, shape 0 = 32x32x64, 1 = 16x16x128, on all-zero or on random
- * operand bytes.  Timed by the caller; on random operands this is the matrix throughput the chip sustains under
- * its power limit.  sink: float32 [workgroups * 256], overwritten.
- * ------------------------------------------------------------------------------------------- */
-int mi8_probe_mfma_loop(int mfma_shape, int random_operands, int iterations, int workgroups, float* sink, void* stream);
-/* What the operand feed of a GEMM K step costs a stream of MFMAs (diagnostic, no counterpart in the reference):
- * 256 workgroups of four waves run 64 16x16x128 MFMAs per iteration from resident registers and, beside them,
- * `loads` (0, 8, 16) loads of 1 KB per wave - kind 0: direct to LDS, 1: to registers, 2: LDS stores of resident
- * registers instead, 3: loads to registers and LDS stores interleaved - and `reads` (0, 32) 16-byte LDS fragment
- * reads per wave, with `barriers` (0..2) workgroup barriers per iteration.  window: at least 2 MiB + 128 KiB of
- * readable device memory; sink: 65536 floats;
- * clocks[0] = shader-clock cycles of the loop on one workgroup, clocks[1] = the same span in ticks of the constant
- * 100 MHz clock (host-visible or device memory). */
-int mi8_probe_mfma_feed(int kind, int loads, int reads, int barriers, int random_operands, int iterations, const void* window,
-                        float* sink, unsigned long long* clocks, void* stream);
 
 #ifdef __cplusplus
 }

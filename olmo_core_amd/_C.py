@@ -130,8 +130,6 @@ _SIGNATURES = {
         c_int,
         [c_void_p, c_void_p, c_int, c_int64, c_int64, c_void_p, c_void_p, c_int32, c_int64, c_int32, c_void_p, c_void_p],
     ),
-    "mi8_probe_mfma_loop": (c_int, [c_int, c_int, c_int, c_int, c_void_p, c_void_p]),
-    "mi8_probe_mfma_feed": (c_int, [c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p]),
     "mi8_grouped_padded_rows": (c_int64, [c_int64, c_int32]),
     "mi8_grouped_cast_colwise_t": (
         c_int,
@@ -176,6 +174,15 @@ _SIGNATURES = {
 
 EXPORTED_SYMBOLS = tuple(_SIGNATURES)
 
+# libmi8_diag.so (include/mi8_diag.h): measurement kernels, loaded by bench.py only
+DIAG_LIB_PATH = LIB_PATH.parent / "libmi8_diag.so"
+_DIAG_SIGNATURES = {
+    "mi8_diag_last_error": (c_char_p, []),
+    "mi8_probe_mfma_loop": (c_int, [c_int, c_int, c_int, c_int, c_void_p, c_void_p]),
+    "mi8_probe_mfma_feed": (c_int, [c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p]),
+}
+DIAG_EXPORTED_SYMBOLS = tuple(_DIAG_SIGNATURES)
+
 
 class MI8LibraryMissing(RuntimeError):
     pass
@@ -200,6 +207,30 @@ def lib() -> ctypes.CDLL:
             fn.argtypes = args
         _lib = handle
     return _lib
+
+
+_diag: Optional[ctypes.CDLL] = None
+
+
+def diag() -> ctypes.CDLL:
+    """The diagnostics library (loads on first use)."""
+    global _diag
+    if _diag is None:
+        if not DIAG_LIB_PATH.exists():
+            raise MI8LibraryMissing(f"{DIAG_LIB_PATH} is not built. Build it with `python -m olmo_core_amd.build`.")
+        handle = ctypes.CDLL(str(DIAG_LIB_PATH))
+        for name, (res, args) in _DIAG_SIGNATURES.items():
+            fn = getattr(handle, name)
+            fn.restype = res
+            fn.argtypes = args
+        _diag = handle
+    return _diag
+
+
+def check_diag(status: int, what: str = "") -> None:
+    if status != 0:
+        msg = diag().mi8_diag_last_error()
+        raise MI8KernelError(f"{what or 'libmi8_diag'}: error {status}: {msg.decode() if msg else ''}")
 
 
 def is_built() -> bool:

@@ -1,5 +1,6 @@
 """
-Build recipe for libmi8.so: plain ``hipcc`` for gfx950, no torch headers (the library has a C ABI).
+Build recipe for libmi8.so (the float8 linear path) and libmi8_diag.so (measurement kernels used by bench.py only):
+plain ``hipcc`` for gfx950, no torch headers (the libraries have a C ABI).
 
     python -m olmo_core_amd.build            # compile if sources are newer than the library
     python -m olmo_core_amd.build --force    # always compile
@@ -18,9 +19,12 @@ from pathlib import Path
 PKG_DIR = Path(__file__).resolve().parent
 CSRC = PKG_DIR / "csrc"
 LIB_PATH = PKG_DIR / "lib" / "libmi8.so"
+DIAG_LIB_PATH = PKG_DIR / "lib" / "libmi8_diag.so"
 OBJ_DIR = PKG_DIR / "lib" / "obj"
 
-SOURCES = ["mi8_api.hip", "mi8_cast.hip", "mi8_gemm.hip", "mi8_gemm_m16.hip", "mi8_gemm_skinny.hip", "mi8_pointwise.hip", "mi8_swiglu_amax.hip", "mi8_grouped.hip", "mi8_permute.hip", "mi8_probe.hip"]
+SOURCES = ["mi8_api.hip", "mi8_cast.hip", "mi8_gemm.hip", "mi8_gemm_m16.hip", "mi8_gemm_skinny.hip", "mi8_pointwise.hip", "mi8_swiglu_amax.hip", "mi8_grouped.hip", "mi8_permute.hip"]
+# the diagnostics library: the probe kernels plus the error-text / launch helpers they share with the main library
+DIAG_SOURCES = ["mi8_api.hip", "mi8_probe.hip"]
 
 HIPCC_FLAGS = [
     "--offload-arch=gfx950",
@@ -44,14 +48,15 @@ def hipcc() -> str:
 
 
 def sources() -> list[Path]:
-    return [CSRC / s for s in SOURCES if (CSRC / s).exists()]
+    names = SOURCES + [s for s in DIAG_SOURCES if s not in SOURCES]
+    return [CSRC / s for s in names if (CSRC / s).exists()]
 
 
 def is_stale() -> bool:
-    if not LIB_PATH.exists():
+    if not LIB_PATH.exists() or not DIAG_LIB_PATH.exists():
         return True
-    built = LIB_PATH.stat().st_mtime
-    deps = list(CSRC.glob("*.hip")) + list(CSRC.glob("*.h")) + [PKG_DIR.parent / "include" / "mi8.h"]
+    built = min(LIB_PATH.stat().st_mtime, DIAG_LIB_PATH.stat().st_mtime)
+    deps = list(CSRC.glob("*.hip")) + list(CSRC.glob("*.h")) + list((PKG_DIR.parent / "include").glob("*.h"))
     return any(d.stat().st_mtime > built for d in deps)
 
 
@@ -77,13 +82,14 @@ def build(force: bool = True, verbose: bool = False) -> Path:
 
     jobs = min(len(sources()), int(os.environ.get("MAX_JOBS", "8")))
     with ThreadPoolExecutor(max_workers=max(jobs, 1)) as pool:
-        objs = list(pool.map(compile_one, sources()))
-    tmp = LIB_PATH.with_suffix(".so.tmp")
-    cmd = [cc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", str(tmp), *map(str, objs)]
-    res = subprocess.run(cmd, capture_output=True, text=True)
-    if res.returncode != 0:
-        raise RuntimeError(f"link failed:\n{res.stdout}\n{res.stderr}")
-    os.replace(tmp, LIB_PATH)
+        objs = {o.stem: o for o in pool.map(compile_one, sources())}
+    for target, names in ((LIB_PATH, SOURCES), (DIAG_LIB_PATH, DIAG_SOURCES)):
+        tmp = target.with_suffix(".so.tmp")
+        cmd = [cc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", str(tmp), *(str(objs[Path(n).stem]) for n in names)]
+        res = subprocess.run(cmd, capture_output=True, text=True)
+        if res.returncode != 0:
+            raise RuntimeError(f"link of {target.name} failed:\n{res.stdout}\n{res.stderr}")
+        os.replace(tmp, target)
     return LIB_PATH
 
 

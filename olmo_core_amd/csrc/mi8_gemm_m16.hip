@@ -636,6 +636,16 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_fp8_m16_kernel(Problem pb)
     }
 }
 
+// Workgroups of a persistent launch: one per compute unit, or, for fewer tiles, as many as the tiles need - rounded
+// up to a multiple of 8, because every XCD takes an eighth of the tiles (rounded up) and needs that many workgroups
+// to finish in one round (43 tiles on 43 workgroups: XCDs with 5 workgroups for 6 tiles).
+int persistent_blocks(int max_tiles)
+{
+    const int blocks = num_compute_units();
+    const int wanted = (max_tiles + 7) / 8 * 8;
+    return blocks > wanted ? wanted : blocks;
+}
+
 // persistent: one workgroup per CU walks a static share of the tiles; otherwise one workgroup per tile, handed to
 // free CUs by the hardware dispatcher.
 template <typename Problem, int CBSZ_A, int BLGP_B>
@@ -645,12 +655,7 @@ int launch(const Problem& pb, int max_tiles, bool persistent, hipStream_t st)
     static std::atomic<uint64_t> configured{0};
     if (int rc = reserve_dynamic_lds(reinterpret_cast<const void*>(kern), LDS_BYTES, configured, "mi8 16x16x128 GEMM"))
         return rc;
-    // Persistent: one workgroup per compute unit, or, for fewer tiles, as many as the tiles need - rounded up to
-    // a multiple of 8, because every XCD takes an eighth of the tiles (rounded up) and needs that many
-    // workgroups to finish in one round (43 tiles on 43 workgroups: XCDs with 5 workgroups for 6 tiles).
-    int blocks = persistent ? num_compute_units() : max_tiles;
-    const int wanted = persistent ? (max_tiles + 7) / 8 * 8 : max_tiles;
-    if (blocks > wanted) blocks = wanted;
+    const int blocks = persistent ? persistent_blocks(max_tiles) : max_tiles;
     hipLaunchKernelGGL(kern, dim3(blocks), dim3(kThreads), LDS_BYTES, st, pb);
     return launch_status("mi8 16x16x128 GEMM");
 }
@@ -697,10 +702,7 @@ int launch_m16_swiglu(GemmArgs& g, const uint8_t* b3, const float* sb3, uint16_t
     SwigluProblem pb{g, g.lda, g.ldb, g.ldc, (int64_t)(b3 - g.B), (int64_t)(x3 - reinterpret_cast<uint16_t*>(g.C)),
                      (int64_t)(h - reinterpret_cast<uint16_t*>(g.C)), sb3, h_slots, x_codes};
     const int tiles = g.tiles_m * g.tiles_n;
-    int blocks = num_compute_units();
-    const int wanted = (tiles + 7) / 8 * 8;
-    if (blocks > wanted) blocks = wanted;
-    *n_slots = 4 * blocks;
+    *n_slots = 4 * persistent_blocks(tiles);  // one partial maximum per wave of the grid launch() forms from `tiles`
     return launch_typed(pb, tiles, true, a_dtype, b_dtype, st);
 }
 

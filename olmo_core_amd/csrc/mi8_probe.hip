@@ -1,4 +1,4 @@
-// Diagnostics: back-to-back fp8 MFMAs with nothing else running, on all-zero or on random operand registers; and the
+// Diagnostics (libmi8_diag.so, declared in include/mi8_diag.h; not part of libmi8.so): back-to-back fp8 MFMAs with nothing else running, on all-zero or on random operand registers; and the
 // same stream with the operand feed of a GEMM K step beside it (mi8_probe_mfma_feed).
 // The rate on random operands is what the chip sustains under its power limit (the clock drops under matrix load),
 // the rate on zeros what the matrix pipes do at full clock: the two numbers bracket what a GEMM can reach.
@@ -235,3 +235,6 @@ extern "C" int mi8_probe_mfma_loop(int mfma_shape, int random_operands, int iter
         hipLaunchKernelGGL((mfma_loop_kernel<1>), dim3(workgroups), dim3(256), 0, st, iterations, random_operands, sink);
     return launch_status("mi8_probe_mfma_loop");
 }
+
+extern "C" const char* mi8_last_error(void);
+extern "C" const char* mi8_diag_last_error(void) { return mi8_last_error(); }

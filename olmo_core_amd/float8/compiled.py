@@ -1,5 +1,5 @@
 """
-The float8 linear as registered custom operators, for ``torch.compile``.
+The float8 linear and the fused SwiGLU feed-forward block as registered custom operators, for ``torch.compile``.
 
 A ctypes call is opaque to Dynamo; wrapped in ``torch.library.custom_op`` with a shape function it becomes one
 node of the traced graph, so that compiled blocks (the reference compiles every transformer block,
@@ -9,7 +9,7 @@ call the same forward / backward routines as the eager ``autograd.Function``.
 
 from __future__ import annotations
 
-from typing import Optional, Tuple
+from typing import List, Optional, Tuple
 
 import torch
 
@@ -101,4 +101,91 @@ def linear(x2: torch.Tensor, weight: torch.Tensor, cfg_id: int, weight_scale: Op
     return out[0]
 
 
-__all__ = ["linear", "ops"]
+# ---- the fused SwiGLU feed-forward block (olmo_core_amd.nn.feed_forward) ------------------------------------------
+# One operator forward, one backward: a compiled transformer block keeps the launches the eager block makes (both
+# input projections and the activation in one GEMM launch, the amax of the gate gradients from row-segment codes, the
+# accumulating grad_x epilogue), bit for bit.  The forward returns y and the 13 tensors the backward takes.
+
+_N_SAVED = 13
+
+
+def _ff():
+    from ..nn import feed_forward
+
+    return feed_forward
+
+
+@torch.library.custom_op("olmo_core_amd::float8_swiglu_mlp_fwd", mutates_args=())
+def _mlp_fwd(x: torch.Tensor, w1: torch.Tensor, w2: torch.Tensor, w3: torch.Tensor, cfg: int, need_x: bool, need_w1: bool,
+             need_w2: bool, need_w3: bool) -> List[torch.Tensor]:
+    y, saved = _ff()._mlp_forward(x, w1, w2, w3, _CONFIGS[cfg], (need_x, need_w1, need_w2, need_w3))
+    return [y, *saved]
+
+
+@_mlp_fwd.register_fake
+def _(x, w1, w2, w3, cfg, need_x, need_w1, need_w2, need_w3):
+    c = _CONFIGS[cfg]
+    ff = _ff()
+    M, D = x.shape
+    H = w1.shape[0]
+    any_grad = need_x or need_w1 or need_w2 or need_w3
+    in_dt, w_dt = c.cast_config_input.target_dtype, c.cast_config_weight.target_dtype
+    pad16 = lambda n: (n + 15) // 16 * 16  # noqa: E731
+    none = lambda: x.new_empty(0)  # noqa: E731
+    f32 = lambda: x.new_empty(1, dtype=torch.float32)  # noqa: E731
+    q_t = lambda rows, cols, dt, wanted: x.new_empty((cols, pad16(rows)), dtype=dt) if wanted else none()  # noqa: E731
+    codes = none()
+    if ff._fused_launch_ok(M, D, H) and ff._use_codes(M, D, H, any_grad):
+        codes = x.new_empty(((H + 63) // 64) * M, dtype=torch.int16)
+    return [
+        x.new_empty((M, w2.shape[0])),
+        q_t(M, D, in_dt, need_w1 or need_w3), f32(), x.new_empty((M, H)), x.new_empty((M, H)),
+        q_t(M, H, in_dt, need_w2), f32(),
+        q_t(H, D, w_dt, need_x), f32(), q_t(w2.shape[0], H, w_dt, any_grad), f32(), q_t(H, D, w_dt, need_x), f32(),
+        codes,
+    ]
+
+
+@torch.library.custom_op("olmo_core_amd::float8_swiglu_mlp_bwd", mutates_args=())
+def _mlp_bwd(gy: torch.Tensor, saved: List[torch.Tensor], cfg: int, m: int, d: int, h: int, need_x: bool, need_w1: bool,
+             need_w2: bool, need_w3: bool, x_dtype: torch.dtype, w1_dtype: torch.dtype, w2_dtype: torch.dtype,
+             w3_dtype: torch.dtype) -> List[torch.Tensor]:
+    grads = _ff()._mlp_backward(gy, saved, _CONFIGS[cfg], (m, d, h), (x_dtype, w1_dtype, w2_dtype, w3_dtype),
+                                (need_x, need_w1, need_w2, need_w3))
+    return [g if g is not None else gy.new_empty(0) for g in grads]
+
+
+@_mlp_bwd.register_fake
+def _(gy, saved, cfg, m, d, h, need_x, need_w1, need_w2, need_w3, x_dtype, w1_dtype, w2_dtype, w3_dtype):
+    none = lambda: gy.new_empty(0)  # noqa: E731
+    return [
+        gy.new_empty((m, d), dtype=x_dtype) if need_x else none(),
+        gy.new_empty((h, d), dtype=w1_dtype) if need_w1 else none(),
+        gy.new_empty((d, h), dtype=w2_dtype) if need_w2 else none(),
+        gy.new_empty((h, d), dtype=w3_dtype) if need_w3 else none(),
+    ]
+
+
+def _mlp_setup_context(ctx, inputs, output):
+    x, w1, w2, w3, cfg, need_x, need_w1, need_w2, need_w3 = inputs
+    ctx.meta = (cfg, x.shape[0], x.shape[1], w1.shape[0], need_x, need_w1, need_w2, need_w3, x.dtype, w1.dtype, w2.dtype,
+                w3.dtype)
+    ctx.save_for_backward(*output[1:])
+
+
+def _mlp_backward_fn(ctx, grads):
+    need = ctx.meta[4:8]
+    gx, gw1, gw2, gw3 = _mlp_bwd(grads[0].contiguous(), list(ctx.saved_tensors), *ctx.meta)
+    pick = lambda g, wanted: g if wanted else None  # noqa: E731
+    return pick(gx, need[0]), pick(gw1, need[1]), pick(gw2, need[2]), pick(gw3, need[3]), None, None, None, None, None
+
+
+_mlp_fwd.register_autograd(_mlp_backward_fn, setup_context=_mlp_setup_context)
+
+
+def swiglu_mlp(x2: torch.Tensor, w1: torch.Tensor, w2: torch.Tensor, w3: torch.Tensor, cfg_id: int) -> torch.Tensor:
+    """The fused feed-forward block on ``x2 [M, D]`` (bfloat16) as a traceable operator call."""
+    return _mlp_fwd(x2, w1, w2, w3, cfg_id, x2.requires_grad, w1.requires_grad, w2.requires_grad, w3.requires_grad)[0]
+
+
+__all__ = ["linear", "swiglu_mlp", "ops"]

@@ -21,7 +21,6 @@ transposed copy for operands reduced along their columns.
 
 from __future__ import annotations
 
-import weakref
 from typing import Callable, Optional, Tuple
 
 import torch
@@ -30,7 +29,7 @@ import torch.nn as nn
 from . import ops
 from .native_config import CastConfig, Float8LinearConfig, ScalingGranularity, ScalingType
 
-__all__ = ["Float8Linear", "convert_to_float8_training", "float8_linear_function"]
+__all__ = ["Float8Linear", "convert_to_float8_training", "float8_linear_function", "float8_projections"]
 
 
 def _is_tensorwise(c: CastConfig) -> bool:
@@ -84,36 +83,9 @@ def _saves_quantised(c: Float8LinearConfig, need_gx: bool, need_gw: bool) -> Tup
     return x_is_q, w_is_q
 
 
-# Sibling projections applied to one tensor (q, k and v of an attention block) would each quantise it again, to the
-# same bytes and scales (the reference does: every Float8Linear casts its own input).  The operands of the last input
-# are remembered - keyed by the identity of the tensor the module was called with, its address and version counter,
-# and the cast - and dropped when that tensor dies or another input arrives.  Eager mode only.
-SHARE_INPUT_CASTS = True
-_INPUT_MEMO = None  # (weakref to the input, version, address, key, operands)
-
-
-def _drop_input_memo(_ref=None) -> None:
-    global _INPUT_MEMO
-    if _ref is None or (_INPUT_MEMO is not None and _INPUT_MEMO[0] is _ref):
-        _INPUT_MEMO = None
-
-
-def _input_operands(x2, c: Float8LinearConfig, pow2: bool, share_x: bool, origin):
+def _input_operands(x2, c: Float8LinearConfig, pow2: bool, share_x: bool):
     """``(xq, sx, x_saved)`` for the forward GEMM: the by-rows operand, its scale, and what the backward keeps."""
-    global _INPUT_MEMO
     ci = c.cast_config_input
-    src = origin[0] if origin is not None and SHARE_INPUT_CASTS and x2.is_cuda else None
-    if src is not None and torch.cuda.is_current_stream_capturing():
-        src = None  # what a graph capture allocates belongs to the graph's memory pool: nothing of it is remembered
-    key = None
-    if src is not None:
-        # (the stream is part of the key: operands made on one stream are not handed to work queued on another)
-        key = (ci.scaling_type, ci.scaling_granularity, ci.target_dtype, pow2, share_x, tuple(x2.shape), x2.dtype,
-               torch.cuda.current_stream(x2.device).cuda_stream)
-    memo = _INPUT_MEMO
-    if (src is not None and memo is not None and memo[0]() is src and memo[1] == src._version
-            and memo[2] == x2.data_ptr() and memo[3] == key):
-        return memo[4]
     x_saved = None
     if _is_tensorwise(ci):
         xq, xq_t, sx = ops.cast_tensorwise(x2, ci.target_dtype, pow2=pow2, want_rowmajor=True, want_transposed=share_x)
@@ -124,25 +96,13 @@ def _input_operands(x2, c: Float8LinearConfig, pow2: bool, share_x: bool, origin
         x_saved = (xq_t, sxc)
     else:
         xq, sx = ops.cast_rowwise(x2, ci.target_dtype, pow2=pow2)
-    res = (xq, sx, x_saved)
-    if src is not None:
-        _INPUT_MEMO = (weakref.ref(src, _drop_input_memo), src._version, x2.data_ptr(), key, res)
-    return res
+    return xq, sx, x_saved
 
 
-def _forward_impl(x2, weight, c: Float8LinearConfig, weight_scale, need_gx: bool, need_gw: bool, weight_ops=None,
-                  origin=None):
-    """y = x2 @ weight^T in float8.  Returns ``(y, x_saved, w_saved)``: the tensors the backward needs for x and
-    for the weight, each either ``(q_t, scale)`` (see :func:`_saves_quantised`) or ``None`` (keep the input).
-    ``weight_ops``: ``(q, q_t, scale)`` of the weight kept by the module (:meth:`Float8Linear.weight_operands`);
-    the weight is then not quantised here.  ``origin``: ``(tensor,)``, the tensor the module was called with (x2 is
-    a view of it), for :func:`_input_operands`."""
-    pow2 = c.round_scales_to_power_of_2
-    share_x, share_w = _saves_quantised(c, need_gx, need_gw)
+def _weight_operands(weight, c: Float8LinearConfig, pow2: bool, share_w: bool, weight_scale=None, weight_ops=None):
+    """``(wq, sw, w_saved)`` for the forward GEMM: the weight's by-rows operand, its scale(s), and what the backward
+    keeps for grad_input (``(q_t, scale)`` or ``None``: keep the weight itself)."""
     w_saved = None
-    if _is_disabled(c.cast_config_input):
-        return torch.mm(x2, weight.t().to(x2.dtype)), None, None
-    xq, sx, x_saved = _input_operands(x2, c, pow2, share_x, origin)
     if weight_ops is not None:
         wq, wq_t, sw = weight_ops
         if share_w:
@@ -159,13 +119,29 @@ def _forward_impl(x2, weight, c: Float8LinearConfig, weight_scale, need_gx: bool
         w_saved = (wq_t, swc)
     else:
         wq, sw = ops.cast_rowwise(weight, c.cast_config_weight.target_dtype, pow2=pow2)
+    return wq, sw, w_saved
+
+
+def _forward_impl(x2, weight, c: Float8LinearConfig, weight_scale, need_gx: bool, need_gw: bool, weight_ops=None):
+    """y = x2 @ weight^T in float8.  Returns ``(y, x_saved, w_saved)``: the tensors the backward needs for x and
+    for the weight, each either ``(q_t, scale)`` (see :func:`_saves_quantised`) or ``None`` (keep the input).
+    ``weight_ops``: ``(q, q_t, scale)`` of the weight kept by the module (:meth:`Float8Linear.weight_operands`);
+    the weight is then not quantised here."""
+    pow2 = c.round_scales_to_power_of_2
+    share_x, share_w = _saves_quantised(c, need_gx, need_gw)
+    if _is_disabled(c.cast_config_input):
+        return torch.mm(x2, weight.t().to(x2.dtype)), None, None
+    xq, sx, x_saved = _input_operands(x2, c, pow2, share_x)
+    wq, sw, w_saved = _weight_operands(weight, c, pow2, share_w, weight_scale, weight_ops)
     return ops.gemm_fp8(xq, sx, wq, sw, out_dtype=x2.dtype), x_saved, w_saved
 
 
 def _backward_impl(go2, c: Float8LinearConfig, N: int, x_dtype, w_dtype, x_part, w_part, x_is_q: bool, w_is_q: bool,
-                   need_gx: bool, need_gw: bool):
+                   need_gx: bool, need_gw: bool, gx_into=None):
     """grad_input and grad_weight from grad_output ``go2 [M, N]``; ``x_part`` / ``w_part`` are what the forward
-    kept: ``(q_t, scale)`` if the flag says so, else ``(tensor,)``."""
+    kept: ``(q_t, scale)`` if the flag says so, else ``(tensor,)``.  ``gx_into``: a ``[M, K]`` tensor of ``x_dtype``
+    that this linear's grad_input is added to (the bits of ``gx_into + grad_input``, formed in the GEMM's epilogue)
+    and that is returned as ``gx``."""
     pow2 = c.round_scales_to_power_of_2
     if go2.dtype != x_dtype:
         go2 = go2.to(x_dtype)
@@ -183,11 +159,14 @@ def _backward_impl(go2, c: Float8LinearConfig, N: int, x_dtype, w_dtype, x_part,
     if need_gx:
         if _is_disabled(cg):
             gx = torch.mm(go2, w_part[0].to(go2.dtype))
+            if gx_into is not None:
+                gx = gx_into.add_(gx)
         else:
             if go_rows is None:
                 go_rows = _rows_operand(go2, cg, pow2)
             w_op = (w_part[0], w_part[1]) if w_is_q else _cols_operand(w_part[0], c.cast_config_weight_for_grad_input, pow2)
-            gx = ops.gemm_fp8(go_rows[0], go_rows[1], w_op[0], w_op[1], k=N, out_dtype=x_dtype)
+            gx = ops.gemm_fp8(go_rows[0], go_rows[1], w_op[0], w_op[1], k=N, out_dtype=x_dtype, out=gx_into,
+                              accumulate=gx_into is not None)
     if need_gw:
         if _is_disabled(cgw):
             gw = torch.mm(go2.t(), x_part[0].to(go2.dtype))
@@ -206,9 +185,9 @@ class _Float8Matmul(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, x2: torch.Tensor, weight: torch.Tensor, config: Float8LinearConfig, weight_scale=None,
-                weight_ops=None, origin=None):
+                weight_ops=None):
         need_gx, need_gw = ctx.needs_input_grad[0], ctx.needs_input_grad[1]
-        y, x_saved, w_saved = _forward_impl(x2, weight, config, weight_scale, need_gx, need_gw, weight_ops, origin)
+        y, x_saved, w_saved = _forward_impl(x2, weight, config, weight_scale, need_gx, need_gw, weight_ops)
         ctx.config = config
         ctx.x_dtype, ctx.w_dtype = x2.dtype, weight.dtype
         ctx.shapes = (x2.shape[0], x2.shape[1], weight.shape[0])
@@ -230,7 +209,112 @@ class _Float8Matmul(torch.autograd.Function):
             go.reshape(M, N), ctx.config, N, ctx.x_dtype, ctx.w_dtype, saved[: ctx.n_x], saved[ctx.n_x :],
             ctx.x_is_q, ctx.w_is_q, ctx.needs_input_grad[0], ctx.needs_input_grad[1],
         )
-        return gx, gw, None, None, None, None
+        return gx, gw, None, None, None
+
+
+def _shared_input_forward(x2, weights, c: Float8LinearConfig, scales, w_ops, need_gx: bool, need_gw: bool):
+    """``ys[i] = x2 @ weights[i]^T`` with x2 quantised once.  Returns ``(ys, x_saved, w_saved)``, ``x_saved`` and each
+    ``w_saved[i]`` as :func:`_forward_impl` returns them."""
+    if _is_disabled(c.cast_config_input):
+        return [torch.mm(x2, w.t().to(x2.dtype)) for w in weights], None, [None] * len(weights)
+    pow2 = c.round_scales_to_power_of_2
+    share_x, share_w = _saves_quantised(c, need_gx, need_gw)
+    xq, sx, x_saved = _input_operands(x2, c, pow2, share_x)
+    ys, w_saved = [], []
+    for w, ws, wo in zip(weights, scales, w_ops):
+        wq, sw, kept = _weight_operands(w, c, pow2, share_w, ws, wo)
+        ys.append(ops.gemm_fp8(xq, sx, wq, sw, out_dtype=x2.dtype))
+        w_saved.append(kept)
+    return ys, x_saved, w_saved
+
+
+class _Float8SharedInputMatmul(torch.autograd.Function):
+    """``ys[i] = x @ W_i^T`` for several weights applied to ONE input (the q, k and v projections of an attention
+    block, reference src/olmo_core/nn/attention/__init__.py:582): x is quantised once by construction, one copy of
+    it is kept for all the weight gradients, and the grad_input terms are summed by the GEMM epilogues
+    (``C += product``) in the order autograd adds them - the last projection's first - so outputs and gradients carry
+    the bits of the modules applied one by one."""
+
+    @staticmethod
+    def forward(ctx, x2, config, n, *rest):
+        weights, scales, w_ops = rest[:n], rest[n:2 * n], rest[2 * n:3 * n]
+        need_gx = ctx.needs_input_grad[0]
+        need_gws = [ctx.needs_input_grad[3 + i] for i in range(n)]
+        ctx.set_materialize_grads(False)
+        ys, x_saved, w_saved = _shared_input_forward(x2, weights, config, scales, w_ops, need_gx, any(need_gws))
+        ctx.config = config
+        ctx.x_dtype, ctx.w_dtypes = x2.dtype, [w.dtype for w in weights]
+        ctx.M, ctx.ns = x2.shape[0], [w.shape[0] for w in weights]
+        ctx.x_is_q, ctx.w_is_q = x_saved is not None, [k is not None for k in w_saved]
+        ctx.need_gws = need_gws
+        to_save = []
+        if any(need_gws):
+            to_save += list(x_saved) if ctx.x_is_q else [x2]
+        ctx.n_x = len(to_save)
+        if need_gx:
+            for w, kept in zip(weights, w_saved):
+                to_save += list(kept) if kept is not None else [w]
+        ctx.save_for_backward(*to_save)
+        return tuple(ys)
+
+    @staticmethod
+    def backward(ctx, *gos):
+        n = len(ctx.ns)
+        saved = ctx.saved_tensors
+        need_gx = ctx.needs_input_grad[0]
+        x_part, pos = saved[:ctx.n_x], ctx.n_x
+        w_parts = []
+        for i in range(n):
+            k = (2 if ctx.w_is_q[i] else 1) if need_gx else 0
+            w_parts.append(saved[pos:pos + k])
+            pos += k
+        gx, gws = None, [None] * n
+        for i in reversed(range(n)):
+            if gos[i] is None:
+                continue
+            gx, gws[i] = _backward_impl(
+                gos[i].reshape(ctx.M, ctx.ns[i]), ctx.config, ctx.ns[i], ctx.x_dtype, ctx.w_dtypes[i], x_part, w_parts[i],
+                ctx.x_is_q, ctx.w_is_q[i], need_gx, ctx.need_gws[i], gx_into=gx,
+            )
+        return (gx, None, None, *gws, *([None] * (2 * n)))
+
+
+@torch.compiler.disable
+def _eager_shared_input_matmul(x2, config, weights, scales, w_ops):
+    return _Float8SharedInputMatmul.apply(x2, config, len(weights), *weights, *scales, *w_ops)
+
+
+def float8_projections(x: torch.Tensor, *modules: nn.Module) -> Tuple[torch.Tensor, ...]:
+    """``tuple(m(x) for m in modules)`` for linear modules applied to one tensor, e.g. ``q, k, v =
+    float8_projections(x, self.w_q, self.w_k, self.w_v)`` in place of the three calls at
+    src/olmo_core/nn/attention/__init__.py:582.  When every module is a :class:`Float8Linear` of one config the
+    input is quantised once for all of them and its gradient leaves the last grad_input GEMM already summed; outputs
+    and gradients have the bits of the separate calls.  Anything else (plain ``nn.Linear``, mixed configs, a traced
+    graph) is applied module by module."""
+    mods = modules
+    fusable = (
+        len(mods) > 1 and all(isinstance(m, Float8Linear) for m in mods) and x.is_cuda
+        and all(m.config is mods[0].config or m.config == mods[0].config for m in mods)
+        and all(m.in_features == x.shape[-1] for m in mods) and not torch.compiler.is_compiling()
+    )
+    if not fusable:
+        return tuple(m(x) for m in mods)
+    if torch.is_autocast_enabled():
+        x = x.to(torch.get_autocast_dtype(x.device.type))
+    c = mods[0].config
+    x2 = x.reshape(-1, x.shape[-1])
+    weights = [m.weight for m in mods]
+    scales = [m.precomputed_weight_scale() for m in mods]
+    w_ops = [m.weight_operands() for m in mods]
+    if torch.is_grad_enabled() and (x2.requires_grad or any(w.requires_grad for w in weights)):
+        ys = _eager_shared_input_matmul(x2, c, weights, scales, w_ops)
+    else:
+        ys = _shared_input_forward(x2, weights, c, scales, w_ops, False, False)[0]
+    outs = []
+    for m, y in zip(mods, ys):
+        y = y.reshape(*x.shape[:-1], m.weight.shape[0])
+        outs.append(y if m.bias is None else y + m.bias.to(y.dtype))
+    return tuple(outs)
 
 
 # Operator arguments must be plain values: under torch.compile a config travels as its index in this list.  Configs
@@ -248,8 +332,8 @@ def _register_config(c: Float8LinearConfig) -> int:
 
 
 @torch.compiler.disable
-def _eager_matmul(x2, weight, config, weight_scale, weight_ops=None, origin=None):
-    return _Float8Matmul.apply(x2, weight, config, weight_scale, weight_ops, origin)
+def _eager_matmul(x2, weight, config, weight_scale, weight_ops=None):
+    return _Float8Matmul.apply(x2, weight, config, weight_scale, weight_ops)
 
 
 def float8_linear_function(
@@ -278,9 +362,9 @@ def float8_linear_function(
         y = compiled.linear(x2, weight, cfg_id, weight_scale)
     elif not compiling and not (torch.is_grad_enabled() and (x2.requires_grad or weight.requires_grad)):
         # nothing to differentiate (evaluation, generation): no autograd node, nothing kept for a backward
-        y = _forward_impl(x2, weight, config, weight_scale, False, False, weight_ops, (x,))[0]
+        y = _forward_impl(x2, weight, config, weight_scale, False, False, weight_ops)[0]
     else:  # eager, or a config no module registered: a graph break
-        y = _eager_matmul(x2, weight, config, weight_scale, weight_ops, None if compiling else (x,))
+        y = _eager_matmul(x2, weight, config, weight_scale, weight_ops)
     return y.reshape(*x.shape[:-1], weight.shape[0])
 
 
@@ -322,6 +406,8 @@ class Float8Linear(nn.Linear):
             return None
         scale, ptr, version = entry
         w = self.weight
+        if w.is_inference():  # (inference tensors have no version counter)
+            return None
         if w.data_ptr() != ptr or w._version != version or not _is_tensorwise(self.config.cast_config_weight):
             return None
         return scale
@@ -345,7 +431,7 @@ class Float8Linear(nn.Linear):
         w = self.weight
         if not _shared_tensorwise(c.cast_config_weight, c.cast_config_weight_for_grad_input):
             return None
-        if not w.is_cuda or not w.is_contiguous() or w.dtype not in (torch.bfloat16, torch.float32):
+        if not w.is_cuda or not w.is_contiguous() or w.dtype not in (torch.bfloat16, torch.float32) or w.is_inference():
             return None
         key = (w.data_ptr(), w._version, w.dtype, tuple(w.shape))
         entry = getattr(self, "_weight_operands", None)

@@ -281,11 +281,17 @@ def gemm_fp8(
         out = torch.empty((M, N), dtype=out_dtype, device=a.device)
     elif tuple(out.shape) != (M, N) or out.dtype != out_dtype or out.stride(1) != 1 or out.device != a.device:
         raise ValueError(f"gemm_fp8: out must be a [{M}, {N}] {out_dtype} tensor with contiguous rows on {a.device}")
+    elif not out.is_inference():
+        # the kernels write through the raw pointer: tell autograd and any cache keyed on the version counter
+        torch._C._increment_version((out,))
     sink = GEMM_EVENT_SINK
     if sink is not None:
         ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         ev0.record()
     L = _C.lib()
+    if accumulate and variant < 0 and splits != 1 and L.mi8_gemm_splitk_suggest(M, N, K) > 1:
+        # few output tiles: the plain call cuts K into slices (another summation order); the sum keeps its bits
+        return out.add_(gemm_fp8(a, sa, b, sb, k=K, out_dtype=out_dtype, splits=splits))
     if accumulate:
         _C.check(
             L.mi8_gemm_fp8_accumulate(
@@ -772,6 +778,8 @@ def grouped_gemm_fp8(
         out = accumulate_into
         if tuple(out.shape) != (T, n) or out.dtype != out_dtype or out.stride(1) != 1 or out.device != a.device:
             raise ValueError(f"grouped_gemm_fp8: accumulate_into must be a [{T}, {n}] {out_dtype} tensor on {a.device}")
+        if not out.is_inference():
+            torch._C._increment_version((out,))
         fn, what = _C.lib().mi8_grouped_gemm_fp8_accumulate, "mi8_grouped_gemm_fp8_accumulate"
     else:
         out = torch.empty((T, n), dtype=out_dtype, device=a.device)

@@ -56,125 +56,149 @@ def swiglu(x1: torch.Tensor, x3: torch.Tensor) -> torch.Tensor:
     return _SwiGLU.apply(x1, x3)
 
 
+def _use_codes(M: int, D: int, H: int, any_grad: bool) -> bool:
+    """Whether the fused forward launch records the row-segment codes of x1 and x3 for the backward pass."""
+    return any_grad and SWIGLU_AMAX_FROM_CODES and H % 64 == 0
+
+
+def _fused_launch_ok(M: int, D: int, H: int) -> bool:
+    return FUSE_SWIGLU_EPILOGUE and ops.swiglu_gemm_matches_separate(M, H, D)
+
+
+def _mlp_forward(x, w1, w2, w3, c, need, ws=(None, None, None), wo=(None, None, None)):
+    """y = (silu(x W1^T) * (x W3^T)) W2^T with tensorwise float8 GEMMs; x [M, D] bf16, W1/W3 [H, D], W2 [D, H].
+    need: which of (x, w1, w2, w3) get a gradient.  ws: weight scales precomputed after the optimizer step (None: reduce
+    the amax here); wo: float8 copies the modules keep between calls (None: quantise the weight here); both in the
+    order (w1, w2, w3).  Returns ``(y, saved)``, ``saved`` being the 13 tensors :func:`_mlp_backward` takes (an empty
+    tensor where nothing is kept)."""
+    pow2 = c.round_scales_to_power_of_2
+    in_dt, w_dt = c.cast_config_input.target_dtype, c.cast_config_weight.target_dtype
+    any_grad = any(need)
+    ws1, ws2, ws3 = ws
+    wo1, wo2, wo3 = wo
+    x_codes = None
+    # The amax of x and of every weight that still needs one is taken in a single launch.
+    todo = [x] + [w for w, s, o in ((w1, ws1, wo1), (w3, ws3, wo3), (w2, ws2, wo2)) if s is None and o is None]
+    part = {}
+    if len(todo) > 1 and all(t.dtype == x.dtype and t.is_contiguous() for t in todo):
+        part = {id(t): p for t, p in zip(todo, ops.amax_partials_batch(todo))}
+    xq, xq_t, sx = ops.cast_tensorwise(x, in_dt, pow2=pow2, want_transposed=need[1] or need[3], slots=part.get(id(x)))
+    w1q, w1q_t, s1 = wo1 or ops.cast_tensorwise(w1, w_dt, pow2=pow2, want_transposed=need[0], scale=ws1,
+                                                slots=part.get(id(w1)))
+    w3q, w3q_t, s3 = wo3 or ops.cast_tensorwise(w3, w_dt, pow2=pow2, want_transposed=need[0], scale=ws3,
+                                                slots=part.get(id(w3)))
+    w2q, w2q_t, s2 = wo2 or ops.cast_tensorwise(w2, w_dt, pow2=pow2, want_transposed=any_grad, scale=ws2,
+                                                slots=part.get(id(w2)))
+    M, D, H = x.shape[0], x.shape[1], w1.shape[0]
+    if _fused_launch_ok(M, D, H):
+        # both input projections and the activation in one launch: x1 and x3 are never read back
+        if _use_codes(M, D, H, any_grad):
+            x1, x3, h, h_slots, x_codes = ops.gemm_fp8_swiglu(xq, sx, w1q, s1, w3q, s3, want_codes=True)
+        else:
+            x1, x3, h, h_slots = ops.gemm_fp8_swiglu(xq, sx, w1q, s1, w3q, s3)
+    else:
+        x1 = ops.gemm_fp8(xq, sx, w1q, s1, out_dtype=x.dtype)
+        x3 = ops.gemm_fp8(xq, sx, w3q, s3, out_dtype=x.dtype)
+        h, h_slots = ops.swiglu_fwd(x1, x3, want_amax=True)
+    if STAGE_SINK is not None:
+        STAGE_SINK.update(x1=x1.clone(), x3=x3.clone(), h=h.clone())
+    hq, hq_t, sh = ops.cast_tensorwise(h, in_dt, pow2=pow2, want_transposed=need[2], slots=h_slots)
+    if STAGE_SINK is not None:
+        STAGE_SINK.update(sh=sh.clone(), hq=hq.clone())
+    y = ops.gemm_fp8(hq, sh, w2q, s2, out_dtype=x.dtype)
+    opt = lambda t: t if t is not None else x.new_empty(0)  # noqa: E731
+    saved = (opt(xq_t), sx, x1, x3, opt(hq_t), sh, opt(w1q_t), s1, opt(w2q_t), s2, opt(w3q_t), s3, opt(x_codes))
+    return y, saved
+
+
+def _mlp_backward(gy, saved, c, dims, dtypes, need):
+    """The four gradients ``(gx, gw1, gw2, gw3)`` (``None`` where not needed) of :func:`_mlp_forward`."""
+    xq_t, sx, x1, x3, hq_t, sh, w1q_t, s1, w2q_t, s2, w3q_t, s3, x_codes = saved
+    pow2 = c.round_scales_to_power_of_2
+    go_dt = c.cast_config_grad_output.target_dtype
+    x_dt, w1_dt, w2_dt, w3_dt = dtypes
+    M, D, H = dims
+    need_x, need_w1, need_w2, need_w3 = need
+    gy = gy.reshape(M, D)
+    if gy.dtype != x_dt:
+        gy = gy.to(x_dt)
+    need_gh = need_x or need_w1 or need_w3
+    gyq, gyq_t, sgy = ops.cast_tensorwise(gy, go_dt, pow2=pow2, want_rowmajor=need_gh, want_transposed=need_w2)
+    gw2 = ops.gemm_fp8(gyq_t, sgy, hq_t, sh, out_dtype=x_dt) if need_w2 else None
+    gx = gw1 = gw3 = None
+    if need_gh:
+        # g1 and g3 are needed in fp8 only, and their tensorwise scales need the amax of both first.  Where the
+        # forward recorded the row-segment codes of x1 and x3, the GEMM that produces gh records those of gh, and the
+        # amax follows by computing a small share of the segments; otherwise a pass over the three tensors takes it.
+        codes = None
+        if x_codes.numel() and x_dt == torch.bfloat16 and ops.gemm_codes_supported(M, H, D):
+            gh, gh_codes = ops.gemm_fp8_codes(gyq, sgy, w2q_t, s2, k=D)
+            codes = (gh_codes, x_codes)
+        else:
+            gh = ops.gemm_fp8(gyq, sgy, w2q_t, s2, k=D, out_dtype=x_dt)
+        if STAGE_SINK is not None:
+            STAGE_SINK.update(gh=gh.clone())
+        need_t = need_w1 or need_w3
+        # then the recompute-and-cast pass (no bf16 round trip of g1, g3)
+        g1q, g1q_t, sg1, g3q, g3q_t, sg3 = ops.swiglu_bwd_cast(
+            x1, x3, gh, go_dt, pow2=pow2, want_rowmajor=need_x, want_transposed=need_t, codes=codes)
+        del gh
+        if STAGE_SINK is not None:
+            STAGE_SINK.update(sg1=sg1.clone(), sg3=sg3.clone(), amax_from_codes=codes is not None,
+                              g1q=None if g1q is None else g1q.clone(), g3q=None if g3q is None else g3q.clone())
+        if need_x:
+            # the sum of the two halves as autograd forms it (two bf16 tensors added), by the second GEMM's epilogue
+            gx = ops.gemm_fp8(g1q, sg1, w1q_t, s1, k=H, out_dtype=x_dt)
+            ops.gemm_fp8(g3q, sg3, w3q_t, s3, k=H, out_dtype=x_dt, out=gx, accumulate=True)
+        if need_w1:
+            gw1 = ops.gemm_fp8(g1q_t, sg1, xq_t, sx, out_dtype=x_dt)
+        if need_w3:
+            gw3 = ops.gemm_fp8(g3q_t, sg3, xq_t, sx, out_dtype=x_dt)
+
+    def as_param(g, dt):
+        return g if g is None or g.dtype == dt else g.to(dt)
+
+    return gx, as_param(gw1, w1_dt), as_param(gw2, w2_dt), as_param(gw3, w3_dt)
+
+
 class _Float8SwiGLUMLP(torch.autograd.Function):
-    """y = (silu(x W1^T) * (x W3^T)) W2^T with tensorwise float8 GEMMs; x [M, D], W1/W3 [H, D], W2 [D, H]."""
+    """The fused block as an eager autograd function (a traced graph takes the registered operators of
+    ``olmo_core_amd.float8.compiled`` instead, which run the same two routines)."""
 
     @staticmethod
     def forward(ctx, x, w1, w2, w3, config, ws1=None, ws2=None, ws3=None, wo1=None, wo2=None, wo3=None):
-        c = config
-        pow2 = c.round_scales_to_power_of_2
-        in_dt, w_dt, go_dt = (
-            c.cast_config_input.target_dtype,
-            c.cast_config_weight.target_dtype,
-            c.cast_config_grad_output.target_dtype,
-        )
-        need = ctx.needs_input_grad
-        any_grad = any(need[:4])
-        x_codes = None
-        # ws*: weight scales precomputed after the optimizer step (None: reduce the amax here);
-        # wo*: float8 copies the modules keep between calls (None: quantise the weight here)
-        # The amax of x and of every weight that still needs one is taken in a single launch.
-        todo = [x] + [w for w, ws, wo in ((w1, ws1, wo1), (w3, ws3, wo3), (w2, ws2, wo2)) if ws is None and wo is None]
-        part = {}
-        if len(todo) > 1 and all(t.dtype == x.dtype and t.is_contiguous() for t in todo):
-            part = {id(t): p for t, p in zip(todo, ops.amax_partials_batch(todo))}
-        xq, xq_t, sx = ops.cast_tensorwise(x, in_dt, pow2=pow2, want_transposed=need[1] or need[3], slots=part.get(id(x)))
-        w1q, w1q_t, s1 = wo1 or ops.cast_tensorwise(w1, w_dt, pow2=pow2, want_transposed=need[0], scale=ws1,
-                                                    slots=part.get(id(w1)))
-        w3q, w3q_t, s3 = wo3 or ops.cast_tensorwise(w3, w_dt, pow2=pow2, want_transposed=need[0], scale=ws3,
-                                                    slots=part.get(id(w3)))
-        w2q, w2q_t, s2 = wo2 or ops.cast_tensorwise(w2, w_dt, pow2=pow2, want_transposed=any_grad, scale=ws2,
-                                                    slots=part.get(id(w2)))
-        if FUSE_SWIGLU_EPILOGUE and x.dtype == torch.bfloat16 and ops.swiglu_gemm_matches_separate(x.shape[0], w1.shape[0], x.shape[1]):
-            # both input projections and the activation in one launch: x1 and x3 are never read back
-            if any_grad and SWIGLU_AMAX_FROM_CODES and w1.shape[0] % 64 == 0:
-                x1, x3, h, h_slots, x_codes = ops.gemm_fp8_swiglu(xq, sx, w1q, s1, w3q, s3, want_codes=True)
-            else:
-                x1, x3, h, h_slots = ops.gemm_fp8_swiglu(xq, sx, w1q, s1, w3q, s3)
-        else:
-            x1 = ops.gemm_fp8(xq, sx, w1q, s1, out_dtype=x.dtype)
-            x3 = ops.gemm_fp8(xq, sx, w3q, s3, out_dtype=x.dtype)
-            h, h_slots = ops.swiglu_fwd(x1, x3, want_amax=True)
-        if STAGE_SINK is not None:
-            STAGE_SINK.update(x1=x1.clone(), x3=x3.clone(), h=h.clone())
-        hq, hq_t, sh = ops.cast_tensorwise(h, in_dt, pow2=pow2, want_transposed=need[2], slots=h_slots)
-        if STAGE_SINK is not None:
-            STAGE_SINK.update(sh=sh.clone(), hq=hq.clone())
-        y = ops.gemm_fp8(hq, sh, w2q, s2, out_dtype=x.dtype)
-        ctx.config = c
-        ctx.dtypes = (x.dtype, w1.dtype, w2.dtype, w3.dtype, go_dt)
+        need = tuple(ctx.needs_input_grad[:4])
+        y, saved = _mlp_forward(x, w1, w2, w3, config, need, (ws1, ws2, ws3), (wo1, wo2, wo3))
+        ctx.config = config
+        ctx.dtypes = (x.dtype, w1.dtype, w2.dtype, w3.dtype)
         ctx.dims = (x.shape[0], x.shape[1], w1.shape[0])
-        none = x.new_empty(0)
-        ctx.save_for_backward(
-            xq_t if xq_t is not None else none, sx, x1, x3, hq_t if hq_t is not None else none, sh,
-            w1q_t if w1q_t is not None else none, s1, w2q_t if w2q_t is not None else none, s2,
-            w3q_t if w3q_t is not None else none, s3, x_codes if x_codes is not None else none,
-        )
+        ctx.save_for_backward(*saved)
         return y
 
     @staticmethod
     def backward(ctx, gy):
-        xq_t, sx, x1, x3, hq_t, sh, w1q_t, s1, w2q_t, s2, w3q_t, s3, x_codes = ctx.saved_tensors
-        c = ctx.config
-        pow2 = c.round_scales_to_power_of_2
-        x_dt, w1_dt, w2_dt, w3_dt, go_dt = ctx.dtypes
-        M, D, H = ctx.dims
-        need_x, need_w1, need_w2, need_w3 = ctx.needs_input_grad[:4]
-        gy = gy.reshape(M, D)
-        if gy.dtype != x_dt:
-            gy = gy.to(x_dt)
-        need_gh = need_x or need_w1 or need_w3
-        gyq, gyq_t, sgy = ops.cast_tensorwise(gy, go_dt, pow2=pow2, want_rowmajor=need_gh, want_transposed=need_w2)
-        gw2 = ops.gemm_fp8(gyq_t, sgy, hq_t, sh, out_dtype=x_dt) if need_w2 else None
-        gx = gw1 = gw3 = None
-        if need_gh:
-            # g1 and g3 are needed in fp8 only, and their tensorwise scales need the amax of both first.  Where the
-            # forward recorded the row-segment codes of x1 and x3, the GEMM that produces gh records those of gh, and the
-            # amax follows by computing a small share of the segments; otherwise a pass over the three tensors takes it.
-            codes = None
-            if x_codes.numel() and x_dt == torch.bfloat16 and ops.gemm_codes_supported(M, H, D):
-                gh, gh_codes = ops.gemm_fp8_codes(gyq, sgy, w2q_t, s2, k=D)
-                codes = (gh_codes, x_codes)
-            else:
-                gh = ops.gemm_fp8(gyq, sgy, w2q_t, s2, k=D, out_dtype=x_dt)
-            if STAGE_SINK is not None:
-                STAGE_SINK.update(gh=gh.clone())
-            need_t = need_w1 or need_w3
-            # then the recompute-and-cast pass (no bf16 round trip of g1, g3)
-            g1q, g1q_t, sg1, g3q, g3q_t, sg3 = ops.swiglu_bwd_cast(
-                x1, x3, gh, go_dt, pow2=pow2, want_rowmajor=need_x, want_transposed=need_t, codes=codes)
-            del gh
-            if STAGE_SINK is not None:
-                STAGE_SINK.update(sg1=sg1.clone(), sg3=sg3.clone(), amax_from_codes=codes is not None,
-                                  g1q=None if g1q is None else g1q.clone(), g3q=None if g3q is None else g3q.clone())
-            if need_x:
-                # the sum of the two halves as autograd forms it (two bf16 tensors added), by the second GEMM's epilogue
-                gx = ops.gemm_fp8(g1q, sg1, w1q_t, s1, k=H, out_dtype=x_dt)
-                ops.gemm_fp8(g3q, sg3, w3q_t, s3, k=H, out_dtype=x_dt, out=gx, accumulate=True)
-            if need_w1:
-                gw1 = ops.gemm_fp8(g1q_t, sg1, xq_t, sx, out_dtype=x_dt)
-            if need_w3:
-                gw3 = ops.gemm_fp8(g3q_t, sg3, xq_t, sx, out_dtype=x_dt)
-
-        def as_param(g, dt):
-            return g if g is None or g.dtype == dt else g.to(dt)
-
-        return (gx, as_param(gw1, w1_dt), as_param(gw2, w2_dt), as_param(gw3, w3_dt)) + (None,) * 7
+        grads = _mlp_backward(gy, ctx.saved_tensors, ctx.config, ctx.dims, ctx.dtypes, tuple(ctx.needs_input_grad[:4]))
+        return grads + (None,) * 7
 
 
-def _fusable(ff: "FeedForward", x: torch.Tensor) -> bool:
-    mods = (ff.w1, ff.w2, ff.w3)
-    if not all(isinstance(m, Float8Linear) and m.bias is None for m in mods):
+def _fusable_modules(ff: "FeedForward", same_object: bool = False) -> bool:
+    """The three projections are float8 modules of one tensorwise config without bias.  same_object: only accept one
+    shared config object (what a model conversion hands to every module), without comparing configs field by field:
+    the form a traced graph evaluates."""
+    if not ff.fuse_float8:
         return False
+    for m in (ff.w1, ff.w2, ff.w3):
+        if not isinstance(m, Float8Linear) or m.bias is not None:
+            return False
     c = ff.w1.config
-    if ff.w2.config is not c and ff.w2.config != c or ff.w3.config is not c and ff.w3.config != c:
-        return False
-    same = (
+    for m in (ff.w2, ff.w3):
+        if m.config is not c and (same_object or m.config != c):
+            return False
+    return (
         _shared_tensorwise(c.cast_config_input, c.cast_config_input_for_grad_weight)
         and _shared_tensorwise(c.cast_config_weight, c.cast_config_weight_for_grad_input)
         and _shared_tensorwise(c.cast_config_grad_output, c.cast_config_grad_output_for_grad_weight)
     )
-    return same and x.is_cuda and x.dtype == torch.bfloat16 and not torch.is_autocast_enabled()
 
 
 @torch.compiler.disable
@@ -204,9 +228,25 @@ class FeedForward(nn.Module):
         self.w3 = nn.Linear(d_model, hidden_size, bias=bias, dtype=dtype, device=init_device)
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
-        compiling = torch.compiler.is_compiling()  # traced graphs take the per-linear operators
-        if self.fuse_float8 and not compiling and _fusable(self, x):
-            x2 = x.reshape(-1, x.shape[-1])
+        # The fused block does what the three modules do one by one, including their first step under autocast (the
+        # input goes to the autocast type: src/olmo_core/train/train_module/transformer/train_module.py:593-597 runs the
+        # model that way); it takes bfloat16 activations on the GPU.
+        compiling = torch.compiler.is_compiling()
+        xa = x
+        if self.fuse_float8 and x.is_cuda and torch.is_autocast_enabled():
+            xa = x.to(torch.get_autocast_dtype("cuda"))
+        if compiling:
+            # a traced graph (the reference compiles every block, src/olmo_core/nn/transformer/block.py:78-79) keeps the
+            # fused launches: the block is one registered operator with a shape function
+            cfg_id = getattr(self.w1.config, "_compiled_id", -1) if _fusable_modules(self, same_object=True) else -1
+            if cfg_id >= 0 and xa.is_cuda and xa.dtype == torch.bfloat16:
+                from ..float8 import compiled
+
+                x2 = xa.reshape(-1, xa.shape[-1])
+                y = compiled.swiglu_mlp(x2, self.w1.weight, self.w2.weight, self.w3.weight, cfg_id)
+                return y.reshape(*x.shape[:-1], self.w2.weight.shape[0])
+        elif xa.is_cuda and xa.dtype == torch.bfloat16 and _fusable_modules(self):
+            x2 = xa.reshape(-1, xa.shape[-1])
             y = _fused_mlp(x2, self.w1.weight, self.w2.weight, self.w3.weight, self.w1.config,
                            self.w1.precomputed_weight_scale(), self.w2.precomputed_weight_scale(),
                            self.w3.precomputed_weight_scale(), self.w1.weight_operands(), self.w2.weight_operands(),

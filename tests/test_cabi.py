@@ -11,8 +11,8 @@ from olmo_core_amd import _C
 ROOT = Path(__file__).resolve().parent.parent
 
 
-def _declared_symbols():
-    text = (ROOT / "include" / "mi8.h").read_text()
+def _declared_symbols(header="mi8.h"):
+    text = (ROOT / "include" / header).read_text()
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
     return sorted(set(re.findall(r"\b(mi8_[a-z0-9_]+)\s*\(", text)))
 
@@ -26,6 +26,21 @@ def test_library_exports_every_declared_symbol():
     handle = ctypes.CDLL(str(_C.LIB_PATH))
     for name in _declared_symbols():
         assert hasattr(handle, name), f"libmi8.so does not export {name}"
+
+
+def test_diagnostics_live_in_their_own_library():
+    """The measurement kernels are no part of the drop-in boundary: mi8.h / libmi8.so do not carry them,
+    mi8_diag.h / libmi8_diag.so do."""
+    diag_syms = _declared_symbols("mi8_diag.h")
+    assert diag_syms == sorted(_C.DIAG_EXPORTED_SYMBOLS)
+    assert not set(diag_syms) & set(_declared_symbols())
+    assert _C.DIAG_LIB_PATH.exists(), "libmi8_diag.so is not built: run `python -m olmo_core_amd.build`"
+    main, diag = ctypes.CDLL(str(_C.LIB_PATH)), ctypes.CDLL(str(_C.DIAG_LIB_PATH))
+    for name in diag_syms:
+        assert hasattr(diag, name), f"libmi8_diag.so does not export {name}"
+        assert not hasattr(main, name), f"libmi8.so exports the diagnostic {name}"
+    assert _C.diag().mi8_probe_mfma_loop(7, 0, 1, 1, None, None) == -1  # argument check, nothing launched
+    assert b"sink" in _C.diag().mi8_diag_last_error()
 
 
 def test_host_only_entry_points():

@@ -297,13 +297,15 @@ def test_argument_errors(dev):
     assert rc != 0 and b"workspace" in L.mi8_last_error()
 
 
-@pytest.mark.parametrize("shape", [(512, 768, 256), (1024, 512, 1152), (300, 272, 144), (64, 512, 256), (2048, 2048, 128)],
+@pytest.mark.parametrize("shape", [(512, 768, 256), (1024, 512, 1152), (300, 272, 144), (64, 512, 256), (2048, 2048, 128),
+                                   (256, 1024, 4096), (128, 4096, 2816)],
                          ids=lambda s: "x".join(map(str, s)))
 @pytest.mark.parametrize("vec", [False, True], ids=["single-scales", "scale-vectors"])
 @pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float32], ids=["bf16", "f32"])
 def test_accumulating_gemm_equals_gemm_plus_add(dev, shape, vec, out_dtype):
     """out += product: the bits of `out + gemm(...)` on tensors of the output type (the new term rounded first, the
-    sum formed in float32 and rounded once), on the persistent kernel (full 256-tiles) and on the general one."""
+    sum formed in float32 and rounded once), on the persistent kernel (full 256-tiles), on the general one, and for
+    shapes with few tiles and a long K, which the plain call sums in slices of K (the last two shapes)."""
     M, N, K = shape
     a, b = seeded((M, K), 31, std=1e-3), seeded((N, K), 32)
     if vec:

@@ -356,21 +356,30 @@ def test_kept_weight_operands(dev, monkeypatch):
 
 
 
-@pytest.mark.parametrize("recipe", RECIPES)
-def test_sibling_projections_share_the_input_cast(dev, recipe, monkeypatch):
-    """q/k/v-style modules applied to one tensor quantise it once; outputs and gradients are the bits of modules that
-    each quantise it themselves; writing to the tensor in place, or another tensor at the same address, is seen."""
-    from olmo_core_amd.float8 import linear as L
-
-    M, K, N = 384, 256, 320
+def _projection_modules(dev, recipe, K, ns, bias_on=()):
     mods = []
-    for i in range(3):
-        lin = nn.Linear(K, N, bias=False, dtype=torch.bfloat16)
+    for i, N in enumerate(ns):
+        lin = nn.Linear(K, N, bias=i in bias_on, dtype=torch.bfloat16)
         with torch.no_grad():
             lin.weight.copy_(seeded((N, K), 40 + i, std=0.02))
+            if lin.bias is not None:
+                lin.bias.copy_(seeded((N,), 60 + i, std=0.1))
         mods.append(Float8Linear.from_float(lin.to(dev), Float8LinearConfig.from_recipe_name(recipe)))
-    gos = [seeded((M, N), 50 + i, std=1e-3).to(dev) for i in range(3)]
+    return mods
 
+
+@pytest.mark.parametrize("recipe", RECIPES)
+@pytest.mark.parametrize("shape", [(384, 256, (320, 128, 128)), (1024, 512, (512, 512, 512)), (4096, 1024, (1024, 256, 256))],
+                         ids=["small", "tiles", "gqa"])
+def test_projections_of_one_input(dev, recipe, shape, monkeypatch):
+    """float8_projections(x, w_q, w_k, w_v): the input is quantised once, and outputs, grad_x (summed by the GEMM
+    epilogues) and the weight gradients carry the bits of the three modules applied one by one and differentiated in
+    one backward call (src/olmo_core/nn/attention/__init__.py:582)."""
+    from olmo_core_amd.float8.linear import float8_projections
+
+    M, K, ns = shape
+    mods = _projection_modules(dev, recipe, K, ns, bias_on=(1,))
+    gos = [seeded((2, M // 2, N), 50 + i, std=1e-3).to(dev) for i, N in enumerate(ns)]
     calls = {"n": 0}
     for name in ("cast_tensorwise", "cast_rows_and_colwise_t", "cast_rowwise"):
         orig = getattr(ops, name)
@@ -382,62 +391,71 @@ def test_sibling_projections_share_the_input_cast(dev, recipe, monkeypatch):
 
         monkeypatch.setattr(ops, name, counted)
 
-    def run(share):
-        monkeypatch.setattr(L, "SHARE_INPUT_CASTS", share)
-        L._drop_input_memo()
+    def run(fused, used=(0, 1, 2)):
         calls["n"] = 0
-        x = seeded((M, K), 7).to(dev).requires_grad_(True)
+        x = seeded((2, M // 2, K), 7).to(dev).requires_grad_(True)
         for m in mods:
             m.weight.grad = None
-        ys = [m(x) for m in mods]
+            if m.bias is not None:
+                m.bias.grad = None
+        ys = float8_projections(x, *mods) if fused else tuple(m(x) for m in mods)
         n_fwd = calls["n"]
-        for y, go in zip(ys, gos):
-            y.backward(go)
-        return n_fwd, ys, x.grad, [m.weight.grad.clone() for m in mods]
+        torch.autograd.backward([ys[i] for i in used], [gos[i] for i in used])
+        grads = [None if m.weight.grad is None else m.weight.grad.clone() for m in mods]
+        return n_fwd, ys, x.grad, grads, mods[1].bias.grad
 
-    n1, ys1, gx1, gw1 = run(True)
-    n0, ys0, gx0, gw0 = run(False)
-    assert (n1, n0) == (1, 3)
-    assert torch.equal(gx1, gx0)
-    for a, b in zip(ys1 + gw1, ys0 + gw0):
-        assert torch.equal(a, b)
+    for used in ((0, 1, 2), (0, 2), (1,)):
+        n1, ys1, gx1, gw1, gb1 = run(True, used)
+        n0, ys0, gx0, gw0, gb0 = run(False, used)
+        assert (n1, n0) == (1, 3)
+        assert torch.equal(gx1, gx0), used
+        for a, b in zip(list(ys1) + gw1 + [gb1], list(ys0) + gw0 + [gb0]):
+            assert (a is None and b is None) or torch.equal(a, b), used
 
-    # operands made on one stream are not handed to work queued on another
-    monkeypatch.setattr(L, "SHARE_INPUT_CASTS", True)
-    L._drop_input_memo()
+    # no gradients: same outputs, one cast; frozen weights: only grad_x
     with torch.no_grad():
         xs = seeded((M, K), 11).to(dev)
         calls["n"] = 0
-        y_main = mods[0](xs)
-        side = torch.cuda.Stream()
-        side.wait_stream(torch.cuda.current_stream())
-        with torch.cuda.stream(side):
-            y_side = mods[0](xs)
-        torch.cuda.current_stream().wait_stream(side)
-        assert calls["n"] == 2 and torch.equal(y_main, y_side)
+        outs = float8_projections(xs, *mods)
+        assert calls["n"] == 1
+        for o, m in zip(outs, mods):
+            assert torch.equal(o, m(xs))
+    for m in mods:
+        m.weight.requires_grad_(False)
+    n1, ys1, gx1, gw1, _ = run(True)
+    n0, ys0, gx0, gw0, _ = run(False)
+    assert torch.equal(gx1, gx0) and all(g is None for g in gw1 + gw0)
 
-    # an in-place write invalidates the remembered operands
-    L._drop_input_memo()
+    # anything that is not a set of Float8Linear modules of one config is applied module by module
+    plain = nn.Linear(K, 64, bias=False, dtype=torch.bfloat16).to(dev)
+    outs = float8_projections(xs, mods[0], plain)
+    assert torch.equal(outs[0], mods[0](xs)) and torch.equal(outs[1], plain(xs))
+
+
+@pytest.mark.parametrize("recipe", RECIPES)
+def test_forward_under_inference_mode(dev, recipe):
+    """Generation runs under torch.inference_mode (src/olmo_core/generate/generation_module/transformer/
+    generation_module.py:135,141): inputs are inference tensors without a version counter; modules, projections and
+    the feed-forward block give the bits of the no_grad call."""
+    from olmo_core_amd.float8.linear import float8_projections
+    from olmo_core_amd.nn import FeedForward
+
+    M, K = 320, 256
+    mods = _projection_modules(dev, recipe, K, (256, 128, 128))
+    ff = FeedForward(d_model=K, hidden_size=512, bias=False, dtype=torch.bfloat16).to(dev)
+    Float8Config(ao_recipe=AOFloat8LinearRecipe(recipe)).apply_float8_linear(ff)
+    x_plain = seeded((M, K), 3).to(dev)
     with torch.no_grad():
-        x = seeded((M, K), 8).to(dev)
-        y_a = mods[0](x)
-        x.mul_(2.0)
-        y_b = mods[0](x)
-        monkeypatch.setattr(L, "SHARE_INPUT_CASTS", False)
-        assert torch.equal(y_b, mods[0](x)) and not torch.equal(y_a, y_b)
-        monkeypatch.setattr(L, "SHARE_INPUT_CASTS", True)
-        # a different tensor object (here: at the same address, the first one having died) is never taken for the old one
-        L._drop_input_memo()
-        x1 = seeded((M, K), 9).to(dev)
-        y1 = mods[1](x1)
-        ptr = x1.data_ptr()
-        del x1
-        assert L._INPUT_MEMO is None  # dropped with the tensor
-        x2 = seeded((M, K), 10).to(dev)
-        y2 = mods[1](x2)
-        monkeypatch.setattr(L, "SHARE_INPUT_CASTS", False)
-        assert torch.equal(y2, mods[1](x2))
-        assert x2.data_ptr() != ptr or not torch.equal(y1, y2)
+        want = [m(x_plain) for m in mods] + [ff(x_plain)]
+    with torch.inference_mode():
+        x = seeded((M, K), 3).to(dev)
+        assert x.is_inference()
+        got = [m(x) for m in mods] + [ff(x)]
+        fused = float8_projections(x, *mods)
+    for a, b in zip(got, want):
+        assert torch.equal(a, b)
+    for a, b in zip(fused, want[:3]):
+        assert torch.equal(a, b)
 
 
 @pytest.mark.parametrize("tokens", [16, 300], ids=["few_rows", "split_k"])

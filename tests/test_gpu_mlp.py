@@ -172,3 +172,82 @@ def test_fused_swiglu_epilogue_switch_gives_identical_block_results(dev):
             ff_mod.FUSE_SWIGLU_EPILOGUE = True
     for name, u, v in zip(("y", "gx", "gw1", "gw2", "gw3"), *res):
         assert torch.equal(u, v), name
+
+
+@pytest.mark.parametrize("mdh", [(4096, 512, 1792), (512, 256, 768)], ids=["fused_launch", "separate_launches"])
+def test_compiled_block_keeps_the_fused_function(dev, mdh):
+    """torch.compile(fullgraph=True) over a converted FeedForward (the reference compiles every transformer block,
+    src/olmo_core/nn/transformer/block.py:78-79): one graph, the block is one registered operator, and output and all
+    four gradients carry the bits of the eager fused block - the same launches run."""
+    from olmo_core_amd.nn import feed_forward as ff_mod
+
+    M, D, H = mdh
+    x = seeded((4, M // 4, D), 1).to(dev)
+    go = seeded((4, M // 4, D), 2, std=1e-3).to(dev)
+    ff = _make(dev, D, H, fuse=True)
+    ff.w3.weight.requires_grad_(False)  # a frozen projection: no gradient for it, no transposed copy of g3
+
+    def run(fn):
+        ff.zero_grad()
+        xd = x.clone().requires_grad_(True)
+        ff_mod.STAGE_SINK = sink = {}
+        try:
+            y = fn(xd)
+            y.backward(go)
+        finally:
+            ff_mod.STAGE_SINK = None
+        return sink, (y, xd.grad, ff.w1.weight.grad.clone(), ff.w2.weight.grad.clone())
+
+    sink0, eager = run(ff)
+    compiled = torch.compile(ff, fullgraph=True)
+    sink1, traced = run(compiled)
+    assert "sh" in sink0 and "sh" in sink1 and "sg1" in sink1, "the fused function did not run inside the graph"
+    assert ff.w3.weight.grad is None
+    for name, a, b in zip(("y", "gx", "gw1", "gw2"), traced, eager):
+        assert torch.equal(a, b), f"{name}: the compiled block differs from the eager fused block"
+    with torch.no_grad():
+        assert torch.equal(compiled(x), ff(x))
+    # a block that cannot run fused (a bias) still traces into one graph, through the per-linear operators
+    plain = FeedForward(d_model=D, hidden_size=H, bias=True, dtype=torch.bfloat16).to(dev)
+    Float8Config(ao_recipe=AOFloat8LinearRecipe.tensorwise).apply_float8_linear(plain)
+    y = torch.compile(plain, fullgraph=True)(x)
+    assert y.shape == x.shape
+
+
+@pytest.mark.parametrize("param_dtype", [torch.float32, torch.bfloat16], ids=["fp32_params", "bf16_params"])
+def test_fused_block_under_autocast(dev, param_dtype):
+    """The model runs under torch.autocast when autocast_precision is set
+    (src/olmo_core/train/train_module/transformer/train_module.py:593-597): the block casts its input to the autocast
+    type, as each Float8Linear does, stays fused, and gives the bits of the three modules one by one."""
+    from olmo_core_amd.nn import feed_forward as ff_mod
+
+    M, D, H = 2048, 512, 1792
+    g = torch.Generator().manual_seed(5)
+    blocks = []
+    for fuse in (True, False):
+        ff = FeedForward(d_model=D, hidden_size=H, bias=False, dtype=param_dtype, fuse_float8=fuse)
+        gg = torch.Generator().manual_seed(6)
+        with torch.no_grad():
+            for p in ff.parameters():
+                p.copy_((torch.randn(p.shape, generator=gg) * 0.02).to(param_dtype))
+        ff = ff.to(dev)
+        Float8Config(ao_recipe=AOFloat8LinearRecipe.tensorwise).apply_float8_linear(ff)
+        blocks.append(ff)
+    x = torch.randn(M, D, generator=g).to(dev)  # float32 activations, as a norm under autocast produces
+    go = (torch.randn(M, D, generator=g) * 1e-3).bfloat16().to(dev)
+    results = []
+    for ff in blocks:
+        xd = x.clone().requires_grad_(True)
+        ff_mod.STAGE_SINK = sink = {}
+        try:
+            with torch.autocast("cuda", dtype=torch.bfloat16):
+                y = ff(xd)
+            y.backward(go)
+        finally:
+            ff_mod.STAGE_SINK = None
+        results.append((sink, (y, xd.grad, ff.w1.weight.grad, ff.w2.weight.grad, ff.w3.weight.grad)))
+    assert "sh" in results[0][0] and not results[1][0], "fused block under autocast / module-by-module reference"
+    assert results[0][1][0].dtype == torch.bfloat16 and results[0][1][1].dtype == torch.float32
+    assert results[0][1][2].dtype == param_dtype
+    for name, a, b in zip(("y", "gx", "gw1", "gw2", "gw3"), results[0][1], results[1][1]):
+        assert a.dtype == b.dtype and torch.equal(a, b), f"{name}: fused and module-by-module results differ under autocast"
