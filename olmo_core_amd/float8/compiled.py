@@ -131,15 +131,16 @@ def _(x, w1, w2, w3, cfg, need_x, need_w1, need_w2, need_w3):
     any_grad = need_x or need_w1 or need_w2 or need_w3
     in_dt, w_dt = c.cast_config_input.target_dtype, c.cast_config_weight.target_dtype
     pad16 = lambda n: (n + 15) // 16 * 16  # noqa: E731
-    none = lambda: x.new_empty(0)  # noqa: E731
+    none = lambda: x.new_empty(0, dtype=torch.bfloat16)  # noqa: E731
     f32 = lambda: x.new_empty(1, dtype=torch.float32)  # noqa: E731
     q_t = lambda rows, cols, dt, wanted: x.new_empty((cols, pad16(rows)), dtype=dt) if wanted else none()  # noqa: E731
     codes = none()
     if ff._fused_launch_ok(M, D, H) and ff._use_codes(M, D, H, any_grad):
         codes = x.new_empty(((H + 63) // 64) * M, dtype=torch.int16)
+    bf16 = torch.bfloat16
     return [
-        x.new_empty((M, w2.shape[0])),
-        q_t(M, D, in_dt, need_w1 or need_w3), f32(), x.new_empty((M, H)), x.new_empty((M, H)),
+        x.new_empty((M, w2.shape[0]), dtype=bf16),
+        q_t(M, D, in_dt, need_w1 or need_w3), f32(), x.new_empty((M, H), dtype=bf16), x.new_empty((M, H), dtype=bf16),
         q_t(M, H, in_dt, need_w2), f32(),
         q_t(H, D, w_dt, need_x), f32(), q_t(w2.shape[0], H, w_dt, any_grad), f32(), q_t(H, D, w_dt, need_x), f32(),
         codes,

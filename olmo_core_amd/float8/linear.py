@@ -236,11 +236,17 @@ class _Float8SharedInputMatmul(torch.autograd.Function):
     the bits of the modules applied one by one."""
 
     @staticmethod
-    def forward(ctx, x2, config, n, *rest):
+    def forward(ctx, x2, config, n, act_dtype, *rest):
+        # act_dtype: the type the modules see their input in (the autocast type when autocast is on, else x2's own).
+        # Each module would convert x2 itself and autograd would add the converted-back grad_input terms in x2's type:
+        # that sum is formed here when the types differ.
         weights, scales, w_ops = rest[:n], rest[n:2 * n], rest[2 * n:3 * n]
         need_gx = ctx.needs_input_grad[0]
-        need_gws = [ctx.needs_input_grad[3 + i] for i in range(n)]
+        need_gws = [ctx.needs_input_grad[4 + i] for i in range(n)]
         ctx.set_materialize_grads(False)
+        ctx.gx_dtype = x2.dtype
+        if x2.dtype != act_dtype:
+            x2 = x2.to(act_dtype)
         ys, x_saved, w_saved = _shared_input_forward(x2, weights, config, scales, w_ops, need_gx, any(need_gws))
         ctx.config = config
         ctx.x_dtype, ctx.w_dtypes = x2.dtype, [w.dtype for w in weights]
@@ -269,19 +275,22 @@ class _Float8SharedInputMatmul(torch.autograd.Function):
             w_parts.append(saved[pos:pos + k])
             pos += k
         gx, gws = None, [None] * n
+        chain = ctx.gx_dtype == ctx.x_dtype  # the terms are added in the type the GEMMs write: by their epilogues
         for i in reversed(range(n)):
             if gos[i] is None:
                 continue
-            gx, gws[i] = _backward_impl(
+            term, gws[i] = _backward_impl(
                 gos[i].reshape(ctx.M, ctx.ns[i]), ctx.config, ctx.ns[i], ctx.x_dtype, ctx.w_dtypes[i], x_part, w_parts[i],
-                ctx.x_is_q, ctx.w_is_q[i], need_gx, ctx.need_gws[i], gx_into=gx,
+                ctx.x_is_q, ctx.w_is_q[i], need_gx, ctx.need_gws[i], gx_into=gx if chain else None,
             )
-        return (gx, None, None, *gws, *([None] * (2 * n)))
+            if need_gx:
+                gx = term if chain else (term.to(ctx.gx_dtype) if gx is None else gx.add_(term))
+        return (gx, None, None, None, *gws, *([None] * (2 * n)))
 
 
 @torch.compiler.disable
-def _eager_shared_input_matmul(x2, config, weights, scales, w_ops):
-    return _Float8SharedInputMatmul.apply(x2, config, len(weights), *weights, *scales, *w_ops)
+def _eager_shared_input_matmul(x2, config, act_dtype, weights, scales, w_ops):
+    return _Float8SharedInputMatmul.apply(x2, config, len(weights), act_dtype, *weights, *scales, *w_ops)
 
 
 def float8_projections(x: torch.Tensor, *modules: nn.Module) -> Tuple[torch.Tensor, ...]:
@@ -299,17 +308,16 @@ def float8_projections(x: torch.Tensor, *modules: nn.Module) -> Tuple[torch.Tens
     )
     if not fusable:
         return tuple(m(x) for m in mods)
-    if torch.is_autocast_enabled():
-        x = x.to(torch.get_autocast_dtype(x.device.type))
+    act_dtype = torch.get_autocast_dtype(x.device.type) if torch.is_autocast_enabled() else x.dtype
     c = mods[0].config
     x2 = x.reshape(-1, x.shape[-1])
     weights = [m.weight for m in mods]
     scales = [m.precomputed_weight_scale() for m in mods]
     w_ops = [m.weight_operands() for m in mods]
     if torch.is_grad_enabled() and (x2.requires_grad or any(w.requires_grad for w in weights)):
-        ys = _eager_shared_input_matmul(x2, c, weights, scales, w_ops)
+        ys = _eager_shared_input_matmul(x2, c, act_dtype, weights, scales, w_ops)
     else:
-        ys = _shared_input_forward(x2, weights, c, scales, w_ops, False, False)[0]
+        ys = _shared_input_forward(x2.to(act_dtype), weights, c, scales, w_ops, False, False)[0]
     outs = []
     for m, y in zip(mods, ys):
         y = y.reshape(*x.shape[:-1], m.weight.shape[0])

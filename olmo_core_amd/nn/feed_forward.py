@@ -66,7 +66,9 @@ def _fused_launch_ok(M: int, D: int, H: int) -> bool:
 
 
 def _mlp_forward(x, w1, w2, w3, c, need, ws=(None, None, None), wo=(None, None, None)):
-    """y = (silu(x W1^T) * (x W3^T)) W2^T with tensorwise float8 GEMMs; x [M, D] bf16, W1/W3 [H, D], W2 [D, H].
+    """y = (silu(x W1^T) * (x W3^T)) W2^T with tensorwise float8 GEMMs; x [M, D], W1/W3 [H, D], W2 [D, H].  x is
+    converted to bfloat16 first if it is of another type (float32 activations under autocast: each of the three
+    modules would convert its own input).
     need: which of (x, w1, w2, w3) get a gradient.  ws: weight scales precomputed after the optimizer step (None: reduce
     the amax here); wo: float8 copies the modules keep between calls (None: quantise the weight here); both in the
     order (w1, w2, w3).  Returns ``(y, saved)``, ``saved`` being the 13 tensors :func:`_mlp_backward` takes (an empty
@@ -77,6 +79,8 @@ def _mlp_forward(x, w1, w2, w3, c, need, ws=(None, None, None), wo=(None, None, 
     ws1, ws2, ws3 = ws
     wo1, wo2, wo3 = wo
     x_codes = None
+    if x.dtype != torch.bfloat16:
+        x = x.to(torch.bfloat16)
     # The amax of x and of every weight that still needs one is taken in a single launch.
     todo = [x] + [w for w, s, o in ((w1, ws1, wo1), (w3, ws3, wo3), (w2, ws2, wo2)) if s is None and o is None]
     part = {}
@@ -112,11 +116,15 @@ def _mlp_forward(x, w1, w2, w3, c, need, ws=(None, None, None), wo=(None, None, 
 
 
 def _mlp_backward(gy, saved, c, dims, dtypes, need):
-    """The four gradients ``(gx, gw1, gw2, gw3)`` (``None`` where not needed) of :func:`_mlp_forward`."""
+    """The four gradients ``(gx, gw1, gw2, gw3)`` (``None`` where not needed) of :func:`_mlp_forward`.  dtypes: of the
+    x the forward was given and of the three weights.  For a bfloat16 x the two grad_x terms are added by the second
+    GEMM's epilogue; for an x of another type they are added in that type, as autograd adds the converted-back
+    gradients of the two modules that each converted x."""
     xq_t, sx, x1, x3, hq_t, sh, w1q_t, s1, w2q_t, s2, w3q_t, s3, x_codes = saved
     pow2 = c.round_scales_to_power_of_2
     go_dt = c.cast_config_grad_output.target_dtype
-    x_dt, w1_dt, w2_dt, w3_dt = dtypes
+    gx_dt, w1_dt, w2_dt, w3_dt = dtypes
+    x_dt = torch.bfloat16
     M, D, H = dims
     need_x, need_w1, need_w2, need_w3 = need
     gy = gy.reshape(M, D)
@@ -146,10 +154,14 @@ def _mlp_backward(gy, saved, c, dims, dtypes, need):
         if STAGE_SINK is not None:
             STAGE_SINK.update(sg1=sg1.clone(), sg3=sg3.clone(), amax_from_codes=codes is not None,
                               g1q=None if g1q is None else g1q.clone(), g3q=None if g3q is None else g3q.clone())
-        if need_x:
+        if need_x and gx_dt == x_dt:
             # the sum of the two halves as autograd forms it (two bf16 tensors added), by the second GEMM's epilogue
             gx = ops.gemm_fp8(g1q, sg1, w1q_t, s1, k=H, out_dtype=x_dt)
             ops.gemm_fp8(g3q, sg3, w3q_t, s3, k=H, out_dtype=x_dt, out=gx, accumulate=True)
+        elif need_x:
+            # (autograd runs w3's backward first: its term is the one the other is added to)
+            gx = ops.gemm_fp8(g3q, sg3, w3q_t, s3, k=H, out_dtype=x_dt).to(gx_dt)
+            gx.add_(ops.gemm_fp8(g1q, sg1, w1q_t, s1, k=H, out_dtype=x_dt))
         if need_w1:
             gw1 = ops.gemm_fp8(g1q_t, sg1, xq_t, sx, out_dtype=x_dt)
         if need_w3:
@@ -232,20 +244,19 @@ class FeedForward(nn.Module):
         # input goes to the autocast type: src/olmo_core/train/train_module/transformer/train_module.py:593-597 runs the
         # model that way); it takes bfloat16 activations on the GPU.
         compiling = torch.compiler.is_compiling()
-        xa = x
-        if self.fuse_float8 and x.is_cuda and torch.is_autocast_enabled():
-            xa = x.to(torch.get_autocast_dtype("cuda"))
+        act_dtype = torch.get_autocast_dtype("cuda") if x.is_cuda and torch.is_autocast_enabled() else x.dtype
+        xa = x  # (the conversion to the autocast type happens inside the fused function)
         if compiling:
             # a traced graph (the reference compiles every block, src/olmo_core/nn/transformer/block.py:78-79) keeps the
             # fused launches: the block is one registered operator with a shape function
             cfg_id = getattr(self.w1.config, "_compiled_id", -1) if _fusable_modules(self, same_object=True) else -1
-            if cfg_id >= 0 and xa.is_cuda and xa.dtype == torch.bfloat16:
+            if cfg_id >= 0 and xa.is_cuda and act_dtype == torch.bfloat16:
                 from ..float8 import compiled
 
                 x2 = xa.reshape(-1, xa.shape[-1])
                 y = compiled.swiglu_mlp(x2, self.w1.weight, self.w2.weight, self.w3.weight, cfg_id)
                 return y.reshape(*x.shape[:-1], self.w2.weight.shape[0])
-        elif xa.is_cuda and xa.dtype == torch.bfloat16 and _fusable_modules(self):
+        elif xa.is_cuda and act_dtype == torch.bfloat16 and _fusable_modules(self):
             x2 = xa.reshape(-1, xa.shape[-1])
             y = _fused_mlp(x2, self.w1.weight, self.w2.weight, self.w3.weight, self.w1.config,
                            self.w1.precomputed_weight_scale(), self.w2.precomputed_weight_scale(),

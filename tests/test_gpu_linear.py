@@ -432,6 +432,31 @@ def test_projections_of_one_input(dev, recipe, shape, monkeypatch):
     assert torch.equal(outs[0], mods[0](xs)) and torch.equal(outs[1], plain(xs))
 
 
+@pytest.mark.parametrize("recipe", ["tensorwise", "rowwise"])
+def test_projections_under_autocast(dev, recipe):
+    """Float32 activations under autocast: every module converts its own input, so autograd adds the three grad_input
+    terms after converting each back to float32; float8_projections forms that same sum."""
+    from olmo_core_amd.float8.linear import float8_projections
+
+    M, K = 512, 256
+    mods = _projection_modules(dev, recipe, K, (256, 128, 128))
+    for m in mods:
+        m.float()
+    gos = [seeded((M, N), 50 + i, std=1e-3).to(dev) for i, N in enumerate((256, 128, 128))]
+    out = []
+    for fused in (True, False):
+        x = seeded((M, K), 7, dtype=torch.float32).to(dev).requires_grad_(True)
+        for m in mods:
+            m.weight.grad = None
+        with torch.autocast("cuda", dtype=torch.bfloat16):
+            ys = float8_projections(x, *mods) if fused else tuple(m(x) for m in mods)
+        torch.autograd.backward(ys, gos)
+        out.append(list(ys) + [x.grad] + [m.weight.grad.clone() for m in mods])
+    assert out[0][3].dtype == torch.float32 and out[0][0].dtype == torch.bfloat16 and out[0][4].dtype == torch.float32
+    for a, b in zip(*out):
+        assert a.dtype == b.dtype and torch.equal(a, b)
+
+
 @pytest.mark.parametrize("recipe", RECIPES)
 def test_forward_under_inference_mode(dev, recipe):
     """Generation runs under torch.inference_mode (src/olmo_core/generate/generation_module/transformer/
