@@ -563,6 +563,73 @@ def counter_summary(path):
     print("(kernels shorter than 5 us are left out)")
 
 
+def gemm_compare(shapes, reps=4):
+    """Workload for counter runs that put this library's GEMM beside hipBLASLt's (through torch._scaled_mm) on the same
+    operands: per shape, on all-zero and on N(0,1) operands, `reps` calls of each (the first of each is a warm-up).
+    Under `rocprofv3 --kernel-trace [--pmc ...] --output-format csv`, --counter-cases prints one row per case from the
+    dispatch order; without a profiler the calls are timed with events."""
+    from olmo_core_amd.float8 import ops
+
+    dev = torch.device("cuda:0")
+    one = torch.ones(1, device=dev)
+    e4m3 = torch.float8_e4m3fn
+    for (m, n, k) in shapes:
+        for rnd in (0, 1):
+            if rnd:
+                a = torch.randn(m, k, device=dev).to(e4m3)
+                b = torch.randn(n, k, device=dev).to(e4m3)
+            else:
+                a = torch.zeros(m, k, device=dev, dtype=e4m3)
+                b = torch.zeros(n, k, device=dev, dtype=e4m3)
+            torch.cuda.synchronize()
+            for name, fn in (("mi8_gemm_fp8", lambda: ops.gemm_fp8(a, one, b, one)),
+                             ("hipBLASLt (torch._scaled_mm)", lambda: torch._scaled_mm(a, b.t(), scale_a=one, scale_b=one, out_dtype=torch.bfloat16))):
+                us = _time_us(fn, iters=reps - 1, warmup=1)
+                print(json.dumps({"case": f"{m}x{n}x{k} {'random' if rnd else 'zeros'} {name}", "calls": reps, "us": round(us, 1),
+                                  "TFLOP/s": round(2.0 * m * n * k / us / 1e6, 1)}), flush=True)
+            del a, b
+
+
+def counter_cases(path, group=4):
+    """The GEMM dispatches of a --gemm-compare run in dispatch order, `group` consecutive dispatches of one kernel per
+    case (the first of each group is the warm-up and is left out): kernel, mean duration and mean of every counter."""
+    import csv
+    import glob
+    from collections import OrderedDict
+
+    files = [path] if os.path.isfile(path) else sorted(glob.glob(os.path.join(path, "**", "*counter_collection.csv"), recursive=True))
+    trace = None
+    if not files:
+        files = sorted(glob.glob(os.path.join(path, "**", "*kernel_trace.csv"), recursive=True))
+        trace = True
+    if not files:
+        print(f"no *counter_collection.csv or *kernel_trace.csv under {path}", file=sys.stderr)
+        sys.exit(2)
+    disp = OrderedDict()
+    for r in csv.DictReader(open(files[0])):
+        name = " ".join(r["Kernel_Name"].split())
+        if "gemm_fp8" not in name and "Cijk" not in name:
+            continue
+        d = disp.setdefault(int(r["Dispatch_Id"]), {"name": name, "us": (int(r["End_Timestamp"]) - int(r["Start_Timestamp"])) / 1e3, "c": {}})
+        if not trace:
+            d["c"][r["Counter_Name"]] = d["c"].get(r["Counter_Name"], 0.0) + float(r["Counter_Value"])
+    rows = [disp[k] for k in sorted(disp)]
+    counters = sorted({c for d in rows for c in d["c"]})
+    print(f"{'#':>3s} {'kernel':44s} {'us':>8s} " + " ".join(f"{c[:22]:>22s}" for c in counters))
+    i = case = 0
+    while i < len(rows):
+        j = i
+        while j < len(rows) and j - i < group and rows[j]["name"] == rows[i]["name"]:
+            j += 1
+        use = rows[i + 1:j] if j - i > 1 else rows[i:j]
+        name = rows[i]["name"].replace("(anonymous namespace)::", "").replace("mi8::gemm::", "").replace("void ", "")
+        us = sum(d["us"] for d in use) / len(use)
+        vals = " ".join(f"{sum(d['c'].get(c, 0.0) for d in use) / len(use):22.0f}" for c in counters)
+        print(f"{case:3d} {name[:44]:44s} {us:8.1f} {vals}")
+        case += 1
+        i = j
+
+
 def step(mlp, x, go):
     x.grad = None
     for p in mlp.parameters():
@@ -632,6 +699,10 @@ def main():
     ap.add_argument("--counter-summary", type=str, default=None, metavar="DIR_OR_CSV",
                     help="print per-kernel means of a rocprofv3 --pmc --output-format csv run (no GPU needed)")
     ap.add_argument("--traffic-probe", action="store_true", help="workload for the rocprofv3 --pmc counter runs (a calibration copy, then three benchmark steps)")
+    ap.add_argument("--gemm-compare", type=str, default=None, metavar="M,N,K[;M,N,K...]",
+                    help="this library's GEMM and hipBLASLt's on the same zero / random operands (workload for counter runs)")
+    ap.add_argument("--counter-cases", type=str, default=None, metavar="DIR_OR_CSV",
+                    help="per-case table of a rocprofv3 run of --gemm-compare (no GPU needed)")
     ap.add_argument("--gemm", type=str, default=None, metavar="M,N,K[;M,N,K...]",
                     help="time single scaled GEMMs of these shapes (library's choice of kernel) instead of a step")
     ns = ap.parse_args()
@@ -640,6 +711,9 @@ def main():
         return
     if ns.counter_summary:
         counter_summary(ns.counter_summary)
+        return
+    if ns.counter_cases:
+        counter_cases(ns.counter_cases)
         return
     if ns.gpus != 1:
         print("bench.py: this build measures the float8 linear path on ONE GPU; --gpus must be 1", file=sys.stderr)
@@ -661,6 +735,9 @@ def main():
         return
     if ns.power_probe:
         power_probe()
+        return
+    if ns.gemm_compare:
+        gemm_compare([tuple(int(v) for v in part.split(",")) for part in ns.gemm_compare.split(";")])
         return
     if ns.gemm:
         gemm_shapes([tuple(int(v) for v in part.split(",")) for part in ns.gemm.split(";")], ns.steps, ns.warmup)

@@ -274,6 +274,23 @@ int mi8_grouped_gemm_fp8_accumulate(const void* a, int a_dtype, int64_t lda, con
                                     int64_t N, int64_t K, const float* sa, const float* sb, int64_t sb_group_stride,
                                     void* out, int out_dtype, int64_t ldc, void* stream);
 
+/* out[rows of group e, :N] = (a1 . B1_e^T) / sa1 / sb1_e + (a2 . B2_e^T) / sa2 / sb2_e, both products summed in one
+ * float32 accumulation and rounded once to bf16: the grad_input of an expert layer whose input feeds two projections
+ * (gx = g1 . W1 + g2 . W3, src/olmo_core/nn/moe/mlp.py:272-292 in backward) as one launch instead of
+ * mi8_grouped_gemm_fp8 + mi8_grouped_gemm_fp8_accumulate, without the read-modify-write of the output.  a1 [T, K1] and
+ * a2 [T, K2] share the row pitch lda; B1_e [N, K1] and B2_e [N, K2] the row pitch ldb and the group stride; sa1, sa2:
+ * float32 [T]; sb1, sb2: float32, group e at + e * sb_group_stride, N values.  EVERY SCALE MUST BE AN EXACT POWER OF TWO
+ * (what the casts write under MI8_FLAG_POW2_SCALE): the scales are applied inside the matrix instructions as exponents,
+ * a mantissa is ignored.  The sum differs from the two-call route by one rounding (that route rounds each product to bf16
+ * before adding).  Shapes: mi8_grouped_gemm_fp8_dual_supported (T, N >= 256, N % 8 == 0, K1 and K2 multiples of 256);
+ * out: bf16 [T, ldc], ldc % 8 == 0. */
+int mi8_grouped_gemm_fp8_dual_supported(int64_t T, int64_t N, int64_t K1, int64_t K2);
+int mi8_grouped_gemm_fp8_dual(const void* a1, const void* a2, int a_dtype, int64_t lda, const void* b1, const void* b2,
+                              int b_dtype, int64_t ldb, int64_t b_group_stride, const int64_t* group_sizes,
+                              int32_t num_groups, int64_t T, int64_t N, int64_t K1, int64_t K2, const float* sa1,
+                              const float* sa2, const float* sb1, const float* sb2, int64_t sb_group_stride, void* out,
+                              int64_t ldc, void* stream);
+
 /* out[e, :N, :Kl] = (A_t[:N, S_e] . B_t[:Kl, S_e]^T) / sa[e, n] / sb[e, k]: the contraction runs over group e's
  * 128-aligned segment S_e of the padded token axis (layout written by mi8_grouped_cast_colwise_t; both operands
  * have pitch ld_t).  Empty groups produce zeros.  out is [num_groups, N, Kl] contiguous. */

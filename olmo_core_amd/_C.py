@@ -165,6 +165,12 @@ _SIGNATURES = {
         [c_void_p, c_int, c_int64, c_void_p, c_int, c_int64, c_int64, c_void_p, c_int32, c_int64, c_int64, c_int64,
          c_void_p, c_void_p, c_int64, c_void_p, c_int, c_int64, c_void_p],
     ),
+    "mi8_grouped_gemm_fp8_dual_supported": (c_int, [c_int64, c_int64, c_int64, c_int64]),
+    "mi8_grouped_gemm_fp8_dual": (
+        c_int,
+        [c_void_p, c_void_p, c_int, c_int64, c_void_p, c_void_p, c_int, c_int64, c_int64, c_void_p, c_int32, c_int64, c_int64,
+         c_int64, c_int64, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_void_p, c_int64, c_void_p],
+    ),
     "mi8_grouped_wgrad_fp8": (
         c_int,
         [c_void_p, c_int, c_void_p, c_int, c_int64, c_void_p, c_int32, c_int64, c_int64, c_int64, c_void_p, c_void_p,

@@ -109,6 +109,12 @@ int launch_m16_grouped(const uint8_t* a, int a_dtype, int64_t lda, const uint8_t
                        int64_t b_group_stride, const int64_t* sizes, int E, int64_t T, int N, int K, const float* sa,
                        const float* sb, int64_t sb_group_stride, uint16_t* out, int64_t ldc, bool accumulate,
                        hipStream_t st);
+// out[rows of e] = A1 . B1_e^T + A2 . B2_e^T in one accumulation (power-of-two scale vectors, applied inside the
+// MFMAs); T, N >= 256, K1, K2 multiples of 256
+int launch_m16_grouped_dual(const uint8_t* a1, const uint8_t* a2, int a_dtype, int64_t lda, const uint8_t* b1,
+                            const uint8_t* b2, int b_dtype, int64_t ldb, int64_t b_group_stride, const int64_t* sizes, int E,
+                            int64_t T, int N, int K1, int K2, const float* sa1, const float* sa2, const float* sb1,
+                            const float* sb2, int64_t sb_group_stride, uint16_t* out, int64_t ldc, hipStream_t st);
 int launch_m16_grouped_wgrad(const uint8_t* a_t, int a_dtype, const uint8_t* b_t, int b_dtype, int64_t ld_t,
                              const int64_t* sizes, int E, int64_t T, int N, int Kl, const float* sa, const float* sb,
                              uint16_t* out, hipStream_t st);

@@ -134,6 +134,10 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_fp8_m16_kernel(Problem pb)
     // waits and barriers of the K steps in between make them visible before the tile's epilogue.  Slots are
     // counted over tiles that have K steps (the cursor skips the others, however many): the cursor is at most
     // two steps, hence two such tiles, ahead of the epilogue that reads a slot.
+    // (two-segment problems: a slot holds the four scale vectors of a tile, and two slots are enough - a tile has at
+    // least four K steps, so the load cursor is never more than one tile ahead of the tile whose slot is still read)
+    constexpr int kSlotBytes = Problem::kTwoSegments ? 2 * SCALE_SLOT : SCALE_SLOT;
+    constexpr int kSlotMask = Problem::kTwoSegments ? 1 : SCALE_SLOTS - 1;
     float inv_single = 1.0f;
     if constexpr (Problem::kSwiglu) {
         // The fused problem has two multipliers (x1, x3) and a running maximum of |h| per lane.  They live in the
@@ -151,9 +155,13 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_fp8_m16_kernel(Problem pb)
     int ld_seq = 0, cp_seq = 0;  // tiles with K steps seen by the load cursor / by the epilogue
     auto scale_dma = [&](const TileDesc& d) __attribute__((always_inline)) {
         if constexpr (Problem::kVecScales) {
-            uint8_t* slot = lds + 2 * STAGE + OUT_STAGING + (ld_seq & (SCALE_SLOTS - 1)) * SCALE_SLOT + wave * 256;
+            uint8_t* slot = lds + 2 * STAGE + OUT_STAGING + (ld_seq & kSlotMask) * kSlotBytes + wave * 256;
             __builtin_amdgcn_global_load_lds((gptr_t)(d.sa + wave * 64 + lane), (lptr_t)slot, 4, 0, 0);
             __builtin_amdgcn_global_load_lds((gptr_t)(d.sb + wave * 64 + lane), (lptr_t)(slot + 1024), 4, 0, 0);
+            if constexpr (Problem::kTwoSegments) {
+                __builtin_amdgcn_global_load_lds((gptr_t)(d.sa2 + wave * 64 + lane), (lptr_t)(slot + 2048), 4, 0, 0);
+                __builtin_amdgcn_global_load_lds((gptr_t)(d.sb2 + wave * 64 + lane), (lptr_t)(slot + 3072), 4, 0, 0);
+            }
         }
         ++ld_seq;
     };
@@ -197,6 +205,10 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_fp8_m16_kernel(Problem pb)
     int ld_tile = -1, ld_kt = 0, ld_nk = 0;
     const uint8_t* ld_a = nullptr;
     const uint8_t* ld_b = nullptr;
+    // (two-segment problems) where the cursor continues after step ld_nk1 - 1 of the tile
+    int ld_nk1 = 0;
+    const uint8_t* ld_a2 = nullptr;
+    const uint8_t* ld_b2 = nullptr;
     auto next_load_tile = [&]() __attribute__((always_inline)) {
         while (ld_tile + 1 < my_tiles) {
             ++ld_tile;
@@ -206,20 +218,32 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_fp8_m16_kernel(Problem pb)
                 ld_b = d.b + b_wave_shift;
                 ld_nk = d.nk;
                 ld_kt = 0;
+                if constexpr (Problem::kTwoSegments) {
+                    ld_nk1 = d.nk1;
+                    ld_a2 = d.a2;
+                    ld_b2 = d.b2;
+                }
                 scale_dma(d);
                 return;
             }
         }
-        if (ld_a) {  // no further tile with work: rewind to the start of the current one
-            ld_a -= (int64_t)ld_kt * BK;
-            ld_b -= (int64_t)ld_kt * BK;
-            ld_kt = 0;
+        if (ld_a) {  // no further tile with work: rewind to the start of the current one (of its current segment)
+            const int back = Problem::kTwoSegments ? ld_kt - ld_nk1 : ld_kt;
+            ld_a -= (int64_t)back * BK;
+            ld_b -= (int64_t)back * BK;
+            ld_kt -= back;
         }
     };
     auto advance_load_cursor = [&]() __attribute__((always_inline)) {
         ++ld_kt;
         ld_a += BK;
         ld_b += BK;
+        if constexpr (Problem::kTwoSegments) {
+            if (ld_kt == ld_nk1) {  // (uniform) the first pair of operands is used up
+                ld_a = ld_a2;
+                ld_b = ld_b2;
+            }
+        }
         if (ld_kt >= ld_nk) next_load_tile();
     };
     next_load_tile();
@@ -228,11 +252,45 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_fp8_m16_kernel(Problem pb)
     // D' = B . A^T : the first MFMA operand is the B fragment (its type code goes to cbsz).  `fresh`: the tile's
     // first touch of this accumulator; the MFMA then takes the constant 0 as its addend, so the accumulators
     // never have to be cleared between tiles.
-    auto mma = [&](const v4i (&a)[2], const v4i (&b)[2], v4f& c, bool fresh) __attribute__((always_inline)) {
+    // kMfmaScale: power-of-two scale vectors are applied inside the MFMAs as block scales - an exponent byte per
+    // operand row, 2^(byte - 127), the same for a row's four 32-byte K blocks; the bytes of four tiles share a register
+    // and the instruction selects one (ia, jb: the A and B tile of the wave tile).  Scaling every product of an output
+    // element by one power of two scales every partial sum alike: the bits are those of scaling the finished sum.
+    int ea_lo = 0, ea_hi = 0, eb_lo = 0, eb_hi = 0;
+    bool ms_tile = false;  // (wave-uniform) this tile's scales are applied by the MFMAs: the epilogue does not multiply
+    auto mma = [&](const v4i (&a)[2], const v4i (&b)[2], v4f& c, bool fresh, int ia, int jb) __attribute__((always_inline)) {
         const v8i fa = __builtin_shufflevector(a[0], a[1], 0, 1, 2, 3, 4, 5, 6, 7);
         const v8i fb = __builtin_shufflevector(b[0], b[1], 0, 1, 2, 3, 4, 5, 6, 7);
         const v4f zero = {0, 0, 0, 0};
-        c = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(fb, fa, fresh ? zero : c, BLGP_B, CBSZ_A, 0, 0, 0, 0);
+        if constexpr (Problem::kMfmaScale) {
+            // Written as instructions of their own with the accumulator tied to the result: left to the register
+            // allocator, a share of the scaled MFMAs do not accumulate in place, and with all 256 accumulator registers
+            // in use the moves that follow end in spills.  (op_sel / op_sel_hi: bits 0 / 1 of the byte each scale
+            // register is read at; first the B fragment's, which is the instruction's first matrix operand.)
+            const int sca = ia < 4 ? ea_lo : ea_hi, scb = jb < 4 ? eb_lo : eb_hi;
+#define MI8_MS_ASM(JB, IA)                                                                                                  \
+    case JB * 4 + IA:                                                                                                      \
+        if (fresh)                                                                                                         \
+            asm volatile("v_mfma_scale_f32_16x16x128_f8f6f4 %0, %1, %2, 0, %3, %4 op_sel:[" #JB "&1," #IA "&1,0] "        \
+                         "op_sel_hi:[" #JB ">>1," #IA ">>1,0] cbsz:%5 blgp:%6"                                             \
+                         : "=a"(c)                                                                                         \
+                         : "v"(fb), "v"(fa), "v"(scb), "v"(sca), "n"(BLGP_B), "n"(CBSZ_A));                                \
+        else                                                                                                               \
+            asm volatile("v_mfma_scale_f32_16x16x128_f8f6f4 %0, %1, %2, %0, %3, %4 op_sel:[" #JB "&1," #IA "&1,0] "       \
+                         "op_sel_hi:[" #JB ">>1," #IA ">>1,0] cbsz:%5 blgp:%6"                                             \
+                         : "+a"(c)                                                                                         \
+                         : "v"(fb), "v"(fa), "v"(scb), "v"(sca), "n"(BLGP_B), "n"(CBSZ_A));                                \
+        break;
+            switch ((jb & 3) * 4 + (ia & 3)) {
+                MI8_MS_ASM(0, 0) MI8_MS_ASM(0, 1) MI8_MS_ASM(0, 2) MI8_MS_ASM(0, 3)
+                MI8_MS_ASM(1, 0) MI8_MS_ASM(1, 1) MI8_MS_ASM(1, 2) MI8_MS_ASM(1, 3)
+                MI8_MS_ASM(2, 0) MI8_MS_ASM(2, 1) MI8_MS_ASM(2, 2) MI8_MS_ASM(2, 3)
+                MI8_MS_ASM(3, 0) MI8_MS_ASM(3, 1) MI8_MS_ASM(3, 2) MI8_MS_ASM(3, 3)
+            }
+#undef MI8_MS_ASM
+        } else {
+            c = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(fb, fa, fresh ? zero : c, BLGP_B, CBSZ_A, 0, 0, 0, 0);
+        }
     };
 
     // ---- prologue: stages of steps 0 and 1, fragments of step 0 ----------------------------------------
@@ -268,6 +326,37 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_fp8_m16_kernel(Problem pb)
     for (int cp_tile = 0; cp_tile < my_tiles; ++cp_tile) {
         const TileDesc td = my_tile(cp_tile);
         if (td.c == nullptr) continue;  // (uniform) a grid slot without a tile
+        // (kMfmaScale) The tile's scale vectors are in its LDS slot by now (fetched when the load cursor reached the tile,
+        // at least two K steps - each with a wait that covers them and a barrier - ago).  Every scale of the wave's 128
+        // rows and 128 columns a normal power of two: their inverses go into the MFMAs as exponent bytes.  Anything
+        // else (a mantissa, zero, infinity, NaN): the MFMAs run unscaled (byte 127) and the epilogue multiplies.
+        // Two-segment problems have no such way out (two sets of scales meet in one accumulator): they read every
+        // scale as the power of two its exponent field names.  seg: which pair of vectors of the slot.
+        auto load_exponents = [&](int seg) __attribute__((always_inline)) {
+            ms_tile = Problem::kTwoSegments;
+            ea_lo = ea_hi = eb_lo = eb_hi = 0x7F7F7F7F;
+            if (td.nk > 0) {  // (uniform)
+                const uint8_t* slot = lds + 2 * STAGE + OUT_STAGING + (cp_seq & kSlotMask) * kSlotBytes + seg * 2048;
+                uint32_t pa[2] = {0, 0}, pq[2] = {0, 0}, other = 0;
+#pragma unroll
+                for (int t = 0; t < NT; ++t) {
+                    const uint32_t ua = *reinterpret_cast<const uint32_t*>(slot + (wm * WT + 16 * t + r16) * 4);
+                    const uint32_t ub = *reinterpret_cast<const uint32_t*>(slot + 1024 + (wn * WT + 16 * t + r16) * 4);
+                    pa[t >> 2] |= ((254u - (ua >> 23)) & 0xFFu) << (8 * (t & 3));  // 1 / 2^k as an exponent byte
+                    pq[t >> 2] |= ((254u - (ub >> 23)) & 0xFFu) << (8 * (t & 3));
+                    other |= (ua & 0x7FFFFFu) | (ub & 0x7FFFFFu);
+                    other |= (uint32_t)((ua >> 23) - 1u > 253u) | (uint32_t)((ub >> 23) - 1u > 253u);
+                }
+                if constexpr (!Problem::kTwoSegments) ms_tile = __builtin_amdgcn_ballot_w64(other != 0) == 0;
+                if (ms_tile) {
+                    ea_lo = (int)pa[0];
+                    ea_hi = (int)pa[1];
+                    eb_lo = (int)pq[0];
+                    eb_hi = (int)pq[1];
+                }
+            }
+        };
+        if constexpr (Problem::kMfmaScale) load_exponents(0);
         // One 128-byte K step.  `fresh`: the tile's first step; phase A touches the accumulators of A tiles 0-3,
         // phase B those of A tiles 4-7, so both start from 0 then.  The first step is written out separately
         // from the loop, not as a branch inside it.
@@ -286,7 +375,7 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_fp8_m16_kernel(Problem pb)
 #pragma unroll
             for (int x = 0; x < 32; ++x) {
                 const int j = x >> 2, i = x & 3;
-                mma(fa_lo[i], fb[S][j], acc[i][j], fresh);
+                mma(fa_lo[i], fb[S][j], acc[i][j], fresh, i, j);
                 if (x < 8) read_a(fa_hi[x >> 1], 4 + (x >> 1), x & 1);
                 if (x >= 8 && x % 3 == 2) dma_one(ld_a, ld_b, cur, kLoads + (x - 8) / 3);
                 __builtin_amdgcn_sched_barrier(0);
@@ -314,7 +403,7 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_fp8_m16_kernel(Problem pb)
 #pragma unroll
             for (int x = 0; x < 32; ++x) {
                 const int j = x >> 2, i = x & 3;
-                mma(fa_hi[i], fb[S][j], acc[4 + i][j], fresh);
+                mma(fa_hi[i], fb[S][j], acc[4 + i][j], fresh, 4 + i, j);
                 if (x < 16) read_b(fb[S ^ 1][x >> 1], x >> 1, x & 1);
                 if (x >= 16 && x < 24) read_a(fa_lo[(x - 16) >> 1], (x - 16) >> 1, x & 1);
                 if (i == 1) dma_one(ld_a, ld_b, cur, x >> 2);
@@ -328,6 +417,17 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_fp8_m16_kernel(Problem pb)
             // tile is read again after the epilogue, into set 0
             const std::integral_constant<int, 0> set0;
             const std::integral_constant<int, 1> set1;
+            if constexpr (Problem::kTwoSegments) {
+                // both segments have an even number of steps: the switch to the second pair's scales falls between
+                // two pairs of steps (the fragments of step nk1 were read from the second pair's bytes already)
+                k_step(true, set0);
+                k_step(false, set1);
+                for (int kt = 2; kt < td.nk; kt += 2) {
+                    if (kt == td.nk1) load_exponents(1);
+                    k_step(false, set0);
+                    k_step(false, set1);
+                }
+            } else {
             k_step(true, set0);
             int kt = 1;
             for (; kt + 1 < td.nk; kt += 2) {
@@ -335,6 +435,7 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_fp8_m16_kernel(Problem pb)
                 k_step(false, set0);
             }
             if (kt < td.nk) k_step(false, set1);
+            }
         } else {  // nothing is accumulated (empty group): the tile is all zeros
 #pragma unroll
             for (int i = 0; i < NT; ++i)
@@ -353,7 +454,7 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_fp8_m16_kernel(Problem pb)
         uint8_t* stg = lds + 2 * STAGE + wave * 4096;
         const uint32_t stg_lds = (uint32_t)(uintptr_t)(lptr_t)stg;
         const bool zero_tile = td.nk == 0;  // nothing accumulated; the scales may be unset
-        const uint8_t* sc_slot = lds + 2 * STAGE + OUT_STAGING + (cp_seq & (SCALE_SLOTS - 1)) * SCALE_SLOT;
+        const uint8_t* sc_slot = lds + 2 * STAGE + OUT_STAGING + (cp_seq & kSlotMask) * kSlotBytes;
         if (!zero_tile) ++cp_seq;
         const int ldc_bytes = (int)pb.ldc * 2;
         const uint32_t c_lane_off = (uint32_t)((lane >> 3) * ldc_bytes + (lane & 7) * 16);
@@ -536,10 +637,13 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_fp8_m16_kernel(Problem pb)
                 asm volatile("ds_max_u32 %0, %1" ::"v"(maddr), "v"(hmax) : "memory");
             }
         } else {
+        // no_mul: the scales were applied inside the MFMAs (kMfmaScale problems, decided per tile)
+        auto passes = [&](auto no_mul) __attribute__((always_inline)) {
+        constexpr bool kNoMul = decltype(no_mul)::value;
 #pragma unroll
         for (int jq = 0; jq < 2; ++jq) {
             float isb[4][4];
-            if constexpr (Problem::kVecScales) {
+            if constexpr (Problem::kVecScales && !kNoMul) {
 #pragma unroll
                 for (int jj = 0; jj < 4; ++jj) {
                     const float4 s4 =
@@ -559,11 +663,13 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_fp8_m16_kernel(Problem pb)
                     // A single scale is made opaque in every pass: with a loop-invariant multiplier the compiler
                     // forms the products of the whole tile up front and spills accumulators.
                     float mult = inv_single;
-                    if constexpr (Problem::kVecScales)
+                    if constexpr (kNoMul)
+                        mult = 1.0f;
+                    else if constexpr (Problem::kVecScales)
                         mult = __builtin_amdgcn_rcpf(*reinterpret_cast<const float*>(sc_slot + (rt + 16 * t + r16) * 4));
                     else
                         asm volatile("" : "+v"(mult));
-                    mult = zero_tile ? 0.0f : mult;
+                    if constexpr (!kNoMul) mult = zero_tile ? 0.0f : mult;
 #pragma unroll
                     for (int jj = 0; jj < 4; ++jj) {
                         float v[4];
@@ -574,8 +680,12 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_fp8_m16_kernel(Problem pb)
                             // the top of the epilogue and the kernel spills.
                             float a_;
                             asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(a_) : "a"(acc[2 * ih + t][4 * jq + jj][e]));
-                            v[e] = a_ * mult;
-                            if constexpr (Problem::kVecScales) v[e] *= isb[jj][e];
+                            if constexpr (kNoMul) {
+                                v[e] = a_;
+                            } else {
+                                v[e] = a_ * mult;
+                                if constexpr (Problem::kVecScales) v[e] *= isb[jj][e];
+                            }
                         }
                         o[t][jj].x = pack_bf16x2(v[0], v[1]);
                         o[t][jj].y = pack_bf16x2(v[2], v[3]);
@@ -619,6 +729,17 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_fp8_m16_kernel(Problem pb)
         if constexpr (Problem::kAccumulate) add_held();
         record_codes(7);
         store_staged(1, 3);
+        };
+        if constexpr (Problem::kTwoSegments) {
+            passes(std::true_type{});
+        } else if constexpr (Problem::kMfmaScale) {
+            if (ms_tile)
+                passes(std::true_type{});
+            else
+                passes(std::false_type{});
+        } else {
+            passes(std::false_type{});
+        }
         }
         // The last step's phase B has read the next tile's first fragments like any other step; reading them
         // again here makes those 96 registers free during the epilogue, which otherwise spills (and every
@@ -719,6 +840,19 @@ int launch_m16_grouped(const uint8_t* a, int a_dtype, int64_t lda, const uint8_t
         return launch_typed(pb, max_tiles, true, a_dtype, b_dtype, st);
     }
     GroupedProblem<false> pb{a, b, out, lda, ldb, ldc, b_group_stride, sb_group_stride, sizes, E, T, N, K, tiles_n, sa, sb};
+    return launch_typed(pb, max_tiles, true, a_dtype, b_dtype, st);
+}
+
+int launch_m16_grouped_dual(const uint8_t* a1, const uint8_t* a2, int a_dtype, int64_t lda, const uint8_t* b1,
+                            const uint8_t* b2, int b_dtype, int64_t ldb, int64_t b_group_stride, const int64_t* sizes, int E,
+                            int64_t T, int N, int K1, int K2, const float* sa1, const float* sa2, const float* sb1,
+                            const float* sb2, int64_t sb_group_stride, uint16_t* out, int64_t ldc, hipStream_t st)
+{
+    const int tiles_n = (N + BN - 1) / BN;
+    const int64_t max_tiles64 = ((T + BM - 1) / BM + E) * tiles_n;
+    const int max_tiles = max_tiles64 > (1 << 30) ? (1 << 30) : (int)max_tiles64;
+    GroupedDualProblem pb{{a1, b1, out, lda, ldb, ldc, b_group_stride, sb_group_stride, sizes, E, T, N, K1, tiles_n, sa1, sb1},
+                          lda, ldb, ldc, a2, b2, sa2, sb2, K2};
     return launch_typed(pb, max_tiles, true, a_dtype, b_dtype, st);
 }
 

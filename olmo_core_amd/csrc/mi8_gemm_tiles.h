@@ -21,6 +21,13 @@ struct TileDesc {
     uint16_t* c;       // C element (first row, first column) of the tile; null: the slot holds no tile
     int row_lo, row_hi;  // rows [row_lo, row_hi) of the 256 are stored
     int m0, n0;          // (problems that record row-segment codes) first row and column of the tile
+    // (two-segment problems) the contraction continues, after nk1 steps, over a second pair of operands with scales
+    // of their own
+    const uint8_t* a2;
+    const uint8_t* b2;
+    const float* sa2;
+    const float* sb2;
+    int nk1;
 };
 
 struct NoCache {};
@@ -38,7 +45,7 @@ struct DenseProblem {
     static constexpr bool kVecScales = VEC;  // both scales are vectors (per row / per column) or both single
     static constexpr bool kAccumulate = ACC;  // C += the rounded product
     static constexpr bool kOutCodes = CODES;
-    static constexpr bool kSwiglu = false;
+    static constexpr bool kSwiglu = false, kMfmaScale = false, kTwoSegments = false;
     static constexpr bool kMaskRows = false, kXcdRanges = true;
     using Cache = NoCache;
     __device__ __forceinline__ Cache prepare() const { return Cache{}; }
@@ -82,7 +89,7 @@ struct SwigluProblem {
     uint32_t* h_slots;      // [4 * workgroups] partial maxima of |h| (float32 bit patterns)
     uint16_t* x_codes;      // null, or [H / 64][M] codes of the larger of x1 and x3 per row segment (H % 64 == 0)
     static constexpr bool kVecScales = false, kAccumulate = false, kSwiglu = true, kOutCodes = false;
-    static constexpr bool kMaskRows = false, kXcdRanges = true;
+    static constexpr bool kMaskRows = false, kXcdRanges = true, kMfmaScale = false, kTwoSegments = false;
     using Cache = NoCache;
     __device__ __forceinline__ Cache prepare() const { return Cache{}; }
     __device__ __forceinline__ int total_tiles(const Cache&) const { return g.tiles_m * g.tiles_n; }
@@ -162,10 +169,13 @@ __device__ __forceinline__ GroupSpan locate_group_cached(const GroupCache& c, co
 // Ragged-M grouped problem (dropless-MoE forward / grad_input): rows of A form consecutive groups, group e
 // multiplies B_e = B + e * b_group_stride.  A tile covers up to 256 rows of ONE group; it always loads a full
 // 256-row window (shifted back at the end of the matrix, T >= 256) and stores only its group's rows.
+// Scale vectors that are exact powers of two (the axiswise recipes round theirs) are applied inside the MFMAs as block
+// scales (kMfmaScale): with K of one or two thousand the vector-scale epilogue - two multiplications per element on a
+// wave that has its SIMD to itself - is a third to a half of a tile's time, and this takes the multiplications out.
 template <bool ACC = false>
 struct GroupedProblem {
     static constexpr bool kAccumulate = ACC;
-    static constexpr bool kSwiglu = false, kOutCodes = false;
+    static constexpr bool kSwiglu = false, kOutCodes = false, kMfmaScale = true, kTwoSegments = false;
     const uint8_t* A;
     const uint8_t* B;
     uint16_t* C;
@@ -207,6 +217,40 @@ struct GroupedProblem {
     }
 };
 
+// The sum of two ragged-M grouped products in one accumulation (the grad_input of an expert layer whose input feeds
+// two projections: gx = g1 . W1 + g2 . W3): out[rows of e] = A1 . B1_e^T + A2 . B2_e^T, a contraction over K1 + K2 whose
+// load cursor moves from the first pair of operands to the second after K1 / 128 steps.  The two products carry
+// different scales per row and per column, all exact powers of two (the scale vectors are read as such: only their
+// exponents are used), applied inside the MFMAs - so both terms meet in one float32 accumulator and are rounded once:
+// no second launch, no read-modify-write of the output.  A1, A2 share a row pitch, B1, B2 a row pitch and group stride,
+// the column scales a group stride; K1, K2 are multiples of 256 (an even number of steps each).
+struct GroupedDualProblem {
+    static constexpr bool kAccumulate = false, kSwiglu = false, kOutCodes = false, kMfmaScale = true, kTwoSegments = true;
+    static constexpr bool kVecScales = true, kMaskRows = true, kXcdRanges = true;
+    GroupedProblem<false> first;  // A1, B1, C, pitches, sizes, N, K = K1, sa1, sb1
+    int64_t lda, ldb, ldc;        // (copies of first's, under the names the kernel reads)
+    const uint8_t* A2;
+    const uint8_t* B2;
+    const float* sa2;
+    const float* sb2;
+    int K2;
+    using Cache = GroupCache;
+    __device__ __forceinline__ Cache prepare() const { return first.prepare(); }
+    __device__ __forceinline__ int total_tiles(const Cache& c) const { return first.total_tiles(c); }
+    __device__ __forceinline__ TileDesc tile(int t, const Cache& c) const
+    {
+        TileDesc d = first.tile(t, c);
+        // the same window of rows, columns and group in the second pair of operands
+        d.a2 = A2 + (d.a - first.A);
+        d.b2 = B2 + (d.b - first.B);
+        d.sa2 = sa2 + (d.sa - first.sa);
+        d.sb2 = sb2 + (d.sb - first.sb);
+        d.nk1 = d.nk;
+        d.nk = d.nk1 + K2 / BK;
+        return d;
+    }
+};
+
 // Ragged-K grouped problem (dropless-MoE grad_weight): out[e] = A_t[:, S_e] . B_t[:, S_e]^T over group e's
 // 128-aligned segment S_e of the padded token axis; N, Kl >= 256.  An empty group gives nk = 0: its tiles are
 // written as zeros and its scales (never produced) are ignored.
@@ -236,7 +280,7 @@ struct GroupedWgradProblem {
     const float* sa;  // [E, N]
     const float* sb;  // [E, Kl]
     static constexpr bool kVecScales = true, kMaskRows = false, kXcdRanges = false;
-    static constexpr bool kAccumulate = false, kSwiglu = false, kOutCodes = false;
+    static constexpr bool kAccumulate = false, kSwiglu = false, kOutCodes = false, kMfmaScale = false, kTwoSegments = false;
     using Cache = WgradCache;
     __device__ __forceinline__ Cache prepare() const
     {

@@ -225,6 +225,45 @@ extern "C" int mi8_grouped_gemm_fp8_accumulate(const void* a, int a_dtype, int64
                               sb_group_stride, out, out_dtype, ldc, true, stream);
 }
 
+extern "C" int mi8_grouped_gemm_fp8_dual_supported(int64_t T, int64_t N, int64_t K1, int64_t K2)
+{
+    return (T >= 256 && T < (1 << 30) && N >= 256 && N % 8 == 0 && N < (1 << 30) && K1 >= 256 && K2 >= 256 && K1 % 256 == 0 &&
+            K2 % 256 == 0 && K1 < (1 << 30) && K2 < (1 << 30))
+               ? 1
+               : 0;
+}
+
+extern "C" int mi8_grouped_gemm_fp8_dual(const void* a1, const void* a2, int a_dtype, int64_t lda, const void* b1,
+                                         const void* b2, int b_dtype, int64_t ldb, int64_t b_group_stride,
+                                         const int64_t* group_sizes, int32_t num_groups, int64_t T, int64_t N, int64_t K1,
+                                         int64_t K2, const float* sa1, const float* sa2, const float* sb1, const float* sb2,
+                                         int64_t sb_group_stride, void* out, int64_t ldc, void* stream)
+{
+    MI8_REQUIRE(a1 && a2 && b1 && b2 && group_sizes && sa1 && sa2 && sb1 && sb2 && out, MI8_ERR_ARG,
+                "mi8_grouped_gemm_fp8_dual: null pointer");
+    MI8_REQUIRE(fp8_code(a_dtype) && fp8_code(b_dtype), MI8_ERR_ARG, "mi8_grouped_gemm_fp8_dual: unknown fp8 dtype");
+    MI8_REQUIRE(num_groups > 0, MI8_ERR_ARG, "mi8_grouped_gemm_fp8_dual: no groups");
+    MI8_REQUIRE(mi8_grouped_gemm_fp8_dual_supported(T, N, K1, K2), MI8_ERR_UNSUPPORTED,
+                "mi8_grouped_gemm_fp8_dual: needs T, N >= 256, N %% 8 == 0 and K1, K2 multiples of 256 (got T=%lld N=%lld K1=%lld "
+                "K2=%lld); use mi8_grouped_gemm_fp8 and mi8_grouped_gemm_fp8_accumulate",
+                (long long)T, (long long)N, (long long)K1, (long long)K2);
+    const int64_t kmax = K1 > K2 ? K1 : K2;
+    MI8_REQUIRE(lda % 16 == 0 && ldb % 16 == 0 && lda >= kmax && ldb >= kmax && b_group_stride % 16 == 0 && lda < (1 << 23) &&
+                    ldb < (1 << 23),
+                MI8_ERR_UNSUPPORTED, "mi8_grouped_gemm_fp8_dual: lda, ldb and the group stride must be multiples of 16, lda, ldb >= K1, K2 and below 2^23");
+    MI8_REQUIRE(ldc >= N && ldc % 8 == 0 && ldc < (1 << 22) && aligned16(out), MI8_ERR_UNSUPPORTED,
+                "mi8_grouped_gemm_fp8_dual: the output needs ldc >= N, ldc %% 8 == 0 and 16-byte alignment");
+    MI8_REQUIRE(aligned16(a1) && aligned16(a2) && aligned16(b1) && aligned16(b2) && aligned16(sb1) && aligned16(sb2) &&
+                    sb_group_stride % 4 == 0,
+                MI8_ERR_UNSUPPORTED, "mi8_grouped_gemm_fp8_dual: operands and column scales must be 16-byte aligned");
+    MI8_REQUIRE(N * ldb < ((int64_t)1 << 32), MI8_ERR_UNSUPPORTED, "mi8_grouped_gemm_fp8_dual: operand too large");
+    const int64_t m_tiles = ceil_div(T, 256) + num_groups;
+    MI8_REQUIRE(m_tiles * ceil_div(N, 256) < ((int64_t)1 << 30), MI8_ERR_UNSUPPORTED, "mi8_grouped_gemm_fp8_dual: grid too large");
+    return launch_m16_grouped_dual((const uint8_t*)a1, (const uint8_t*)a2, a_dtype, lda, (const uint8_t*)b1, (const uint8_t*)b2,
+                                   b_dtype, ldb, b_group_stride, group_sizes, num_groups, T, (int)N, (int)K1, (int)K2, sa1, sa2,
+                                   sb1, sb2, sb_group_stride, (uint16_t*)out, ldc, (hipStream_t)stream);
+}
+
 extern "C" int mi8_grouped_wgrad_fp8(const void* a_t, int a_dtype, const void* b_t, int b_dtype, int64_t ld_t,
                                      const int64_t* group_sizes, int32_t num_groups, int64_t T, int64_t N, int64_t Kl,
                                      const float* sa, const float* sb, void* out, int out_dtype, void* stream)

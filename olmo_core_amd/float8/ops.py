@@ -795,6 +795,44 @@ def grouped_gemm_fp8(
     return out
 
 
+def grouped_gemm_dual_supported(T: int, n: int, k1: int, k2: int) -> bool:
+    """Shapes :func:`grouped_gemm_fp8_dual` takes."""
+    return bool(_C.lib().mi8_grouped_gemm_fp8_dual_supported(T, n, k1, k2))
+
+
+def grouped_gemm_fp8_dual(
+    a1: torch.Tensor, sa1: torch.Tensor, b1: torch.Tensor, sb1: torch.Tensor,
+    a2: torch.Tensor, sa2: torch.Tensor, b2: torch.Tensor, sb2: torch.Tensor,
+    group_sizes: torch.Tensor, *, n: int, k1: int, k2: int, b_group_stride: int, sb_group_stride: int,
+) -> torch.Tensor:
+    """
+    ``out[rows of group e] = a1 @ B1_e.T / sa1 / sb1_e + a2 @ B2_e.T / sa2 / sb2_e`` (bf16), both products in one
+    float32 accumulation: one launch in place of :func:`grouped_gemm_fp8` followed by its accumulating form.  All scales
+    must be exact powers of two (casts made with ``pow2=True``).  ``a1`` / ``a2`` and ``b1`` / ``b2`` must share their
+    row pitches; ``B_e`` starts ``e * b_group_stride`` bytes into ``b``, its scales ``e * sb_group_stride`` floats into
+    ``sb``.
+    """
+    _require_gpu(a1, "grouped_gemm_fp8_dual")
+    T = a1.shape[0]
+    if a2.shape[0] != T or a1.stride(0) != a2.stride(0) or b1.stride(0) != b2.stride(0) or a1.dtype != a2.dtype or b1.dtype != b2.dtype:
+        raise ValueError("grouped_gemm_fp8_dual: the two left operands and the two right operands must share rows, pitch and type")
+    if a1.stride(1) != 1 or a2.stride(1) != 1 or b1.stride(1) != 1 or b2.stride(1) != 1:
+        raise ValueError("grouped_gemm_fp8_dual: operands must have contiguous rows")
+    if sa1.numel() != T or sa2.numel() != T or sb1.shape != sb2.shape:
+        raise ValueError("grouped_gemm_fp8_dual: one scale per row of a1 / a2, column scales of one shape")
+    sizes = _sizes_i64(group_sizes, a1.device)
+    out = torch.empty((T, n), dtype=torch.bfloat16, device=a1.device)
+    _C.check(
+        _C.lib().mi8_grouped_gemm_fp8_dual(
+            a1.data_ptr(), a2.data_ptr(), _FP8_CODE[a1.dtype], a1.stride(0), b1.data_ptr(), b2.data_ptr(), _FP8_CODE[b1.dtype],
+            b1.stride(0), b_group_stride, sizes.data_ptr(), sizes.numel(), T, n, k1, k2, sa1.data_ptr(), sa2.data_ptr(),
+            sb1.data_ptr(), sb2.data_ptr(), sb_group_stride, out.data_ptr(), out.stride(0), _stream(a1),
+        ),
+        "mi8_grouped_gemm_fp8_dual",
+    )
+    return out
+
+
 def grouped_wgrad_fp8(
     a_t: torch.Tensor,
     sa: torch.Tensor,

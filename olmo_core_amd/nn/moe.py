@@ -28,6 +28,11 @@ _E4M3 = torch.float8_e4m3fn
 # there, so that a checker can feed each stage's actual input to a reference of that stage.
 STAGE_SINK = None
 
+# The grad_input of the expert layer (the sum of the gate and up projections' terms) as one grouped GEMM over both
+# contractions where the shape allows; False: two launches, the second adding into the first one's output (each term
+# rounded to bf16 before the sum).
+DUAL_GRAD_INPUT = True
+
 
 class _Float8DroplessMLP(torch.autograd.Function):
     @staticmethod
@@ -165,7 +170,12 @@ class _Float8DroplessMLP(torch.autograd.Function):
             g1q, sg1, g1t, sg1c = both(g1, need_x, need_w1, amax1)
             g2q, sg2, g2t, sg2c = both(g2, need_x, need_w3, amax2)
             del g1, g2
-            if need_x:
+            if need_x and DUAL_GRAD_INPUT and pow2 and ops.grouped_gemm_dual_supported(T, D, H, H):
+                # gx_e = g1_e @ w1[e] + g2_e @ w3[e] as ONE contraction over 2 H: the scales of both products (powers of
+                # two) are applied inside the matrix instructions, so the terms meet in one float32 accumulator
+                gx = ops.grouped_gemm_fp8_dual(g1q, sg1, w1t, s1c, g2q, sg2, w3t, s3c, sizes, n=D, k1=H, k2=H,
+                                               b_group_stride=Hp, sb_group_stride=D)
+            elif need_x:
                 # gx_e = g_e @ w[e] : contraction over H, the right operand is w[e]^T [D, H], one scale per input channel
                 gx = ops.grouped_gemm_fp8(g1q, sg1, w1t, s1c, sizes, n=D, k=H, b_group_stride=Hp, sb_group_stride=D)
                 ops.grouped_gemm_fp8(g2q, sg2, w3t, s3c, sizes, n=D, k=H, b_group_stride=Hp, sb_group_stride=D,

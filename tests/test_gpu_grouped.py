@@ -440,3 +440,80 @@ def test_kept_expert_weight_operands(dev):
     assert kept.weight_operands() is not first
     for a, b in zip(run(plain), run(kept)):
         assert torch.equal(a, b)
+
+
+DUAL_SIZE_CASES = [[300, 17, 0, 411, 64], [256], [1, 0, 0, 255, 513], [0, 1000, 0], [5] * 70, [700, 1, 0, 323, 2048, 9]]
+
+
+@pytest.mark.parametrize("sizes", DUAL_SIZE_CASES, ids=lambda s: "-".join(map(str, s[:6])))
+@pytest.mark.parametrize("n,k1,k2", [(256, 256, 256), (320, 512, 256), (512, 256, 1024)])
+def test_grouped_dual_gemm_exact_integers(dev, sizes, n, k1, k2):
+    """out = a1 . B1_e^T / sa1 / sb1_e + a2 . B2_e^T / sa2 / sb2_e in one accumulation.  Small-integer operands and
+    power-of-two scales (different for the two products, per row and per column): every partial sum is exact in
+    float32, so the result must equal the float64 evaluation rounded once to bf16 - any wrong operand window, scale
+    vector, group or segment switch changes an integer."""
+    E, T = len(sizes), sum(sizes)
+    g = torch.Generator().manual_seed(16)
+    a1 = torch.randint(-2, 3, (T, k1), generator=g).float()
+    a2 = torch.randint(-2, 3, (T, k2), generator=g).float()
+    w1 = torch.randint(-2, 3, (E, n, k1), generator=g).float()
+    w2 = torch.randint(-2, 3, (E, n, k2), generator=g).float()
+    pick = lambda vals, count, seed: torch.tensor(vals)[torch.randint(0, len(vals), (count,), generator=torch.Generator().manual_seed(seed))]  # noqa: E731
+    sa1, sa2 = pick([1.0, 2.0, 0.5, 4.0, 64.0], T, 1), pick([1.0, 0.25, 8.0, 2.0 ** -7], T, 2)
+    sb1, sb2 = pick([1.0, 0.25, 8.0], E * n, 3), pick([2.0, 0.5, 16.0, 2.0 ** 9], E * n, 4)
+    starts = _group_starts(sizes)
+    ref = torch.cat([
+        (a1[s:s + m].double() @ w1[e].double().t()) / sb1[e * n:(e + 1) * n].double() / sa1[s:s + m, None].double()
+        + (a2[s:s + m].double() @ w2[e].double().t()) / sb2[e * n:(e + 1) * n].double() / sa2[s:s + m, None].double()
+        for e, (s, m) in enumerate(zip(starts, sizes))
+    ]).float().bfloat16()
+    sz = torch.tensor(sizes).to(dev)
+    kmax = max(k1, k2)
+    # operands of both products in buffers of one row pitch, as the entry point requires
+    a_buf = torch.zeros((2, T, kmax), dtype=E4M3)
+    a_buf[0, :, :k1], a_buf[1, :, :k2] = a1.to(E4M3), a2.to(E4M3)
+    b_buf = torch.zeros((2, E * n, kmax), dtype=E4M3)
+    b_buf[0, :, :k1], b_buf[1, :, :k2] = w1.reshape(E * n, k1).to(E4M3), w2.reshape(E * n, k2).to(E4M3)
+    a_buf, b_buf = a_buf.to(dev), b_buf.to(dev)
+    if not ops.grouped_gemm_dual_supported(T, n, k1, k2):
+        with pytest.raises(Exception):
+            ops.grouped_gemm_fp8_dual(a_buf[0, :, :k1], sa1.to(dev), b_buf[0, :, :k1], sb1.to(dev), a_buf[1, :, :k2], sa2.to(dev),
+                                      b_buf[1, :, :k2], sb2.to(dev), sz, n=n, k1=k1, k2=k2, b_group_stride=n * kmax, sb_group_stride=n)
+        return
+    out = ops.grouped_gemm_fp8_dual(a_buf[0, :, :k1], sa1.to(dev), b_buf[0, :, :k1], sb1.to(dev), a_buf[1, :, :k2], sa2.to(dev),
+                                    b_buf[1, :, :k2], sb2.to(dev), sz, n=n, k1=k1, k2=k2, b_group_stride=n * kmax, sb_group_stride=n)
+    assert torch.equal(out.cpu(), ref)
+
+
+@pytest.mark.parametrize("sizes", [[300, 17, 0, 411, 64], [700, 1, 0, 323, 2048, 9]], ids=lambda s: "-".join(map(str, s[:6])))
+def test_grouped_dual_gemm_against_separate_products(dev, sizes):
+    """Random operands through the product's casts (power-of-two scales): the single launch agrees with the sum of the
+    two separate grouped GEMMs taken in float32 (same K order per product, one rounding instead of three) to within
+    a bf16 rounding of each term, and with the float64 product of the dequantised operands at the single-GEMM bar."""
+    E, T, n, k = len(sizes), sum(sizes), 512, 768
+    sz = torch.tensor(sizes).to(dev)
+    g1, g2 = seeded((T, k), 51, std=1e-3).to(dev), seeded((T, k), 52, std=3e-3).to(dev)
+    w1, w2 = seeded((E * k, n), 53, std=0.02).to(dev), seeded((E * k, n), 54, std=0.3).to(dev)
+    equal = torch.full((E,), k, dtype=torch.int64, device=dev)
+    g1q, s1 = ops.cast_rowwise(g1, E4M3, pow2=True)
+    g2q, s2 = ops.cast_rowwise(g2, E4M3, pow2=True)
+    w1t, c1 = ops.grouped_cast_colwise_t(w1, equal, E4M3, pow2=True)  # [n, E * k]: group e's K columns, one scale per (e, column)
+    w2t, c2 = ops.grouped_cast_colwise_t(w2, equal, E4M3, pow2=True)
+    kw = dict(n=n, b_group_stride=k, sb_group_stride=n)
+    got = ops.grouped_gemm_fp8_dual(g1q, s1, w1t, c1, g2q, s2, w2t, c2, sz, k1=k, k2=k, **kw)
+    p1 = ops.grouped_gemm_fp8(g1q, s1, w1t, c1, sz, k=k, out_dtype=torch.float32, **kw)
+    p2 = ops.grouped_gemm_fp8(g2q, s2, w2t, c2, sz, k=k, out_dtype=torch.float32, **kw)
+    want = (p1 + p2)
+    err = (got.float() - want).abs().max() / want.abs().max()
+    assert float(err) <= 2.0 ** -8, float(err)  # one bf16 rounding of the sum
+    # float64 on the host from the dequantised operands, group by group
+    starts = _group_starts(sizes)
+    for e, (s, m) in enumerate(zip(starts, sizes)):
+        if m == 0:
+            continue
+        ref = 0
+        for q, sr, wt, sc in ((g1q, s1, w1t, c1), (g2q, s2, w2t, c2)):
+            a = q[s:s + m].float().double().cpu() / sr[s:s + m, None].double().cpu()
+            b = wt[:, e * k:(e + 1) * k].float().double().cpu() / sc[e][:, None].double().cpu()
+            ref = ref + a @ b.t()
+        assert_gemm_close(got[s:s + m], ref, f"group {e}")
