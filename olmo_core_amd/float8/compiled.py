@@ -14,23 +14,30 @@ from typing import List, Optional, Tuple
 import torch
 
 from . import ops
-from .linear import _COMPILED_CONFIGS, _backward_impl, _forward_impl, _is_axiswise, _saves_quantised
+from .linear import (_COMPILED_CONFIGS, _backward_impl, _forward_impl, _is_axiswise, _kept_weight_state,
+                     _saves_quantised)
 
 _CONFIGS = _COMPILED_CONFIGS  # configs travel through the operators as indices into this list
 
 
 @torch.library.custom_op("olmo_core_amd::float8_linear_fwd", mutates_args=())
 def _linear_fwd(
-    x2: torch.Tensor, weight: torch.Tensor, weight_scale: Optional[torch.Tensor], cfg: int, need_gx: bool, need_gw: bool
+    x2: torch.Tensor, weight: torch.Tensor, weight_scale: Optional[torch.Tensor], cfg: int, need_gx: bool, need_gw: bool,
+    module_id: int,
 ) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]:
-    y, x_saved, w_saved = _forward_impl(x2, weight, _CONFIGS[cfg], weight_scale, need_gx, need_gw)
+    # (module_id: the calling module, -1 for none; what it keeps for its weight - a scale refreshed after the optimizer
+    # step, float8 copies - is used if still valid: same bytes and scales as quantising here)
+    kept_scale, kept_ops = _kept_weight_state(module_id, weight)
+    if weight_scale is None:
+        weight_scale = kept_scale
+    y, x_saved, w_saved = _forward_impl(x2, weight, _CONFIGS[cfg], weight_scale, need_gx, need_gw, kept_ops)
     xa, xb = x_saved if x_saved is not None else (x2.new_empty(0), x2.new_empty(0))
     wa, wb = w_saved if w_saved is not None else (x2.new_empty(0), x2.new_empty(0))
     return y, xa, xb, wa, wb
 
 
 @_linear_fwd.register_fake
-def _(x2, weight, weight_scale, cfg, need_gx, need_gw):
+def _(x2, weight, weight_scale, cfg, need_gx, need_gw, module_id):
     c = _CONFIGS[cfg]
     M, K = x2.shape
     N = weight.shape[0]
@@ -75,7 +82,7 @@ def _(go, xa, xb, wa, wb, cfg, n, x_is_q, w_is_q, need_gx, need_gw, x_dtype, w_d
 
 
 def _setup_context(ctx, inputs, output):
-    x2, weight, _, cfg, need_gx, need_gw = inputs
+    x2, weight, _, cfg, need_gx, need_gw, _ = inputs
     _, xa, xb, wa, wb = output
     x_is_q, w_is_q = _saves_quantised(_CONFIGS[cfg], need_gx, need_gw)
     ctx.meta = (cfg, weight.shape[0], x_is_q, w_is_q, need_gx, need_gw, x2.dtype, weight.dtype)
@@ -89,15 +96,16 @@ def _backward(ctx, gy, *unused):
     cfg, n, x_is_q, w_is_q, need_gx, need_gw, x_dtype, w_dtype = ctx.meta
     xa, xb, wa, wb = ctx.saved_tensors
     gx, gw = _linear_bwd(gy.contiguous(), xa, xb, wa, wb, cfg, n, x_is_q, w_is_q, need_gx, need_gw, x_dtype, w_dtype)
-    return (gx if need_gx else None), (gw if need_gw else None), None, None, None, None
+    return (gx if need_gx else None), (gw if need_gw else None), None, None, None, None, None
 
 
 _linear_fwd.register_autograd(_backward, setup_context=_setup_context)
 
 
-def linear(x2: torch.Tensor, weight: torch.Tensor, cfg_id: int, weight_scale: Optional[torch.Tensor]):
-    """``x2 [M, K] @ weight[N, K].T`` as a traceable operator call; ``cfg_id`` indexes the registered configs."""
-    out = _linear_fwd(x2, weight, weight_scale, cfg_id, x2.requires_grad, weight.requires_grad)
+def linear(x2: torch.Tensor, weight: torch.Tensor, cfg_id: int, weight_scale: Optional[torch.Tensor], module_id: int = -1):
+    """``x2 [M, K] @ weight[N, K].T`` as a traceable operator call; ``cfg_id`` indexes the registered configs,
+    ``module_id`` the registered modules (-1: none)."""
+    out = _linear_fwd(x2, weight, weight_scale, cfg_id, x2.requires_grad, weight.requires_grad, module_id)
     return out[0]
 
 
@@ -117,13 +125,16 @@ def _ff():
 
 @torch.library.custom_op("olmo_core_amd::float8_swiglu_mlp_fwd", mutates_args=())
 def _mlp_fwd(x: torch.Tensor, w1: torch.Tensor, w2: torch.Tensor, w3: torch.Tensor, cfg: int, need_x: bool, need_w1: bool,
-             need_w2: bool, need_w3: bool) -> List[torch.Tensor]:
-    y, saved = _ff()._mlp_forward(x, w1, w2, w3, _CONFIGS[cfg], (need_x, need_w1, need_w2, need_w3))
+             need_w2: bool, need_w3: bool, id1: int, id2: int, id3: int) -> List[torch.Tensor]:
+    # (id1..3: the three projection modules, for their precomputed scales and kept float8 weights)
+    state = [_kept_weight_state(i, w) for i, w in ((id1, w1), (id2, w2), (id3, w3))]
+    y, saved = _ff()._mlp_forward(x, w1, w2, w3, _CONFIGS[cfg], (need_x, need_w1, need_w2, need_w3),
+                                  tuple(s[0] for s in state), tuple(s[1] for s in state))
     return [y, *saved]
 
 
 @_mlp_fwd.register_fake
-def _(x, w1, w2, w3, cfg, need_x, need_w1, need_w2, need_w3):
+def _(x, w1, w2, w3, cfg, need_x, need_w1, need_w2, need_w3, id1, id2, id3):
     c = _CONFIGS[cfg]
     ff = _ff()
     M, D = x.shape
@@ -168,7 +179,7 @@ def _(gy, saved, cfg, m, d, h, need_x, need_w1, need_w2, need_w3, x_dtype, w1_dt
 
 
 def _mlp_setup_context(ctx, inputs, output):
-    x, w1, w2, w3, cfg, need_x, need_w1, need_w2, need_w3 = inputs
+    x, w1, w2, w3, cfg, need_x, need_w1, need_w2, need_w3 = inputs[:9]
     ctx.meta = (cfg, x.shape[0], x.shape[1], w1.shape[0], need_x, need_w1, need_w2, need_w3, x.dtype, w1.dtype, w2.dtype,
                 w3.dtype)
     ctx.save_for_backward(*output[1:])
@@ -178,15 +189,18 @@ def _mlp_backward_fn(ctx, grads):
     need = ctx.meta[4:8]
     gx, gw1, gw2, gw3 = _mlp_bwd(grads[0].contiguous(), list(ctx.saved_tensors), *ctx.meta)
     pick = lambda g, wanted: g if wanted else None  # noqa: E731
-    return pick(gx, need[0]), pick(gw1, need[1]), pick(gw2, need[2]), pick(gw3, need[3]), None, None, None, None, None
+    return (pick(gx, need[0]), pick(gw1, need[1]), pick(gw2, need[2]), pick(gw3, need[3])) + (None,) * 8
 
 
 _mlp_fwd.register_autograd(_mlp_backward_fn, setup_context=_mlp_setup_context)
 
 
-def swiglu_mlp(x2: torch.Tensor, w1: torch.Tensor, w2: torch.Tensor, w3: torch.Tensor, cfg_id: int) -> torch.Tensor:
-    """The fused feed-forward block on ``x2 [M, D]`` (bfloat16) as a traceable operator call."""
-    return _mlp_fwd(x2, w1, w2, w3, cfg_id, x2.requires_grad, w1.requires_grad, w2.requires_grad, w3.requires_grad)[0]
+def swiglu_mlp(x2: torch.Tensor, w1: torch.Tensor, w2: torch.Tensor, w3: torch.Tensor, cfg_id: int,
+               module_ids=(-1, -1, -1)) -> torch.Tensor:
+    """The fused feed-forward block on ``x2 [M, D]`` as a traceable operator call; ``module_ids``: the registered ids of
+    the w1, w2, w3 modules."""
+    return _mlp_fwd(x2, w1, w2, w3, cfg_id, x2.requires_grad, w1.requires_grad, w2.requires_grad, w3.requires_grad,
+                    module_ids[0], module_ids[1], module_ids[2])[0]
 
 
 __all__ = ["linear", "swiglu_mlp", "ops"]

@@ -329,6 +329,28 @@ def float8_projections(x: torch.Tensor, *modules: nn.Module) -> Tuple[torch.Tens
 # are registered when a module is built (tracing must not mutate the list).
 _COMPILED_CONFIGS: list = []
 
+# Likewise the modules (as weak references): a compiled call names its module by index, and the operator, which runs
+# eagerly, asks that module for its precomputed weight scale and kept float8 weight copies - lookups by address and
+# version counter that a traced graph cannot contain.
+_COMPILED_MODULES: list = []
+
+
+def _register_module(m) -> int:
+    import weakref
+
+    _COMPILED_MODULES.append(weakref.ref(m))
+    return len(_COMPILED_MODULES) - 1
+
+
+def _kept_weight_state(module_id: int, weight: torch.Tensor):
+    """``(precomputed scale, kept operands)`` of the registered module if ``weight`` is that module's weight."""
+    if module_id < 0 or module_id >= len(_COMPILED_MODULES):
+        return None, None
+    m = _COMPILED_MODULES[module_id]()
+    if m is None or m.weight.data_ptr() != weight.data_ptr() or m.weight.shape != weight.shape:
+        return None, None
+    return m.precomputed_weight_scale(), m.weight_operands()
+
 
 def _register_config(c: Float8LinearConfig) -> int:
     idx = getattr(c, "_compiled_id", None)
@@ -346,7 +368,7 @@ def _eager_matmul(x2, weight, config, weight_scale, weight_ops=None):
 
 def float8_linear_function(
     x: torch.Tensor, weight: torch.Tensor, config: Float8LinearConfig, weight_scale: Optional[torch.Tensor] = None,
-    weight_ops: Optional[Tuple[torch.Tensor, torch.Tensor, torch.Tensor]] = None,
+    weight_ops: Optional[Tuple[torch.Tensor, torch.Tensor, torch.Tensor]] = None, module_id: int = -1,
 ) -> torch.Tensor:
     """``x [*, K] @ weight[N, K].T`` through the float8 path, differentiable in x and weight.
 
@@ -367,7 +389,7 @@ def float8_linear_function(
     if compiling and cfg_id >= 0:
         from . import compiled
 
-        y = compiled.linear(x2, weight, cfg_id, weight_scale)
+        y = compiled.linear(x2, weight, cfg_id, weight_scale, module_id)
     elif not compiling and not (torch.is_grad_enabled() and (x2.requires_grad or weight.requires_grad)):
         # nothing to differentiate (evaluation, generation): no autograd node, nothing kept for a backward
         y = _forward_impl(x2, weight, config, weight_scale, False, False, weight_ops)[0]
@@ -390,6 +412,7 @@ class Float8Linear(nn.Linear):
     def _bind_config(self) -> None:
         c = self.config
         _register_config(c)
+        self._module_id = _register_module(self)
         self.scaling_type_input = c.cast_config_input.scaling_type
         self.scaling_type_weight = c.cast_config_weight.scaling_type
         self.scaling_type_grad_output = c.cast_config_grad_output.scaling_type
@@ -401,7 +424,7 @@ class Float8Linear(nn.Linear):
         compiling = torch.compiler.is_compiling()
         scale = None if compiling else self.precomputed_weight_scale()
         w_ops = None if compiling else self.weight_operands()
-        out = float8_linear_function(input, self.weight, self.config, scale, w_ops)
+        out = float8_linear_function(input, self.weight, self.config, scale, w_ops, self._module_id)
         if self.bias is not None:
             out = out + self.bias.to(out.dtype)
         return out

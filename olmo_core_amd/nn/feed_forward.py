@@ -254,7 +254,8 @@ class FeedForward(nn.Module):
                 from ..float8 import compiled
 
                 x2 = xa.reshape(-1, xa.shape[-1])
-                y = compiled.swiglu_mlp(x2, self.w1.weight, self.w2.weight, self.w3.weight, cfg_id)
+                y = compiled.swiglu_mlp(x2, self.w1.weight, self.w2.weight, self.w3.weight, cfg_id,
+                                        (self.w1._module_id, self.w2._module_id, self.w3._module_id))
                 return y.reshape(*x.shape[:-1], self.w2.weight.shape[0])
         elif xa.is_cuda and act_dtype == torch.bfloat16 and _fusable_modules(self):
             x2 = xa.reshape(-1, xa.shape[-1])

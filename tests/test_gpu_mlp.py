@@ -251,3 +251,55 @@ def test_fused_block_under_autocast(dev, param_dtype):
     assert results[0][1][2].dtype == param_dtype
     for name, a, b in zip(("y", "gx", "gw1", "gw2", "gw3"), results[0][1], results[1][1]):
         assert a.dtype == b.dtype and torch.equal(a, b), f"{name}: fused and module-by-module results differ under autocast"
+
+
+def test_compiled_modules_use_their_kept_weights(dev, monkeypatch):
+    """AOFloat8LinearConfig.recommended() (what every production script sets, src/olmo_core/float8/ao.py:173-180) under
+    torch.compile: the registered operators ask their modules for the float8 weight copies kept since the last weight
+    update, so the micro-batches of a step quantise each weight once - in a compiled block as in an eager one - and the
+    results are the bits of the eager modules."""
+    import torch.nn as nn
+
+    from olmo_core_amd.float8 import AOFloat8LinearConfig
+
+    D, H, M = 512, 1792, 4096
+    torch.manual_seed(3)
+    model = nn.ModuleDict({"ff": FeedForward(d_model=D, hidden_size=H, bias=False, dtype=torch.bfloat16),
+                           "proj": nn.Linear(D, 256, bias=True, dtype=torch.bfloat16)}).to(dev)
+    Float8Config(ao=AOFloat8LinearConfig.recommended()).apply_float8_linear(model)
+    weight_shapes = {(H, D), (D, H), (256, D)}
+    casts = []
+    orig = ops.cast_tensorwise
+
+    def counted(t, *a, **k):
+        if tuple(t.shape) in weight_shapes:
+            casts.append(tuple(t.shape))
+        return orig(t, *a, **k)
+
+    monkeypatch.setattr(ops, "cast_tensorwise", counted)
+
+    def fwd(m, x):
+        return m["proj"](m["ff"](x))
+
+    compiled = torch.compile(lambda x: fwd(model, x), fullgraph=True)
+    xs = [seeded((M, D), 20 + i).to(dev) for i in range(3)]
+    go = seeded((M, 256), 30, std=1e-3).to(dev)
+    outs = []
+    for x in xs:
+        xd = x.clone().requires_grad_(True)
+        y = compiled(xd)
+        y.backward(go)
+        outs.append((y, xd.grad))
+    assert len(casts) == 4, casts  # w1, w2, w3 and the projection, once each for the three micro-batches
+    model.zero_grad()
+    for x, (y1, g1) in zip(xs, outs):
+        xd = x.clone().requires_grad_(True)
+        y0 = fwd(model, xd)
+        y0.backward(go)
+        assert torch.equal(y0, y1) and torch.equal(xd.grad, g1)
+    assert len(casts) == 4
+    with torch.no_grad():  # a weight update is seen: the copies are made again
+        for p in model.parameters():
+            p.mul_(1.5)
+    y = compiled(xs[0])
+    assert len(casts) == 8 and torch.equal(y, fwd(model, xs[0]))
