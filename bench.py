@@ -457,6 +457,82 @@ def feed_probe():
                               "TFLOP/s": round(flop / us / 1e6, 1)}), flush=True)
 
 
+def store_probe():
+    """What a compute unit's store path takes (mi8_probe_store_rate): cycles per 16-byte-per-lane store instruction and wave,
+    and bytes per clock and compute unit, by lane pattern, waves per compute unit and number of compute units storing."""
+    from olmo_core_amd import _C
+
+    dev = torch.device("cuda:0")
+    pitch = HIDDEN * 2
+    window = torch.empty(16384 * pitch + 4096, dtype=torch.uint8, device=dev)
+    cycles = torch.zeros(256 * 4, dtype=torch.int32, device=dev)
+    st = torch.cuda.current_stream().cuda_stream
+    iters = 64
+    for workgroups in (256, 8):
+        for rows, waves in ((8, 4), (4, 4), (16, 4), (2, 4), (8, 2), (8, 1), (4, 1)):
+            for _ in range(3):
+                _C.check_diag(_C.diag().mi8_probe_store_rate(rows, waves, workgroups, iters, window.data_ptr(), pitch, cycles.data_ptr(), st))
+            torch.cuda.synchronize()
+            c = cycles.view(256, 4)[:workgroups, :waves].float()
+            per = c.mean().item() / (iters * 8)
+            print(json.dumps({"probe": f"global_store_dwordx4 stream, {rows} rows x {1024 // rows} B per instruction",
+                              "compute_units_storing": workgroups, "waves_per_compute_unit": waves,
+                              "cycles_per_store_and_wave": round(per, 1), "max": round(c.max().item() / (iters * 8), 1),
+                              "bytes_per_clock_and_compute_unit": round(waves * 1024 / per, 1)}), flush=True)
+
+
+def tile_timeline(shapes):
+    """Where the cycles of a GEMM tile go (mi8_diag_gemm_tile_timeline: the library's persistent kernel built with time
+    stamps): per shape and operand content, the mean shader-clock cycles of the K loop, of a K step, of the epilogue and
+    of its passes over all tiles of all workgroups, the clock the chip held, and the duration of the stamped launch next
+    to the product's own launch of the same GEMM."""
+    from olmo_core_amd import _C
+    from olmo_core_amd.float8 import ops
+
+    E4M3 = torch.float8_e4m3fn
+    dev = torch.device("cuda:0")
+    one = torch.ones(1, device=dev)
+    stamps = torch.zeros(256 * 256, dtype=torch.int32, device=dev)
+    st = torch.cuda.current_stream().cuda_stream
+    for (m, n, k) in shapes:
+        for kind in ("N(0,1)", "zeros"):
+            if kind == "zeros":
+                a = torch.zeros(m, k, device=dev).to(E4M3); b = torch.zeros(n, k, device=dev).to(E4M3)
+            else:
+                a = torch.randn(m, k, device=dev).to(E4M3); b = torch.randn(n, k, device=dev).to(E4M3)
+            out = torch.empty(m, n, dtype=torch.bfloat16, device=dev)
+            us_product = _time_us(lambda: ops.gemm_fp8(a, one, b, one, out=out), iters=5, warmup=4)
+            ref = out.clone()
+
+            def run():
+                _C.check_diag(_C.diag().mi8_diag_gemm_tile_timeline(a.data_ptr(), one.data_ptr(), b.data_ptr(), one.data_ptr(), out.data_ptr(),
+                                                              m, n, k, 0, 0, stamps.data_ptr(), st))
+            us_stamped = _time_us(run, iters=5, warmup=2)
+            assert torch.equal(out, ref), "the stamped kernel must produce the product kernel's bits"
+            t = stamps.cpu().view(256, 256).to(torch.int64) & 0xFFFFFFFF
+            ev = t[:, :13 * 16].view(256, 16, 13)
+            used = ev[:, :, 0] != 0
+            d = lambda i, j: ((ev[:, :, j] - ev[:, :, i]) & 0xFFFFFFFF)[used].double()
+            ticks = ((t[:, 255] - t[:, 254]) & 0xFFFFFFFF)[used.any(1)].double()           # 100 MHz
+            first = ev[:, 0, 0]
+            last = torch.stack([ev[w, int(used[w].sum()) - 1, 12] if used[w].any() else first[w] for w in range(256)])
+            span = ((last - first) & 0xFFFFFFFF)[used.any(1)].double()
+            nk = k // 128
+            passes = [round(d(3 + i, 4 + i).mean().item()) for i in range(7)]
+            print(json.dumps({"gemm": f"{m}x{n}x{k}", "operands": kind, "us_product_kernel": round(us_product, 1),
+                              "us_stamped_kernel_incl_two_synchronisations": round(us_stamped, 1),
+                              "tiles_per_workgroup": [int(used.sum(1).min()), int(used.sum(1).max())],
+                              "clock_MHz": round((span / (ticks / 100.0)).mean().item()),
+                              "cycles": {"k_loop": round(d(0, 2).mean().item()), "per_k_step": round(d(0, 2).mean().item() / nk, 1),
+                                         "first_three_k_steps": round(d(0, 1).mean().item()) if nk > 3 else None,
+                                         "epilogue": round(d(2, 12).mean().item()), "epilogue_min_max": [int(d(2, 12).min().item()), int(d(2, 12).max().item())],
+                                         "start_to_first_pass_staged": round(d(2, 3).mean().item()), "pass_to_pass": passes,
+                                         "last_pass_staged_to_last_store_issued": round(d(10, 11).mean().item()),
+                                         "refill_of_fragments": round(d(11, 12).mean().item())},
+                              "epilogue_share_of_tile": round(d(2, 12).mean().item() / (d(0, 12).mean().item()), 4),
+                              "mfma_floor_cycles_per_k_step": 2048}), flush=True)
+
+
 def power_probe():
     """What the power limit leaves of the matrix peak: back-to-back MFMAs with nothing else running, and the
     benchmark's longest-K GEMM, each on all-zero and on random operands (under `rocprofv3 --pmc GRBM_GUI_ACTIVE` the
@@ -694,6 +770,8 @@ def main():
     ap.add_argument("--cast-table", action="store_true", help="time every HBM-bound kernel of the path at the benchmark's shapes")
     ap.add_argument("--power-probe", action="store_true", help="bare MFMA loops and the GEMM on zero / random operands")
     ap.add_argument("--feed-probe", action="store_true", help="an MFMA stream with the loads and LDS reads of a GEMM K step beside it")
+    ap.add_argument("--store-probe", action="store_true", help="streams of 16-byte stores in the layout of a GEMM output tile: cycles per store, bytes per clock")
+    ap.add_argument("--tile-timeline", type=str, default=None, metavar="M,N,K;...", help="shader-clock cycles of the K loop, the epilogue and its passes per tile of the persistent GEMM")
     ap.add_argument("--profile-summary", type=str, default=None, metavar="DIR_OR_CSV",
                     help="print the per-kernel table of a rocprofv3 --stats --output-format csv run (no GPU needed)")
     ap.add_argument("--counter-summary", type=str, default=None, metavar="DIR_OR_CSV",
@@ -729,6 +807,12 @@ def main():
         return
     if ns.cast_table:
         cast_table()
+        return
+    if ns.store_probe:
+        store_probe()
+        return
+    if ns.tile_timeline:
+        tile_timeline([tuple(int(v) for v in sh.split(",")) for sh in ns.tile_timeline.split(";")])
         return
     if ns.feed_probe:
         feed_probe()

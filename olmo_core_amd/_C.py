@@ -186,6 +186,8 @@ _DIAG_SIGNATURES = {
     "mi8_diag_last_error": (c_char_p, []),
     "mi8_probe_mfma_loop": (c_int, [c_int, c_int, c_int, c_int, c_void_p, c_void_p]),
     "mi8_probe_mfma_feed": (c_int, [c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p]),
+    "mi8_probe_store_rate": (c_int, [c_int, c_int, c_int, c_int, c_void_p, c_int64, c_void_p, c_void_p]),
+    "mi8_diag_gemm_tile_timeline": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int, c_int, c_void_p, c_void_p]),
 }
 DIAG_EXPORTED_SYMBOLS = tuple(_DIAG_SIGNATURES)
 

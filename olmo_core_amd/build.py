@@ -25,6 +25,8 @@ OBJ_DIR = PKG_DIR / "lib" / "obj"
 SOURCES = ["mi8_api.hip", "mi8_cast.hip", "mi8_gemm.hip", "mi8_gemm_m16.hip", "mi8_gemm_skinny.hip", "mi8_pointwise.hip", "mi8_swiglu_amax.hip", "mi8_grouped.hip", "mi8_permute.hip"]
 # the diagnostics library: the probe kernels plus the error-text / launch helpers they share with the main library
 DIAG_SOURCES = ["mi8_api.hip", "mi8_probe.hip"]
+# ... and the persistent GEMM once more, compiled with time stamps at fixed points of every tile (object name, source, flag)
+DIAG_EXTRA = [("mi8_gemm_m16_timeline", "mi8_gemm_m16.hip", "-DMI8_TILE_TIMELINE")]
 
 HIPCC_FLAGS = [
     "--offload-arch=gfx950",
@@ -66,26 +68,30 @@ def build(force: bool = True, verbose: bool = False) -> Path:
     OBJ_DIR.mkdir(parents=True, exist_ok=True)
     cc = hipcc()
 
-    def compile_one(src: Path) -> Path:
-        obj = OBJ_DIR / (src.stem + ".o")
-        cmd = [cc, *HIPCC_FLAGS, "-c", str(src), "-o", str(obj)]
+    def compile_one(job) -> Path:
+        stem, src, extra = job
+        obj = OBJ_DIR / (stem + ".o")
+        cmd = [cc, *HIPCC_FLAGS, *extra, "-c", str(src), "-o", str(obj)]
         if verbose:
             print(" ".join(cmd), flush=True)
         res = subprocess.run(cmd, capture_output=True, text=True)
         if res.returncode != 0:
-            raise RuntimeError(f"hipcc failed on {src.name}:\n{res.stdout}\n{res.stderr}")
+            raise RuntimeError(f"hipcc failed on {Path(src).name}:\n{res.stdout}\n{res.stderr}")
         noise = "unknown target feature"  # host pass does not know the device-only feature flag
         warn = "\n".join(line for line in res.stderr.splitlines() if line.strip() and noise not in line and "-packed-fp32-ops" not in line)
         if warn and verbose:
             print(warn, file=sys.stderr)
         return obj
 
-    jobs = min(len(sources()), int(os.environ.get("MAX_JOBS", "8")))
+    work = [(src.stem, src, []) for src in sources()] + [(stem, CSRC / name, [flag]) for stem, name, flag in DIAG_EXTRA]
+    jobs = min(len(work), int(os.environ.get("MAX_JOBS", "8")))
     with ThreadPoolExecutor(max_workers=max(jobs, 1)) as pool:
-        objs = {o.stem: o for o in pool.map(compile_one, sources())}
-    for target, names in ((LIB_PATH, SOURCES), (DIAG_LIB_PATH, DIAG_SOURCES)):
+        objs = {o.stem: o for o in pool.map(compile_one, work)}
+    diag_names = DIAG_SOURCES + [stem for stem, _, _ in DIAG_EXTRA]
+    # (-Bsymbolic: the diagnostics library binds its own copies of the helpers it shares with libmi8.so)
+    for target, names, link_flags in ((LIB_PATH, SOURCES, []), (DIAG_LIB_PATH, diag_names, ["-Wl,-Bsymbolic"])):
         tmp = target.with_suffix(".so.tmp")
-        cmd = [cc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", str(tmp), *(str(objs[Path(n).stem]) for n in names)]
+        cmd = [cc, "--offload-arch=gfx950", "-shared", "-fPIC", *link_flags, "-o", str(tmp), *(str(objs[Path(n).stem]) for n in names)]
         res = subprocess.run(cmd, capture_output=True, text=True)
         if res.returncode != 0:
             raise RuntimeError(f"link of {target.name} failed:\n{res.stdout}\n{res.stderr}")

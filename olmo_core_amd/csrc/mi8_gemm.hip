@@ -217,7 +217,8 @@ int gemm_fp8_entry(const void* a, int a_dtype, int64_t lda, const void* b, int b
     hipStream_t st = (hipStream_t)stream;
     // (the persistent kernel shifts its last tile row / column back over the previous one when M or N is not a
     // multiple of 256 and rewrites the overlap with identical values: not possible when accumulating)
-    const bool dma_ok = (K % 128 == 0) && M >= 256 && N >= 256 && N % 8 == 0 && ldc % 8 == 0 && aligned16(out) &&
+    // (its output stores address a tile's 256 rows with 32-bit byte offsets: ldc < 2^22)
+    const bool dma_ok = (K % 128 == 0) && M >= 256 && N >= 256 && N % 8 == 0 && ldc % 8 == 0 && ldc < (1 << 22) && aligned16(out) &&
                         out_dtype == MI8_BF16 && (!sb_is_vector || aligned16(sb)) &&
                         (sa_is_vector != 0) == (sb_is_vector != 0) && (!accumulate || (M % 256 == 0 && N % 256 == 0));
     // measured on MI355X on the benchmark configurations' shapes: the four-wave layout beats the eight-wave one

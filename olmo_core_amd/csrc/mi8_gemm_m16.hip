@@ -40,7 +40,23 @@ constexpr int STAGE = (BM + BN) * BK;        // 64 KB
 constexpr int OUT_STAGING = 4 * 4096;        // 4 KB of output staging per wave
 constexpr int SCALE_SLOT = 2 * 256 * 4;      // one tile's 256 row scales and 256 column scales
 constexpr int SCALE_SLOTS = 4;
-constexpr int LDS_BYTES = 2 * STAGE + OUT_STAGING + SCALE_SLOTS * SCALE_SLOT;
+// Tile timeline (only in the diagnostics library, which compiles this file with -DMI8_TILE_TIMELINE): wave 0 of every
+// workgroup records the shader clock at fixed points of each of its tiles - K loop start, after three K steps, epilogue
+// start, every epilogue pass, last store issued, tile end - in 1 KB of LDS of its own and copies them out when the
+// kernel ends.  A stamp costs one s_memtime and its wait (placed where nothing else the wave waits for is in flight).
+#ifdef MI8_TILE_TIMELINE
+constexpr int TIMELINE_BYTES = 1024;
+constexpr int TIMELINE_STAMPS = 13;          // per tile
+constexpr int TIMELINE_TILES = 16;           // tiles recorded per workgroup (later tiles overwrite the last record)
+__device__ uint32_t* g_timeline = nullptr;   // [workgroups][256]: TIMELINE_TILES x TIMELINE_STAMPS, [254], [255]: 100 MHz clock at start / end
+#define MI8_TL(k) tl_stamp(k)
+#define MI8_TL_NEXT_TILE() (tl_ev += tl_ev < TIMELINE_STAMPS * (TIMELINE_TILES - 1) ? TIMELINE_STAMPS : 0)
+#else
+constexpr int TIMELINE_BYTES = 0;
+#define MI8_TL(k) ((void)0)
+#define MI8_TL_NEXT_TILE() ((void)0)
+#endif
+constexpr int LDS_BYTES = 2 * STAGE + OUT_STAGING + SCALE_SLOTS * SCALE_SLOT + TIMELINE_BYTES;
 constexpr int kThreads = 256;
 constexpr int WT = 128;                      // wave tile edge
 constexpr int NT = WT / 16;                  // MFMA tiles per wave tile edge
@@ -65,6 +81,22 @@ __device__ __forceinline__ uint32_t dpp_pk_umax16_over8(uint32_t v)
     return v;
 }
 
+// Output stores.  A tile's 128 KB are written once and read by a later kernel; left in the L2 as ordinary dirty lines
+// they displace the operand panels the XCD's 32 tiles share, and their write-back competes with the next tile's
+// first operand loads.  Marked write-through and streaming (sc0 sc1 nt) they pass through: the K steps after an
+// epilogue run at the rate of the others (K = 1024: 2350 instead of 2650 cycles per step, the GEMM -9 %), at the price of
+// a few hundred cycles more in the epilogue itself; whole steps of the benchmark configurations gain 1-2 %.
+// All output stores are buffer stores through the compiler's builtin, which takes these bits.  (Not inline asm: the
+// hardware reads a store's data registers after the instruction has issued, and only for stores it knows of does the
+// compiler keep later writes to those registers at a distance - an asm store followed by address arithmetic that
+// reused its data registers wrote garbage.)
+constexpr int kOutStoreAux = 1 | 2 | 16;  // sc0, nt, sc1
+// descriptor of `bytes` bytes at p (raw buffer, 32-bit offsets; an offset at or past `bytes` drops the lane's store)
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t out_rows(void* p, int bytes)
+{
+    return __builtin_amdgcn_make_buffer_rsrc(p, 0, bytes, 0x00020000);
+}
+
 template <typename Problem, int CBSZ_A, int BLGP_B>
 __global__ __launch_bounds__(kThreads, 1) void gemm_fp8_m16_kernel(Problem pb)
 {
@@ -75,6 +107,28 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_fp8_m16_kernel(Problem pb)
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wm = wave >> 1, wn = wave & 1;
     const int r16 = lane & 15, kb = lane >> 4;  // fragment row inside a tile; 32-byte K block of the lane
+#ifdef MI8_TILE_TIMELINE
+    uint32_t* const tl_out = g_timeline;
+    int tl_ev = 0;
+    const uint32_t tl_lds = (uint32_t)(uintptr_t)(lptr_t)(lds + LDS_BYTES - TIMELINE_BYTES);
+    auto tl_put = [&](int slot, uint64_t t) __attribute__((always_inline)) {
+        const uint32_t at = tl_lds + (uint32_t)(slot * 4);
+        asm volatile("ds_write_b32 %0, %1" ::"v"(at), "v"((uint32_t)t) : "memory");
+    };
+    auto tl_stamp = [&](int k) __attribute__((always_inline)) {
+        if (tl_out != nullptr && wave == 0) {  // (uniform)
+            uint64_t t;
+            asm volatile("s_memtime %0\n\ts_waitcnt lgkmcnt(0)" : "=s"(t)::"memory");
+            tl_put(tl_ev + k, t);
+        }
+    };
+    if (tl_out != nullptr && wave == 0) {
+        for (int i = lane; i < 256; i += 64) tl_put(i, 0);
+        uint64_t t;
+        asm volatile("s_memrealtime %0\n\ts_waitcnt lgkmcnt(0)" : "=s"(t)::"memory");
+        tl_put(254, t);
+    }
+#endif
 
     // ---- fragment read addresses of the stage being read (half q of the lane's 32 K bytes); tile t adds 2048 t
     uint32_t ra[2], rb[2];
@@ -357,6 +411,7 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_fp8_m16_kernel(Problem pb)
             }
         };
         if constexpr (Problem::kMfmaScale) load_exponents(0);
+        MI8_TL(0);
         // One 128-byte K step.  `fresh`: the tile's first step; phase A touches the accumulators of A tiles 0-3,
         // phase B those of A tiles 4-7, so both start from 0 then.  The first step is written out separately
         // from the loop, not as a branch inside it.
@@ -433,6 +488,7 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_fp8_m16_kernel(Problem pb)
             for (; kt + 1 < td.nk; kt += 2) {
                 k_step(false, set1);
                 k_step(false, set0);
+                if (kt == 1) MI8_TL(1);
             }
             if (kt < td.nk) k_step(false, set1);
             }
@@ -450,6 +506,7 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_fp8_m16_kernel(Problem pb)
         // The wave's output goes through its private staging area 32 rows x 64 columns at a time (4 KB, pitch 128
         // bytes, 16-byte chunk index XORed with (row >> 1) & 7), i.e. two A tiles by four B tiles per pass.
         // (the copies below are opaque to the compiler's hazard handling: the last MFMA has retired after these)
+        MI8_TL(2);
         asm volatile("s_nop 15\n\ts_nop 15");
         uint8_t* stg = lds + 2 * STAGE + wave * 4096;
         const uint32_t stg_lds = (uint32_t)(uintptr_t)(lptr_t)stg;
@@ -460,8 +517,7 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_fp8_m16_kernel(Problem pb)
         const uint32_t c_lane_off = (uint32_t)((lane >> 3) * ldc_bytes + (lane & 7) * 16);
         __amdgpu_buffer_rsrc_t c_rows;
         if constexpr (Problem::kMaskRows)
-            c_rows = __builtin_amdgcn_make_buffer_rsrc(td.c + (int64_t)td.row_lo * pb.ldc, 0,
-                                                       (td.row_hi - td.row_lo) * ldc_bytes, 0x00020000);
+            c_rows = out_rows(td.c + (int64_t)td.row_lo * pb.ldc, (td.row_hi - td.row_lo) * ldc_bytes);
         // The passes are software pipelined: the staged rows of a pass are read back into registers, and go to
         // memory only after the arithmetic of the next pass, so that each pass exposes one LDS round trip instead
         // of two.
@@ -528,16 +584,14 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_fp8_m16_kernel(Problem pb)
                 const int voff = (rt + (lane >> 3) - td.row_lo) * ldc_bytes + (wn * WT + jq * 64 + (lane & 7) * 8) * 2;
 #pragma unroll
                 for (int it = 0; it < 4; ++it)
-                    __builtin_amdgcn_raw_buffer_store_b128(staged[it], c_rows, voff + it * 8 * ldc_bytes, 0, 0);
+                    __builtin_amdgcn_raw_buffer_store_b128(staged[it], c_rows, voff + it * 8 * ldc_bytes, 0, kOutStoreAux);
             } else {
-                // uniform 64-bit base + one 32-bit lane offset shared by all passes (no per-pass lane pointers)
+                // the tile's 256 rows as one buffer: a uniform offset per instruction + one lane offset shared by all passes
+                const __amdgpu_buffer_rsrc_t c_tile = out_rows(td.c, 256 * ldc_bytes);
 #pragma unroll
-                for (int it = 0; it < 4; ++it) {
-                    uint8_t* base = reinterpret_cast<uint8_t*>(td.c + (int64_t)(rt + it * 8) * pb.ldc + wn * WT + jq * 64);
-                    uint32_t o = c_lane_off;
-                    asm volatile("" : "+v"(o));
-                    *reinterpret_cast<v4i*>(base + o) = staged[it];
-                }
+                for (int it = 0; it < 4; ++it)
+                    __builtin_amdgcn_raw_buffer_store_b128(staged[it], c_tile, c_lane_off,
+                                                           (rt + it * 8) * ldc_bytes + (wn * WT + jq * 64) * 2, kOutStoreAux);
             }
         };
         if constexpr (Problem::kSwiglu) {
@@ -550,13 +604,11 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_fp8_m16_kernel(Problem pb)
             auto store_out = [&](int which, int ih) __attribute__((always_inline)) {
                 const int rt = wm * WT + ih * 32;
                 const int64_t shift = which == 0 ? 0 : (which == 1 ? pb.x3_offset : pb.h_offset);
+                const __amdgpu_buffer_rsrc_t c_tile = out_rows(td.c + shift, 256 * ldc_bytes);
 #pragma unroll
-                for (int it = 0; it < 4; ++it) {
-                    uint8_t* base = reinterpret_cast<uint8_t*>(td.c + shift + (int64_t)(rt + it * 8) * pb.ldc + wn * 64);
-                    uint32_t o = c_lane_off;
-                    asm volatile("" : "+v"(o));
-                    *reinterpret_cast<v4i*>(base + o) = staged[it];
-                }
+                for (int it = 0; it < 4; ++it)
+                    __builtin_amdgcn_raw_buffer_store_b128(staged[it], c_tile, c_lane_off, (rt + it * 8) * ldc_bytes + wn * 64 * 2,
+                                                           kOutStoreAux);
             };
             // stage one pass (32 rows x 64 columns held as o[t][jj]); the pass before it goes to memory first
             auto stage = [&](const uint2 (&o)[2][4], int prev_which, int prev_ih) __attribute__((always_inline)) {
@@ -716,6 +768,7 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_fp8_m16_kernel(Problem pb)
                         asm volatile("ds_write_b64 %0, %1" ::"v"(saddr), "v"(o[t][jj]) : "memory");
                     }
                 __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): the wave's own LDS writes have landed
+                MI8_TL(3 + 4 * jq + ih);
                 __builtin_amdgcn_wave_barrier();
 #pragma unroll
                 for (int it = 0; it < 4; ++it) {
@@ -729,6 +782,7 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_fp8_m16_kernel(Problem pb)
         if constexpr (Problem::kAccumulate) add_held();
         record_codes(7);
         store_staged(1, 3);
+        MI8_TL(11);
         };
         if constexpr (Problem::kTwoSegments) {
             passes(std::true_type{});
@@ -746,10 +800,22 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_fp8_m16_kernel(Problem pb)
         // reload from scratch waits on the in-order vector memory counter, i.e. on the stores above).
         __builtin_amdgcn_sched_barrier(0);  // (or the scheduler moves these reads up into the epilogue)
         read_step_head();
+        MI8_TL(12);
+        MI8_TL_NEXT_TILE();
     }
     // direct loads issued for steps past the end must have landed before the LDS allocation is released
     __builtin_amdgcn_s_waitcnt(0x0070);  // vmcnt(0) lgkmcnt(0)
     __syncthreads();
+#ifdef MI8_TILE_TIMELINE
+    if (tl_out != nullptr && wave == 0) {
+        uint64_t t;
+        asm volatile("s_memrealtime %0\n\ts_waitcnt lgkmcnt(0)" : "=s"(t)::"memory");
+        tl_put(255, t);
+        __builtin_amdgcn_s_waitcnt(0xc07f);
+        for (int i = lane; i < 256; i += 64)
+            tl_out[(int)blockIdx.x * 256 + i] = reinterpret_cast<const uint32_t*>(lds + LDS_BYTES - TIMELINE_BYTES)[i];
+    }
+#endif
     if constexpr (Problem::kSwiglu) {  // one partial maximum of |h| per wave
         uint32_t m = reinterpret_cast<const uint32_t*>(lds + 2 * STAGE + OUT_STAGING)[64 + tid];
         m = wave_umax(m);
@@ -773,6 +839,9 @@ template <typename Problem, int CBSZ_A, int BLGP_B>
 int launch(const Problem& pb, int max_tiles, bool persistent, hipStream_t st)
 {
     auto kern = gemm_fp8_m16_kernel<Problem, CBSZ_A, BLGP_B>;
+    // the output stores address the 256 rows of a tile with 32-bit byte offsets
+    MI8_REQUIRE(pb.ldc > 0 && pb.ldc < (1 << 22), MI8_ERR_UNSUPPORTED, "mi8 16x16x128 GEMM: output row pitch %lld outside (0, 2^22) elements",
+                (long long)pb.ldc);
     static std::atomic<uint64_t> configured{0};
     if (int rc = reserve_dynamic_lds(reinterpret_cast<const void*>(kern), LDS_BYTES, configured, "mi8 16x16x128 GEMM"))
         return rc;
@@ -869,3 +938,30 @@ int launch_m16_grouped_wgrad(const uint8_t* a_t, int a_dtype, const uint8_t* b_t
 
 }  // namespace gemm
 }  // namespace mi8
+
+#ifdef MI8_TILE_TIMELINE
+#include "../../include/mi8_diag.h"
+// (declared in mi8_diag.h) One plain GEMM launch, single scales, bf16 output, with the tile timeline recorded.
+extern "C" int mi8_diag_gemm_tile_timeline(const void* a, const float* sa, const void* b, const float* sb, void* out, int64_t M,
+                                           int64_t N, int64_t K, int a_dtype, int b_dtype, uint32_t* stamps, void* stream)
+{
+    using namespace mi8;
+    MI8_REQUIRE(a && b && sa && sb && out && stamps, MI8_ERR_ARG, "mi8_diag_gemm_tile_timeline: null pointer");
+    MI8_REQUIRE(M >= 256 && N >= 256 && K >= 128 && K % 128 == 0 && N % 8 == 0 && M <= (1 << 30) && N <= (1 << 30) && K <= (1 << 30),
+                MI8_ERR_UNSUPPORTED, "mi8_diag_gemm_tile_timeline: needs M, N >= 256, K a multiple of 128, N a multiple of 8");
+    MI8_REQUIRE((a_dtype == MI8_E4M3 || a_dtype == MI8_E5M2) && (b_dtype == MI8_E4M3 || b_dtype == MI8_E5M2), MI8_ERR_ARG,
+                "mi8_diag_gemm_tile_timeline: operand types must be MI8_E4M3 or MI8_E5M2");
+    hipStream_t st = (hipStream_t)stream;
+    gemm::GemmArgs g{(const uint8_t*)a, (const uint8_t*)b, out, 0, K, K, N, (int)M, (int)N, (int)K, sa, sb, 0, 0, 0, 0, 0};
+    // the pointer is a device global of this library: set for this launch only, between stream synchronisations
+    MI8_REQUIRE(hipStreamSynchronize(st) == hipSuccess &&
+                    hipMemcpyToSymbol(HIP_SYMBOL(gemm::g_timeline), &stamps, sizeof(stamps)) == hipSuccess,
+                MI8_ERR_LAUNCH, "mi8_diag_gemm_tile_timeline: could not set the timeline pointer");
+    const int rc = gemm::launch_m16(g, a_dtype, b_dtype, st);
+    uint32_t* none = nullptr;
+    MI8_REQUIRE(hipStreamSynchronize(st) == hipSuccess &&
+                    hipMemcpyToSymbol(HIP_SYMBOL(gemm::g_timeline), &none, sizeof(none)) == hipSuccess,
+                MI8_ERR_LAUNCH, "mi8_diag_gemm_tile_timeline: launch or reset failed");
+    return rc;
+}
+#endif

@@ -236,5 +236,47 @@ extern "C" int mi8_probe_mfma_loop(int mfma_shape, int random_operands, int iter
     return launch_status("mi8_probe_mfma_loop");
 }
 
+// ---- store path -----------------------------------------------------------------------------------
+// Every active wave streams 16-byte-per-lane stores into its 128-row x 256-byte quadrant of the workgroup's 256 x 512-byte
+// window (the layout of a GEMM output tile with a row pitch of `pitch` bytes): one instruction covers `rows` rows with
+// 64 / rows lanes each.  Lane 0 of every wave reports the shader-clock cycles of its loop.
+__global__ __launch_bounds__(256, 1) void store_rate_kernel(uint8_t* out, int64_t pitch, int rows, int waves, int iterations,
+                                                            uint32_t* cycles)
+{
+    typedef int v4i __attribute__((ext_vector_type(4)));
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    if (wave >= waves) return;
+    const int lanes_per_row = 64 / rows, row = lane / lanes_per_row, chunk = lane % lanes_per_row;
+    const int row_bytes = lanes_per_row * 16;                    // bytes of one row written by one instruction
+    const int col_blocks = row_bytes >= 256 ? 1 : 256 / row_bytes;
+    const int per_sweep = 128 / rows >= 8 ? 8 : 128 / rows;      // instructions per unrolled group
+    uint8_t* p0 = out + (int64_t)((int)blockIdx.x % 64) * 256 * pitch + ((int)blockIdx.x / 64) * 512 + (int64_t)(wave >> 1) * 128 * pitch +
+                  (wave & 1) * 256 + (int64_t)row * pitch + chunk * 16;
+    const int64_t step = (int64_t)rows * pitch;
+    const v4i v = {lane, tid, iterations, 7};
+    const uint64_t t0 = __builtin_readcyclecounter();
+    for (int it = 0; it < iterations; ++it) {
+        const int first = it * per_sweep * rows;
+        uint8_t* p = p0 + (int64_t)(first & 127) * pitch + ((first >> 7) & (col_blocks - 1)) * row_bytes;
+#pragma unroll
+        for (int u = 0; u < 8; ++u) *reinterpret_cast<v4i*>(p + (u % per_sweep) * step) = v;
+    }
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
+    const uint64_t t1 = __builtin_readcyclecounter();
+    if (lane == 0) cycles[blockIdx.x * 4 + wave] = (uint32_t)(t1 - t0);
+}
+
+extern "C" int mi8_probe_store_rate(int rows, int waves, int workgroups, int iterations, void* window, int64_t pitch,
+                                    uint32_t* cycles, void* stream)
+{
+    MI8_REQUIRE(window && cycles, MI8_ERR_ARG, "mi8_probe_store_rate: null pointer");
+    MI8_REQUIRE((rows == 2 || rows == 4 || rows == 8 || rows == 16) && waves >= 1 && waves <= 4 && workgroups >= 1 &&
+                    workgroups <= 256 && iterations > 0 && iterations <= (1 << 16) && pitch >= 2048 && pitch % 16 == 0,
+                MI8_ERR_ARG, "mi8_probe_store_rate: rows 2, 4, 8 or 16, 1..4 waves, 1..256 workgroups, pitch >= 2048 and a multiple of 16");
+    hipLaunchKernelGGL(store_rate_kernel, dim3(workgroups), dim3(256), 0, (hipStream_t)stream, (uint8_t*)window, pitch, rows, waves,
+                       iterations, cycles);
+    return launch_status("mi8_probe_store_rate");
+}
+
 extern "C" const char* mi8_last_error(void);
 extern "C" const char* mi8_diag_last_error(void) { return mi8_last_error(); }
