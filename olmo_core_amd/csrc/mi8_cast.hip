@@ -248,7 +248,10 @@ __device__ __forceinline__ void tile_cast_body(const void* x, int64_t row_end, i
                 src = gathered_row(gather, top_k, src_rows, r, r < row_end);
                 ok = ok && src >= 0;
             }
-            HpVec<HP>::load8(xb + (src * cols + c8) * HpVec<HP>::kBytes, ok, f[it][j]);
+            if (gather)  // (uniform) a token's row is read top_k times: it stays cached
+                HpVec<HP>::load8(xb + (src * cols + c8) * HpVec<HP>::kBytes, ok, f[it][j]);
+            else
+                HpVec<HP>::template load8<true>(xb + (src * cols + c8) * HpVec<HP>::kBytes, ok, f[it][j]);
             if (gather_w) {  // (uniform) weighted gather: the product, rounded to the element type
                 const float w = gathered_weight(gather, gather_w, gather_w_dtype, r, ok);
 #pragma unroll
@@ -277,12 +280,12 @@ __device__ __forceinline__ void tile_cast_body(const void* x, int64_t row_end, i
             lo[j] = quant4<FP8, SW>(v[0], v[1], v[2], v[3], sc[0], sc[1], sc[2], sc[3]);
             hi[j] = quant4<FP8, SW>(v[4], v[5], v[6], v[7], sc[4], sc[5], sc[6], sc[7]);
             if (!ok) lo[j] = hi[j] = 0;  // padding is zero bytes whatever the scale is (0 * NaN is NaN)
-            if (out && ok) *reinterpret_cast<uint2*>(out + r * ld_out + c8) = make_uint2(lo[j], hi[j]);
+            if (out && ok) store_stream8(out + r * ld_out + c8, lo[j], hi[j]);
             if (out_r && ok) {  // the same values quantised with the row's own scale
                 const float sr = srow[it][j];
                 const uint32_t rl = quant4<FP8, SW>(v[0], v[1], v[2], v[3], sr, sr, sr, sr);
                 const uint32_t rh = quant4<FP8, SW>(v[4], v[5], v[6], v[7], sr, sr, sr, sr);
-                *reinterpret_cast<uint2*>(out_r + r * ld_r + c8) = make_uint2(rl, rh);
+                store_stream8(out_r + r * ld_r + c8, rl, rh);
             }
         }
         if (out_t) {
@@ -307,7 +310,7 @@ __device__ __forceinline__ void tile_cast_body(const void* x, int64_t row_end, i
             const uint4 v = reinterpret_cast<const uint4*>(lds_t)[tile_lds_chunk(col, part)];
             const int64_t c = col0 + col;
             const int64_t d = dst0 + 16 * part;
-            if (c < cols && d < dst_end) *reinterpret_cast<uint4*>(out_t + c * ld_t + d) = v;
+            if (c < cols && d < dst_end) store_stream16(out_t + c * ld_t + d, v);
         }
     }
 }
@@ -457,7 +460,7 @@ __global__ __launch_bounds__(kThreads) void rowwise_cast_kernel(const void* __re
 #pragma unroll
     for (int i = 0; i < NV; ++i) {
         const int v = lane + TPR * i;
-        HpVec<HP>::load8(xr + (int64_t)v * 8 * HpVec<HP>::kBytes, row_ok && v < nvec, f[i]);
+        HpVec<HP>::template load8<true>(xr + (int64_t)v * 8 * HpVec<HP>::kBytes, row_ok && v < nvec, f[i]);
         m = umax32(m, absmax8_bits(f[i]));
     }
     if constexpr (TPR == 64)
@@ -473,7 +476,7 @@ __global__ __launch_bounds__(kThreads) void rowwise_cast_kernel(const void* __re
         if (row_ok && v < nvec) {
             const uint32_t lo = quant4<FP8, SW>(f[i][0], f[i][1], f[i][2], f[i][3], s, s, s, s);
             const uint32_t hi = quant4<FP8, SW>(f[i][4], f[i][5], f[i][6], f[i][7], s, s, s, s);
-            *reinterpret_cast<uint2*>(orow + (int64_t)v * 8) = make_uint2(lo, hi);
+            store_stream8(orow + (int64_t)v * 8, lo, hi);
         }
     }
 }
@@ -691,7 +694,7 @@ __global__ __launch_bounds__(kThreads) void swiglu_bwd_cast_kernel(SwigluBwdCast
             p[0][j] = p[1][j] = make_uint4(0, 0, 0, 0);
             if (col_ok && r < a.rows) {
                 const int64_t v = (r * a.cols + c8) >> 3;
-                swiglu_bwd8(a.x1[v], a.x3[v], a.gh[v], p[0][j], p[1][j]);
+                swiglu_bwd8(load_stream16(a.x1 + v), load_stream16(a.x3 + v), load_stream16(a.gh + v), p[0][j], p[1][j]);
             }
         }
 #pragma unroll
@@ -706,7 +709,7 @@ __global__ __launch_bounds__(kThreads) void swiglu_bwd_cast_kernel(SwigluBwdCast
                 lo[j] = quant4<FP8, SW>(v[0], v[1], v[2], v[3], sc[o], sc[o], sc[o], sc[o]);
                 hi[j] = quant4<FP8, SW>(v[4], v[5], v[6], v[7], sc[o], sc[o], sc[o], sc[o]);
                 if (!ok) lo[j] = hi[j] = 0;  // padding is zero bytes whatever the scale is (0 * NaN is NaN)
-                if (out[o] && ok) *reinterpret_cast<uint2*>(out[o] + r * a.ld_out + c8) = make_uint2(lo[j], hi[j]);
+                if (out[o] && ok) store_stream8(out[o] + r * a.ld_out + c8, lo[j], hi[j]);
             }
             if (want_t) {
                 uint32_t t[8];
@@ -733,7 +736,7 @@ __global__ __launch_bounds__(kThreads) void swiglu_bwd_cast_kernel(SwigluBwdCast
                 const uint4 v = reinterpret_cast<const uint4*>(lds_t[o])[tile_lds_chunk(col, part)];
                 const int64_t c = col0 + col;
                 const int64_t d = row0 + 16 * part;
-                if (c < a.cols && d < dst_end) *reinterpret_cast<uint4*>(out_t[o] + c * a.ld_t + d) = v;
+                if (c < a.cols && d < dst_end) store_stream16(out_t[o] + c * a.ld_t + d, v);
             }
     }
 }
@@ -787,11 +790,11 @@ __global__ __launch_bounds__(kThreads) void grouped_swiglu_kernel(GroupedSwigluA
             const int64_t v = (r * a.cols + c8) >> 3;
             uint4 out[2];
             if constexpr (BWD) {
-                swiglu_bwd8(a.x1[v], a.x2[v], a.gh[v], out[0], out[1]);
+                swiglu_bwd8(load_stream16(a.x1 + v), load_stream16(a.x2 + v), load_stream16(a.gh + v), out[0], out[1]);
                 a.o1[v] = out[0];
                 a.o2[v] = out[1];
             } else {
-                out[0] = swiglu_fwd8(a.x1[v], a.x2[v]);
+                out[0] = swiglu_fwd8(load_stream16(a.x1 + v), load_stream16(a.x2 + v));
                 a.o1[v] = out[0];
             }
 #pragma unroll
