@@ -184,7 +184,7 @@ int mi8_gemm_fp8_accumulate(const void* a, int a_dtype, int64_t lda, const void*
  * Every workgroup computes matching 128-column tiles of x1 and x3 and forms h in its epilogue, so x1 and x3 are written
  * once and never read back.  A fp8 [M, lda]; B1, B3 fp8 [H, ldb] of one type; single scales (float32 [1] each);
  * x1, x3, h bf16 [M, ldc]; slots_h must hold MI8_AMAX_SLOTS uint32.  Needs M >= 256, H >= 128, H % 8 == 0,
- * K % 128 == 0 (MI8_ERR_UNSUPPORTED otherwise: run the three calls it stands for).
+ * K % 128 == 0, ldc < 2^22 (MI8_ERR_UNSUPPORTED otherwise: run the three calls it stands for).
  * x_codes: NULL, or uint16[mi8_rowseg_code_count(M, H)] that receives the row-segment codes of the element-wise
  * larger of x1 and x3 (what mi8_rowseg_max_codes(x1, x3) computes; needs H % 64 == 0), for the backward pass's
  * mi8_swiglu_bwd_amax_from_codes. */
@@ -343,7 +343,7 @@ int mi8_swiglu_bwd_amax_from_codes(const void* x1, const void* x3, const void* g
 /* out = mi8_gemm_fp8(a, b) for single scales and a bf16 output, with the row-segment codes of out written by the
  * epilogue (the gradient reaching h = silu(x1) * x3, grad_h = grad_y W2 of src/olmo_core/nn/feed_forward.py:171, is
  * produced this way).  mi8_gemm_fp8_codes_supported: shapes it takes (those mi8_gemm_fp8 runs on the same kernel, so
- * out has the same bits; N % 64 == 0). */
+ * out has the same bits; N % 64 == 0; ldc < 2^22). */
 int mi8_gemm_fp8_codes_supported(int64_t M, int64_t N, int64_t K);
 int mi8_gemm_fp8_codes(const void* a, int a_dtype, int64_t lda, const void* b, int b_dtype, int64_t ldb, int64_t M, int64_t N,
                        int64_t K, const float* sa, const float* sb, void* out, int64_t ldc, uint16_t* codes, void* stream);

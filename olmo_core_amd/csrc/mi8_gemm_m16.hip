@@ -532,14 +532,14 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_fp8_m16_kernel(Problem pb)
                 const int voff = (rt + (lane >> 3) - td.row_lo) * ldc_bytes + (wn * WT + jq * 64 + (lane & 7) * 8) * 2;
 #pragma unroll
                 for (int it = 0; it < 4; ++it)  // (rows outside the group read as zeros and are not stored)
-                    held[it] = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(c_rows, voff + it * 8 * ldc_bytes, 0, 0));
+                    held[it] = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(c_rows, voff + it * 8 * ldc_bytes, 0, 2));  // (nt: read once)
             } else {
 #pragma unroll
                 for (int it = 0; it < 4; ++it) {
                     const uint8_t* base = reinterpret_cast<const uint8_t*>(td.c + (int64_t)(rt + it * 8) * pb.ldc + wn * WT + jq * 64);
                     uint32_t o = c_lane_off;
                     asm volatile("" : "+v"(o));
-                    held[it] = *reinterpret_cast<const v4i*>(base + o);
+                    held[it] = __builtin_nontemporal_load(reinterpret_cast<const v4i*>(base + o));  // (read once)
                 }
             }
         };
