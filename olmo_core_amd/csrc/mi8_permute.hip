@@ -174,31 +174,82 @@ __global__ __launch_bounds__(kThreads) void scatter_reduce_kernel(PermuteArgs a,
     T* out = reinterpret_cast<T*>(a.out) + t * a.hidden;
     if (a.vec) {
         const int64_t chunks = a.hidden / N;
-        for (int64_t c = lane; c < chunks; c += 64) {
-            float acc[N];
-            Chunk<T> first;
-            first.raw = make_uint4(0, 0, 0, 0);
-#pragma unroll
-            for (int e = 0; e < N; ++e) acc[e] = 0.0f;
-            for (int j = 0; j < k; ++j) {
-                const int64_t slot = t * k + j;
-                const int32_t r = a.inverse[slot];
-                if (r < 0) continue;
-                Chunk<T> v;
-                v.raw = reinterpret_cast<const uint4*>(x + (int64_t)r * a.hidden)[c];
-                if (SCALE) {
-                    const float w = load_weight(a.weights, a.w_dtype, slot);
-#pragma unroll
-                    for (int e = 0; e < N; ++e) v.e[e] = El<DT>::from_f32(El<DT>::to_f32(v.e[e]) * w);
-                }
-                if (k == 1) first = v;
-#pragma unroll
-                for (int e = 0; e < N; ++e) acc[e] += El<DT>::to_f32(v.e[e]);
+        // The token's rows and weights are fetched once, slot j by lane j, and handed round as wave-uniform values (top_k
+        // up to 64; beyond, every term reads its own).  A lane then has four chunks of two rows in flight at a time: a
+        // chain of one index load and one row load per term left the memory system idle most of the time.
+        const bool held = k <= 64;
+        int32_t my_r = -1;
+        float my_w = 1.0f;
+        if (held && lane < k) {
+            my_r = a.inverse[t * k + lane];
+            if (SCALE && my_r >= 0) my_w = load_weight(a.weights, a.w_dtype, t * k + lane);
+        }
+        auto term = [&](int j, int32_t& r, float& w) __attribute__((always_inline)) {
+            if (held) {
+                r = __builtin_amdgcn_readlane(my_r, j);
+                w = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, my_w), j));
+            } else {
+                r = a.inverse[t * k + j];
+                w = (SCALE && r >= 0) ? load_weight(a.weights, a.w_dtype, t * k + j) : 1.0f;
             }
-            Chunk<T> o;
+        };
+        constexpr int U = 4;
+        for (int64_t c0 = lane; c0 < chunks; c0 += 64 * U) {
+            float acc[U][N];
+            Chunk<T> first[U];
 #pragma unroll
-            for (int e = 0; e < N; ++e) o.e[e] = El<DT>::from_f32(acc[e]);
-            reinterpret_cast<uint4*>(out)[c] = (k == 1) ? first.raw : o.raw;  // top_k 1 is a pure move (keeps -0)
+            for (int u = 0; u < U; ++u) {
+                first[u].raw = make_uint4(0, 0, 0, 0);
+#pragma unroll
+                for (int e = 0; e < N; ++e) acc[u][e] = 0.0f;
+            }
+            auto fetch = [&](int32_t r, Chunk<T> (&v)[U]) __attribute__((always_inline)) {
+                const uint4* row = reinterpret_cast<const uint4*>(x + (int64_t)(r < 0 ? 0 : r) * a.hidden);
+#pragma unroll
+                for (int u = 0; u < U; ++u)
+                    v[u].raw = (r >= 0 && c0 + 64 * u < chunks) ? load_stream16(row + c0 + 64 * u) : make_uint4(0, 0, 0, 0);
+            };
+            auto add = [&](int32_t r, float w, Chunk<T> (&v)[U]) __attribute__((always_inline)) {
+                if (r < 0) return;  // (uniform) an unfilled slot adds nothing, not even +0 to a -0
+#pragma unroll
+                for (int u = 0; u < U; ++u) {
+                    if (SCALE) {
+#pragma unroll
+                        for (int e = 0; e < N; ++e) v[u].e[e] = El<DT>::from_f32(El<DT>::to_f32(v[u].e[e]) * w);
+                    }
+                    if (k == 1) first[u] = v[u];
+#pragma unroll
+                    for (int e = 0; e < N; ++e) acc[u][e] += El<DT>::to_f32(v[u].e[e]);
+                }
+            };
+            int j = 0;
+            for (; j + 1 < k; j += 2) {  // two terms' rows in flight; added in slot order
+                int32_t r0, r1;
+                float w0, w1;
+                term(j, r0, w0);
+                term(j + 1, r1, w1);
+                Chunk<T> v0[U], v1[U];
+                fetch(r0, v0);
+                fetch(r1, v1);
+                add(r0, w0, v0);
+                add(r1, w1, v1);
+            }
+            if (j < k) {
+                int32_t r0;
+                float w0;
+                term(j, r0, w0);
+                Chunk<T> v0[U];
+                fetch(r0, v0);
+                add(r0, w0, v0);
+            }
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                if (c0 + 64 * u >= chunks) continue;
+                Chunk<T> o;
+#pragma unroll
+                for (int e = 0; e < N; ++e) o.e[e] = El<DT>::from_f32(acc[u][e]);
+                reinterpret_cast<uint4*>(out)[c0 + 64 * u] = (k == 1) ? first[u].raw : o.raw;  // top_k 1 is a pure move (keeps -0)
+            }
         }
     } else {
         for (int64_t c = lane; c < a.hidden; c += 64) {
@@ -242,12 +293,21 @@ __global__ __launch_bounds__(kThreads) void scatter_wgrad_kernel(PermuteArgs a, 
     float acc = 0.0f;
     if (a.vec) {
         const int64_t chunks = a.hidden / N;
-        for (int64_t c = lane; c < chunks; c += 64) {
-            Chunk<T> xv, gv;
-            xv.raw = reinterpret_cast<const uint4*>(x)[c];
-            gv.raw = reinterpret_cast<const uint4*>(g)[c];
+        constexpr int U = 4;  // chunks in flight per lane; summed in the order of a chunk-by-chunk loop
+        for (int64_t c0 = lane; c0 < chunks; c0 += 64 * U) {
+            Chunk<T> xv[U], gv[U];
 #pragma unroll
-            for (int e = 0; e < N; ++e) acc += El<DT>::to_f32(xv.e[e]) * El<DT>::to_f32(gv.e[e]);
+            for (int u = 0; u < U; ++u) {
+                const bool ok = c0 + 64 * u < chunks;
+                xv[u].raw = ok ? load_stream16(reinterpret_cast<const uint4*>(x) + c0 + 64 * u) : make_uint4(0, 0, 0, 0);
+                gv[u].raw = ok ? reinterpret_cast<const uint4*>(g)[c0 + 64 * u] : make_uint4(0, 0, 0, 0);
+            }
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                if (c0 + 64 * u >= chunks) continue;
+#pragma unroll
+                for (int e = 0; e < N; ++e) acc += El<DT>::to_f32(xv[u].e[e]) * El<DT>::to_f32(gv[u].e[e]);
+            }
         }
     } else {
         for (int64_t c = lane; c < a.hidden; c += 64) acc += El<DT>::to_f32(x[c]) * El<DT>::to_f32(g[c]);
