@@ -57,6 +57,29 @@ def test_integer_operands_exact(dev, mnk):
             assert torch.equal(out.cpu(), ref), f"variant {ops.gemm_variants()[v]} {da} x {db}: max diff {(out.cpu() - ref).abs().max()}"
 
 
+@pytest.mark.parametrize("mnk", [(520, 776, 256), (2088, 1032, 384), (256, 264, 128)], ids=lambda s: "x".join(map(str, s)))
+@pytest.mark.parametrize("vec", [False, True], ids=["single-scales", "scale-vectors"])
+def test_persistent_kernel_pitched_output(dev, mnk, vec):
+    """The persistent kernel writes its tiles through buffer stores addressed from the tile's origin: an output with a
+    row pitch wider than N, M and N that are not multiples of 256 (the last tile row / column is shifted back over the
+    previous one).  Integer operands and power-of-two scales: exact; the columns past N keep what they held."""
+    M, N, K = mnk
+    a, b = _int_operand((M, K), 70 + M, E4M3), _int_operand((N, K), 71 + N, E5M2)
+    g = torch.Generator().manual_seed(72)
+    if vec:
+        sa, sb = 2.0 ** torch.randint(-3, 4, (M,), generator=g).float(), 2.0 ** torch.randint(-3, 4, (N,), generator=g).float()
+        want = a.float() @ b.float().t() / sa[:, None] / sb[None, :]
+    else:
+        sa, sb = torch.tensor([4.0]), torch.tensor([0.5])
+        want = a.float() @ b.float().t() / 2.0
+    kM16 = ops.gemm_variants().index("256x256_dma_w4x128_m16x128")
+    wide = torch.full((M, N + 24), 7.0, dtype=torch.bfloat16, device=dev)
+    res = ops.gemm_fp8(a.to(dev), sa.to(dev), b.to(dev), sb.to(dev), out=wide[:, :N], variant=kM16)
+    assert res.data_ptr() == wide.data_ptr()
+    assert torch.equal(wide[:, :N].float().cpu(), want.bfloat16().float())
+    assert bool((wide[:, N:] == 7.0).all())
+
+
 @pytest.mark.parametrize("M", [1, 5, 16, 31, 64])
 def test_few_rows_scales_and_outputs(dev, M):
     """The default route for M <= 64: every mix of single scales and scale vectors, both output types, padded row
